@@ -1,0 +1,73 @@
+"""ctypes loader for librfa_hip.so, the C-ABI kernel library (include/rfa_hip.h).
+
+There is no fallback: if the library has not been built, importing any
+kernel-backed function raises, and calling one with tensors that are not on a
+HIP device raises as well.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import re
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "librfa_hip.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "rfa_hip.h")
+
+RFA_OK = 0
+ERROR_NAMES = {
+    -1: "RFA_ERR_NULL_POINTER", -2: "RFA_ERR_BAD_SHAPE", -3: "RFA_ERR_UNSUPPORTED",
+    -4: "RFA_ERR_ALIGNMENT", -5: "RFA_ERR_WORKSPACE", -6: "RFA_ERR_HIP",
+}
+
+
+class RfaHipError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        self.code = code
+        super().__init__(f"{ERROR_NAMES.get(code, code)}: {message}")
+
+
+# name -> (restype, argtypes); kept in step with include/rfa_hip.h (tests check it)
+SIGNATURES = {
+    "rfa_version": (c_int, []),
+    "rfa_last_error": (c_char_p, []),
+    "rfa_shape_supported": (c_int, [c_int, c_int]),
+    "rfa_selftest_layout": (c_int, [c_void_p]),
+    "rfa_causal_num_segments": (c_int, [c_int64, c_int64]),
+    "rfa_causal_forward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
+    "rfa_causal_forward": (c_int, [c_void_p] * 4 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "rfa_causal_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
+    "rfa_causal_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once; raise ImportError with build instructions if absent."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m rfa_amd.build` "
+                "(hipcc, --offload-arch=gfx950). There is no CPU fallback.")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(code: int) -> None:
+    if code != RFA_OK:
+        raise RfaHipError(code, load().rfa_last_error().decode())
+
+
+def declared_symbols() -> list:
+    """Function names declared in include/rfa_hip.h."""
+    with open(HEADER_PATH) as f:
+        text = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(rfa_[a-z0-9_]+)\s*\(", text)))

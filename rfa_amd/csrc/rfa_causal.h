@@ -1,0 +1,850 @@
+// Causal random-feature attention as a chunked scan on MFMA tiles (gfx950).
+//
+// Replaces the reference's serial-in-time kernels
+//   rfa_forward   (random_feature_attention/cuda/forward.cu:86-126)
+//   rfa_backward  (random_feature_attention/cuda/backward.cu:453-527)
+// and computes the formulas of RFA.forward_torch / RFA.backward_torch
+// (random_feature_attention/rfa.py:46-103) with fp16 inputs, fp32 accumulation
+// and an fp32 running state.
+//
+// Work decomposition.  One (batch*head) sequence n is cut into `nseg` segments
+// of `seg_len` steps (a multiple of 64); one workgroup handles one (n, segment)
+// and walks its 64-step chunks serially, carrying the state
+//     S[k][c] = sum_t phi_k[t][k] v[t][c]   (K x d, fp32, in MFMA accumulators)
+//     z[k]    = sum_t phi_k[t][k]           (K,     fp32)
+// Segment totals are produced by a first pass (k_segment_state) and summed by
+// the consumer, so all (n, segment) workgroups of a pass run concurrently.
+//
+// Per chunk (Q, K: 64 x KD features; V, G: 64 x DH values), forward:
+//     A   = tril(Q K^T)                       den_raw = rowsum(A) + Q z
+//     out = (A V + Q S) / max(den_raw, 1)     S += K^T V ;  z += K^T 1
+// backward, forward-in-time sweep (k_causal_bwd_dq):
+//     X = G V^T, Y = G S^T                    e = rowsum(A*X) + rowsum(Q*Y)  (= G . num)
+//     den = max(den_raw,1);  gz = den_raw > 1 ? -e/den^2 : 0     (rfa.py:87-91)
+//     P = tril(X/den + gz 1^T);  dQ = P K + Y/den + gz z^T       (rfa.py:93-94)
+//     dR += Q^T (G/den);  dr += Q^T gz       (segment totals for the reverse sweep)
+// backward, reverse-in-time sweep (k_causal_bwd_dkdv), R/r = sums over later steps:
+//     dK = P^T Q + V R^T + 1 r^T ;  dV = A^T (G/den) + K R      (rfa.py:96-101)
+//     R += Q^T (G/den);  r += Q^T gz
+#pragma once
+#include "rfa_common.h"
+
+namespace rfa {
+
+template <int KD, int DH>
+struct CausalCfg {
+    static_assert(KD % 64 == 0 && DH % 64 == 0, "KD and DH must be multiples of 64");
+    static constexpr int C = kChunk;
+    static constexpr int LDQ = KD + 16;   // +16 halves: conflict-free transposing reads
+    static constexpr int LDV = DH + 16;
+    static constexpr int LDA = C + 8;
+    static constexpr int DS = DH / 4;     // value columns owned by one wave
+    static constexpr int KS = KD / 4;     // feature rows owned by one wave
+    static constexpr size_t kSegStateLds = (size_t)(C * LDQ + C * LDV) * 2;
+    static constexpr size_t kFwdLds = (size_t)(2 * C * LDQ + C * LDV + C * LDA) * 2 + (KD + C) * 4;
+    static constexpr size_t kBwdDqLds =
+        (size_t)(2 * C * LDQ + 2 * C * LDV + C * LDA) * 2 + (size_t)(KD + 8 * C) * 4;
+    static constexpr size_t kBwdDkLds =
+        (size_t)(2 * C * LDQ + 2 * C * LDV + 2 * C * LDA) * 2 + (size_t)(KD + C) * 4;
+};
+
+// ---------------------------------------------------------------------------
+// pass 0: per-segment totals  dS = K^T V (KD x DH),  dz = K^T 1
+// grid = N * (nseg - 1): the last segment's total is never consumed.
+// ---------------------------------------------------------------------------
+template <int KD, int DH>
+__global__ __launch_bounds__(kThreads) void k_segment_state(
+    const half_t* __restrict__ k, const half_t* __restrict__ v, float* __restrict__ wsS,
+    float* __restrict__ wsZ, int T, int N, int nseg, int seg_len) {
+    using Cfg = CausalCfg<KD, DH>;
+    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, DS = Cfg::DS;
+    constexpr int NKT = KD / 16, NCT = DS / 16;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    half_t* Ks = reinterpret_cast<half_t*>(smem_raw);
+    half_t* Vs = Ks + C * LDQ;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, G = lane >> 4;
+    const int n = blockIdx.x / (nseg - 1), seg = blockIdx.x % (nseg - 1);
+    const int t_begin = seg * seg_len;
+    const int t_end = min(T, t_begin + seg_len);
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+    const half_t* kb = k + (int64_t)n * KD;
+    const half_t* vb = v + (int64_t)n * DH;
+
+    f4 S[NKT][NCT];
+#pragma unroll
+    for (int a = 0; a < NKT; ++a)
+#pragma unroll
+        for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
+    float zreg = 0.f;
+
+    ChunkRegs<KD> rk;
+    ChunkRegs<DH> rv;
+    chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
+    chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
+    for (int t0 = t_begin; t0 < t_end; t0 += C) {
+        chunk_r2s<KD>(rk, Ks, LDQ, tid);
+        chunk_r2s<DH>(rv, Vs, LDV, tid);
+        __syncthreads();
+        if (t0 + C < t_end) {
+            chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, t_end - t0 - C, tid);
+            chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, t_end - t0 - C, tid);
+        }
+        h8 bv[NCT][2];
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+            for (int js = 0; js < 2; ++js) bv[ct][js] = col8(Vs, LDV, js * 32, w * DS + 16 * ct, lane);
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+            for (int js = 0; js < 2; ++js) {
+                h8 ak = col8(Ks, LDQ, js * 32, 16 * kt, lane);
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, bv[ct][js], S[kt][ct]);
+            }
+        if (tid < KD) {
+            float s = 0.f;
+#pragma unroll 8
+            for (int j = 0; j < C; ++j) s += (float)Ks[j * LDQ + tid];
+            zreg += s;
+        }
+        __syncthreads();
+    }
+    float* so = wsS + ((int64_t)(n * nseg + seg) * KD) * DH;
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                so[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row] = S[kt][ct][e];
+    if (tid < KD) wsZ[(int64_t)(n * nseg + seg) * KD + tid] = zreg;
+}
+
+// ---------------------------------------------------------------------------
+// forward scan.  Wave w owns value columns [w*DS, (w+1)*DS) of S (all KD rows),
+// held as accumulator tiles S[kt][ct] with element (k = 16kt+4G+e, c = w*DS+16ct+i).
+// ---------------------------------------------------------------------------
+template <int KD, int DH>
+__global__ __launch_bounds__(kThreads) void k_causal_fwd(
+    const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ, int T,
+    int N, int nseg, int seg_len) {
+    using Cfg = CausalCfg<KD, DH>;
+    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = Cfg::DS;
+    constexpr int NKT = KD / 16, NCT = DS / 16;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
+    half_t* Ks = Qs + C * LDQ;
+    half_t* Vs = Ks + C * LDQ;
+    half_t* As = Vs + C * LDV;
+    float* zs = reinterpret_cast<float*>(As + C * LDA);
+    float* dens = zs + KD;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, G = lane >> 4;
+    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    const int t_begin = seg * seg_len;
+    const int t_end = min(T, t_begin + seg_len);
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+    const half_t* qb = q + (int64_t)n * KD;
+    const half_t* kb = k + (int64_t)n * KD;
+    const half_t* vb = v + (int64_t)n * DH;
+    half_t* ob = out + (int64_t)n * DH;
+
+    // carried state = sum of the totals of all earlier segments
+    f4 S[NKT][NCT];
+#pragma unroll
+    for (int a = 0; a < NKT; ++a)
+#pragma unroll
+        for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
+    float zreg = 0.f;
+    for (int s = 0; s < seg; ++s) {
+        const float* si = wsS + ((int64_t)(n * nseg + s) * KD) * DH;
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    S[kt][ct][e] += si[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row];
+        if (tid < KD) zreg += wsZ[(int64_t)(n * nseg + s) * KD + tid];
+    }
+
+    ChunkRegs<KD> rq, rk;
+    ChunkRegs<DH> rv;
+    chunk_g2r<KD>(rq, qb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
+    chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
+    chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
+
+    for (int t0 = t_begin; t0 < t_end; t0 += C) {
+        chunk_r2s<KD>(rq, Qs, LDQ, tid);
+        chunk_r2s<KD>(rk, Ks, LDQ, tid);
+        chunk_r2s<DH>(rv, Vs, LDV, tid);
+        if (tid < KD) zs[tid] = zreg;
+        __syncthreads();
+        if (t0 + C < t_end) {
+            const int rows = t_end - t0 - C;
+            chunk_g2r<KD>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+            chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+            chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+        }
+
+        // ---- phase A: wave w computes rows i in [16w, 16w+16) of A (as A^T tiles, m=j, n=i)
+        {
+            f4 at[4];
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) at[jt] = f4_zero();
+#pragma unroll
+            for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt)
+                    if (jt <= w) at[jt] = mfma32(row8(Ks, LDQ, 16 * jt + row, ks * 32, G), bq, at[jt]);
+            }
+            float part = 0.f;
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                if (jt == w) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (4 * G + e > row) at[jt][e] = 0.f;   // keep j <= i
+                }
+                if (jt <= w) part += at[jt][0] + at[jt][1] + at[jt][2] + at[jt][3];
+            }
+            // + q_i . z  (this lane covers features [G*KD/4, (G+1)*KD/4))
+#pragma unroll
+            for (int kk = 0; kk < KD / 4; kk += 8) {
+                h8 qv = *reinterpret_cast<const h8*>(Qs + (16 * w + row) * LDQ + G * (KD / 4) + kk);
+                f4 z0 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk);
+                f4 z1 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    part += (float)qv[e] * z0[e];
+                    part += (float)qv[4 + e] * z1[e];
+                }
+            }
+            part = sum_over_groups(part);
+            if (G == 0) dens[16 * w + row] = fmaxf(part, 1.0f);
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                h4 hv = (jt <= w) ? to_h4(at[jt]) : h4_zero();
+                *reinterpret_cast<h4*>(As + (16 * w + row) * LDA + 16 * jt + 4 * G) = hv;
+            }
+        }
+        __syncthreads();
+
+        // ---- phase B: out^T tiles (m=c, n=i) for this wave's value columns, then state update
+        {
+            h8 av[NCT][2];   // V column fragments: element V[j = 32js+8G+e][c = w*DS+16ct+i]
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                for (int js = 0; js < 2; ++js) av[ct][js] = col8(Vs, LDV, js * 32, w * DS + 16 * ct, lane);
+
+            f4 acc[4][NCT];
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = f4_zero();
+#pragma unroll
+                for (int js = 0; js < 2; ++js) {
+                    if (js == 0 || it >= 2) {
+                        h8 ba = row8(As, LDA, 16 * it + row, js * 32, G);
+#pragma unroll
+                        for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = mfma32(av[ct][js], ba, acc[it][ct]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 hi[NCT], lo[NCT];
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct) acc_to_operand(S[2 * ks][ct], S[2 * ks + 1][ct], hi[ct], lo[ct]);
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    h8 bq = row_split8(Qs, LDQ, 16 * it + row, ks * 32, G);
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct) {
+                        acc[it][ct] = mfma32(hi[ct], bq, acc[it][ct]);
+                        acc[it][ct] = mfma32(lo[ct], bq, acc[it][ct]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int i = 16 * it + row;
+                const float inv = 1.0f / dens[i];
+                if (t0 + i < t_end) {
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct) {
+                        f4 o = acc[it][ct];
+                        o[0] *= inv; o[1] *= inv; o[2] *= inv; o[3] *= inv;
+                        *reinterpret_cast<h4*>(ob + (int64_t)(t0 + i) * v_stride + w * DS + 16 * ct + 4 * G) = to_h4(o);
+                    }
+                }
+            }
+            // S (m=k, n=c) += K^T V
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int js = 0; js < 2; ++js) {
+                    h8 ak = col8(Ks, LDQ, js * 32, 16 * kt, lane);
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, av[ct][js], S[kt][ct]);
+                }
+            if (tid < KD) {
+                float s = 0.f;
+#pragma unroll 8
+                for (int j = 0; j < C; ++j) s += (float)Ks[j * LDQ + tid];
+                zreg += s;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------
+// backward, forward-in-time sweep: dQ, per-step (den, gz) stash, segment totals
+// dR = Q^T (G/den), dr = Q^T gz.  Wave w owns feature rows [w*KS, (w+1)*KS):
+// ST[ct][kt] / RT[ct][kt] hold element (c = 16ct+4G+e, k = w*KS+16kt+i).
+// ---------------------------------------------------------------------------
+template <int KD, int DH>
+__global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
+    const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    const half_t* __restrict__ g, half_t* __restrict__ dq, const float* __restrict__ wsS,
+    const float* __restrict__ wsZ, float* __restrict__ wsR, float* __restrict__ wsr,
+    float* __restrict__ den_ws, float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len) {
+    using Cfg = CausalCfg<KD, DH>;
+    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS;
+    constexpr int NKT = KS / 16, NCT = DH / 16;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
+    half_t* Ks = Qs + C * LDQ;
+    half_t* Vs = Ks + C * LDQ;
+    half_t* Gs = Vs + C * LDV;
+    half_t* Ps = Gs + C * LDV;
+    float* zs = reinterpret_cast<float*>(Ps + C * LDA);
+    float* drs = zs + KD;       // den_raw per row
+    float* e1s = drs + C;       // rowsum(A*X)
+    float* e2p = e1s + C;       // [4][C] per-wave partial rowsum(Q*Y)
+    float* dens = e2p + 4 * C;
+    float* gzs = dens + C;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, G = lane >> 4;
+    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    const int t_begin = seg * seg_len;
+    const int t_end = min(T, t_begin + seg_len);
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+    const half_t* qb = q + (int64_t)n * KD;
+    const half_t* kb = k + (int64_t)n * KD;
+    const half_t* vb = v + (int64_t)n * DH;
+    const half_t* gb = g + (int64_t)n * DH;
+    half_t* dqb = dq + (int64_t)n * KD;
+
+    f4 ST[NCT][NKT], RT[NCT][NKT];
+#pragma unroll
+    for (int a = 0; a < NCT; ++a)
+#pragma unroll
+        for (int b = 0; b < NKT; ++b) { ST[a][b] = f4_zero(); RT[a][b] = f4_zero(); }
+    float zreg = 0.f, rreg = 0.f;
+    for (int s = 0; s < seg; ++s) {
+        const float* si = wsS + ((int64_t)(n * nseg + s) * KD) * DH;
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) {
+                f4 x = *reinterpret_cast<const f4*>(si + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
+                ST[ct][kt] += x;
+            }
+        if (tid < KD) zreg += wsZ[(int64_t)(n * nseg + s) * KD + tid];
+    }
+
+    ChunkRegs<KD> rq, rk;
+    ChunkRegs<DH> rv, rg;
+    {
+        const int rows = t_end - t_begin;
+        chunk_g2r<KD>(rq, qb + (int64_t)t_begin * k_stride, k_stride, rows, tid);
+        chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, rows, tid);
+        chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, rows, tid);
+        chunk_g2r<DH>(rg, gb + (int64_t)t_begin * v_stride, v_stride, rows, tid);
+    }
+
+    for (int t0 = t_begin; t0 < t_end; t0 += C) {
+        chunk_r2s<KD>(rq, Qs, LDQ, tid);
+        chunk_r2s<KD>(rk, Ks, LDQ, tid);
+        chunk_r2s<DH>(rv, Vs, LDV, tid);
+        chunk_r2s<DH>(rg, Gs, LDV, tid);
+        if (tid < KD) zs[tid] = zreg;
+        __syncthreads();
+        if (t0 + C < t_end) {
+            const int rows = t_end - t0 - C;
+            chunk_g2r<KD>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+            chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+            chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+            chunk_g2r<DH>(rg, gb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+        }
+
+        // ---- phase A
+        f4 xt[4];           // X^T tiles (m=j, n=i) for rows i of this wave, kept for phase C
+        f4 yt[NKT][4];      // Y^T tiles (m=k, n=i), k in this wave's slice, all i
+        {
+            f4 at[4];
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) { at[jt] = f4_zero(); xt[jt] = f4_zero(); }
+#pragma unroll
+            for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt)
+                    if (jt <= w) at[jt] = mfma32(row8(Ks, LDQ, 16 * jt + row, ks * 32, G), bq, at[jt]);
+            }
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 bg = row8(Gs, LDV, 16 * w + row, cs * 32, G);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt)
+                    if (jt <= w) xt[jt] = mfma32(row8(Vs, LDV, 16 * jt + row, cs * 32, G), bg, xt[jt]);
+            }
+            float part_d = 0.f, part_e = 0.f;
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                if (jt == w) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (4 * G + e > row) at[jt][e] = 0.f;
+                }
+                if (jt <= w) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        part_d += at[jt][e];
+                        part_e += at[jt][e] * xt[jt][e];
+                    }
+                }
+            }
+#pragma unroll
+            for (int kk = 0; kk < KD / 4; kk += 8) {
+                h8 qv = *reinterpret_cast<const h8*>(Qs + (16 * w + row) * LDQ + G * (KD / 4) + kk);
+                f4 z0 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk);
+                f4 z1 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    part_d += (float)qv[e] * z0[e];
+                    part_d += (float)qv[4 + e] * z1[e];
+                }
+            }
+            part_d = sum_over_groups(part_d);
+            part_e = sum_over_groups(part_e);
+            if (G == 0) {
+                drs[16 * w + row] = part_d;
+                e1s[16 * w + row] = part_e;
+            }
+
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int it = 0; it < 4; ++it) yt[kt][it] = f4_zero();
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 hi[NKT], lo[NKT];
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) acc_to_operand(ST[2 * cs][kt], ST[2 * cs + 1][kt], hi[kt], lo[kt]);
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    h8 bg = row_split8(Gs, LDV, 16 * it + row, cs * 32, G);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) {
+                        yt[kt][it] = mfma32(hi[kt], bg, yt[kt][it]);
+                        yt[kt][it] = mfma32(lo[kt], bg, yt[kt][it]);
+                    }
+                }
+            }
+            float e2[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    h4 qv = *reinterpret_cast<const h4*>(Qs + (16 * it + row) * LDQ + w * KS + 16 * kt + 4 * G);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) e2[it] += yt[kt][it][e] * (float)qv[e];
+                }
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                float x = sum_over_groups(e2[it]);
+                if (G == 0) e2p[w * C + 16 * it + row] = x;
+            }
+        }
+        __syncthreads();
+
+        // ---- phase B: denominators and d(qz) for the 64 rows of the chunk
+        if (tid < C) {
+            const float dr = drs[tid];
+            const float den = fmaxf(dr, 1.0f);
+            const float e = e1s[tid] + ((e2p[tid] + e2p[C + tid]) + (e2p[2 * C + tid] + e2p[3 * C + tid]));
+            const float gz = (dr > 1.0f) ? -e / (den * den) : 0.f;
+            dens[tid] = den;
+            gzs[tid] = gz;
+            if (t0 + tid < t_end) {
+                den_ws[(int64_t)(t0 + tid) * N + n] = den;
+                gz_ws[(int64_t)(t0 + tid) * N + n] = gz;
+            }
+        }
+        __syncthreads();
+
+        // ---- phase C: P rows of this wave; G <- G/den in place
+        {
+            const int i = 16 * w + row;
+            const float inv = 1.0f / dens[i];
+            const float gzi = gzs[i];
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                h4 pv = h4_zero();
+                if (jt <= w) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int j = 16 * jt + 4 * G + e;
+                        pv[e] = (j <= i) ? (half_t)(xt[jt][e] * inv + gzi) : (half_t)0.f;
+                    }
+                }
+                *reinterpret_cast<h4*>(Ps + i * LDA + 16 * jt + 4 * G) = pv;
+            }
+            constexpr int PPR = DH / 8;
+#pragma unroll
+            for (int it = 0; it < ChunkRegs<DH>::kPieces; ++it) {
+                const int p = tid + kThreads * it;
+                const int r_ = p / PPR, c8 = p % PPR;
+                const float sc = 1.0f / dens[r_];
+                h8 x = *reinterpret_cast<const h8*>(Gs + r_ * LDV + c8 * 8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (half_t)((float)x[e] * sc);
+                *reinterpret_cast<h8*>(Gs + r_ * LDV + c8 * 8) = x;
+            }
+        }
+        __syncthreads();
+
+        // ---- phase D: dQ^T tiles (m=k, n=i), then the carried sums
+        {
+            h8 kf[NKT][2];   // K column fragments: K[j = 32js+8G+e][k = w*KS+16kt+i]
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int js = 0; js < 2; ++js) kf[kt][js] = col8(Ks, LDQ, js * 32, w * KS + 16 * kt, lane);
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int i = 16 * it + row;
+                const float inv = 1.0f / dens[i];
+                const float gzi = gzs[i];
+                h8 bp0 = row8(Ps, LDA, i, 0, G);
+                h8 bp1 = row8(Ps, LDA, i, 32, G);
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) {
+                    f4 zv = *reinterpret_cast<const f4*>(zs + w * KS + 16 * kt + 4 * G);
+                    f4 acc;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e] = yt[kt][it][e] * inv + gzi * zv[e];
+                    acc = mfma32(kf[kt][0], bp0, acc);
+                    if (it >= 2) acc = mfma32(kf[kt][1], bp1, acc);
+                    if (t0 + i < t_end)
+                        *reinterpret_cast<h4*>(dqb + (int64_t)(t0 + i) * k_stride + w * KS + 16 * kt + 4 * G) = to_h4(acc);
+                }
+            }
+#pragma unroll
+            for (int js = 0; js < 2; ++js) {
+                h8 qf[NKT];   // Q column fragments
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) qf[kt] = col8(Qs, LDQ, js * 32, w * KS + 16 * kt, lane);
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct) {
+                    h8 gf = col8(Gs, LDV, js * 32, 16 * ct, lane);
+                    h8 vf = col8(Vs, LDV, js * 32, 16 * ct, lane);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) {
+                        RT[ct][kt] = mfma32(gf, qf[kt], RT[ct][kt]);
+                        ST[ct][kt] = mfma32(vf, kf[kt][js], ST[ct][kt]);
+                    }
+                }
+            }
+            if (tid < KD) {
+                float sz = 0.f, sr = 0.f;
+#pragma unroll 8
+                for (int j = 0; j < C; ++j) {
+                    sz += (float)Ks[j * LDQ + tid];
+                    sr += (float)Qs[j * LDQ + tid] * gzs[j];
+                }
+                zreg += sz;
+                rreg += sr;
+            }
+        }
+        __syncthreads();
+    }
+
+    if (seg > 0) {   // totals of segment 0 are never consumed
+        float* ro = wsR + ((int64_t)(n * nseg + seg) * KD) * DH;
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+                *reinterpret_cast<f4*>(ro + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G) = RT[ct][kt];
+        if (tid < KD) wsr[(int64_t)(n * nseg + seg) * KD + tid] = rreg;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// backward, reverse-in-time sweep: dK, dV.  R is carried twice, once per
+// contraction: RT[ct][kt] (c = 16ct+4G+e, k = w*KS+16kt+i) contracts over c for
+// dK; RR[kt][ct] (k = 16kt+4G+e, c = w*DS+16ct+i) contracts over k for dV.
+// ---------------------------------------------------------------------------
+template <int KD, int DH>
+__global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
+    const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    const half_t* __restrict__ g, half_t* __restrict__ dk, half_t* __restrict__ dv,
+    const float* __restrict__ wsR, const float* __restrict__ wsr, const float* __restrict__ den_ws,
+    const float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len) {
+    using Cfg = CausalCfg<KD, DH>;
+    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS, DS = Cfg::DS;
+    constexpr int NKT = KS / 16, NCT = DH / 16;      // RT tiles
+    constexpr int NKT2 = KD / 16, NCT2 = DS / 16;    // RR tiles
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
+    half_t* Ks = Qs + C * LDQ;
+    half_t* Vs = Ks + C * LDQ;
+    half_t* Gs = Vs + C * LDV;       // G / den
+    half_t* ATs = Gs + C * LDV;      // AT[j][i] = A[i][j]
+    half_t* PTs = ATs + C * LDA;     // PT[j][i] = P[i][j]
+    float* rs = reinterpret_cast<float*>(PTs + C * LDA);
+    float* gzs = rs + KD;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, G = lane >> 4;
+    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    const int t_begin = seg * seg_len;
+    const int t_end = min(T, t_begin + seg_len);
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+    const half_t* qb = q + (int64_t)n * KD;
+    const half_t* kb = k + (int64_t)n * KD;
+    const half_t* vb = v + (int64_t)n * DH;
+    const half_t* gb = g + (int64_t)n * DH;
+    half_t* dkb = dk + (int64_t)n * KD;
+    half_t* dvb = dv + (int64_t)n * DH;
+
+    f4 RT[NCT][NKT], RR[NKT2][NCT2];
+#pragma unroll
+    for (int a = 0; a < NCT; ++a)
+#pragma unroll
+        for (int b = 0; b < NKT; ++b) RT[a][b] = f4_zero();
+#pragma unroll
+    for (int a = 0; a < NKT2; ++a)
+#pragma unroll
+        for (int b = 0; b < NCT2; ++b) RR[a][b] = f4_zero();
+    float rreg = 0.f;
+    for (int s = seg + 1; s < nseg; ++s) {
+        const float* ri = wsR + ((int64_t)(n * nseg + s) * KD) * DH;
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+                RT[ct][kt] += *reinterpret_cast<const f4*>(ri + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
+#pragma unroll
+        for (int kt = 0; kt < NKT2; ++kt)
+#pragma unroll
+            for (int ct = 0; ct < NCT2; ++ct)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    RR[kt][ct][e] += ri[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row];
+        if (tid < KD) rreg += wsr[(int64_t)(n * nseg + s) * KD + tid];
+    }
+
+    ChunkRegs<KD> rq, rk;
+    ChunkRegs<DH> rv, rg;
+    float inv_den[ChunkRegs<DH>::kPieces];
+    float gz_next = 0.f;
+    constexpr int PPRV = DH / 8;
+    auto prefetch = [&](int t0) {
+        const int rows = t_end - t0;
+        chunk_g2r<KD>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<KD>(rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<DH>(rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+        chunk_g2r<DH>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+#pragma unroll
+        for (int it = 0; it < ChunkRegs<DH>::kPieces; ++it) {
+            const int r_ = (tid + kThreads * it) / PPRV;
+            inv_den[it] = (r_ < rows) ? 1.0f / den_ws[(int64_t)(t0 + r_) * N + n] : 0.f;
+        }
+        gz_next = (tid < C && tid < rows) ? gz_ws[(int64_t)(t0 + tid) * N + n] : 0.f;
+    };
+
+    const int n_chunks = (t_end - t_begin + C - 1) / C;
+    prefetch(t_begin + (n_chunks - 1) * C);
+    for (int ci = n_chunks - 1; ci >= 0; --ci) {
+        const int t0 = t_begin + ci * C;
+        chunk_r2s<KD>(rq, Qs, LDQ, tid);
+        chunk_r2s<KD>(rk, Ks, LDQ, tid);
+        chunk_r2s<DH>(rv, Vs, LDV, tid);
+        chunk_r2s_scaled<DH>(rg, inv_den, Gs, LDV, tid);
+        if (tid < C) gzs[tid] = gz_next;
+        if (tid < KD) rs[tid] = rreg;
+        __syncthreads();
+        if (ci > 0) prefetch(t0 - C);
+
+        // ---- phase A: wave w computes columns j in [16w, 16w+16) of A and P (tiles m=i, n=j)
+        {
+            f4 a_[4], p_[4];
+#pragma unroll
+            for (int it = 0; it < 4; ++it) { a_[it] = f4_zero(); p_[it] = f4_zero(); }
+#pragma unroll
+            for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 bk = row8(Ks, LDQ, 16 * w + row, ks * 32, G);
+#pragma unroll
+                for (int it = 0; it < 4; ++it)
+                    if (it >= w) a_[it] = mfma32(row8(Qs, LDQ, 16 * it + row, ks * 32, G), bk, a_[it]);
+            }
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 bv = row8(Vs, LDV, 16 * w + row, cs * 32, G);
+#pragma unroll
+                for (int it = 0; it < 4; ++it)
+                    if (it >= w) p_[it] = mfma32(row8(Gs, LDV, 16 * it + row, cs * 32, G), bv, p_[it]);
+            }
+            const int j = 16 * w + row;
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                h4 av = h4_zero(), pv = h4_zero();
+                if (it >= w) {
+                    f4 gzv = *reinterpret_cast<const f4*>(gzs + 16 * it + 4 * G);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int i = 16 * it + 4 * G + e;
+                        if (i >= j) {
+                            av[e] = (half_t)a_[it][e];
+                            pv[e] = (half_t)(p_[it][e] + gzv[e]);
+                        }
+                    }
+                }
+                *reinterpret_cast<h4*>(ATs + j * LDA + 16 * it + 4 * G) = av;
+                *reinterpret_cast<h4*>(PTs + j * LDA + 16 * it + 4 * G) = pv;
+            }
+        }
+        __syncthreads();
+
+        // ---- phase B
+        {
+            h8 qf[NKT][2];    // Q column fragments for this wave's feature slice
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int is = 0; is < 2; ++is) qf[kt][is] = col8(Qs, LDQ, is * 32, w * KS + 16 * kt, lane);
+            h8 gf2[NCT2][2];  // (G/den) column fragments for this wave's value slice
+#pragma unroll
+            for (int ct = 0; ct < NCT2; ++ct)
+#pragma unroll
+                for (int is = 0; is < 2; ++is) gf2[ct][is] = col8(Gs, LDV, is * 32, w * DS + 16 * ct, lane);
+
+            // dK^T tiles (m=k, n=j)
+            f4 dkacc[NKT][4];
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) {
+                f4 rv4 = *reinterpret_cast<const f4*>(rs + w * KS + 16 * kt + 4 * G);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    f4 acc = rv4;
+                    if (jt < 2) acc = mfma32(qf[kt][0], row8(PTs, LDA, 16 * jt + row, 0, G), acc);
+                    acc = mfma32(qf[kt][1], row8(PTs, LDA, 16 * jt + row, 32, G), acc);
+                    dkacc[kt][jt] = acc;
+                }
+            }
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 hi[NKT], lo[NKT];
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) acc_to_operand(RT[2 * cs][kt], RT[2 * cs + 1][kt], hi[kt], lo[kt]);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    h8 bvv = row_split8(Vs, LDV, 16 * jt + row, cs * 32, G);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) {
+                        dkacc[kt][jt] = mfma32(hi[kt], bvv, dkacc[kt][jt]);
+                        dkacc[kt][jt] = mfma32(lo[kt], bvv, dkacc[kt][jt]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                const int jj = 16 * jt + row;
+                if (t0 + jj < t_end) {
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt)
+                        *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + w * KS + 16 * kt + 4 * G) = to_h4(dkacc[kt][jt]);
+                }
+            }
+
+            // dV^T tiles (m=c, n=j)
+            f4 dvacc[NCT2][4];
+#pragma unroll
+            for (int ct = 0; ct < NCT2; ++ct)
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    f4 acc = f4_zero();
+                    if (jt < 2) acc = mfma32(gf2[ct][0], row8(ATs, LDA, 16 * jt + row, 0, G), acc);
+                    acc = mfma32(gf2[ct][1], row8(ATs, LDA, 16 * jt + row, 32, G), acc);
+                    dvacc[ct][jt] = acc;
+                }
+#pragma unroll
+            for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 hi[NCT2], lo[NCT2];
+#pragma unroll
+                for (int ct = 0; ct < NCT2; ++ct) acc_to_operand(RR[2 * ks][ct], RR[2 * ks + 1][ct], hi[ct], lo[ct]);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    h8 bkk = row_split8(Ks, LDQ, 16 * jt + row, ks * 32, G);
+#pragma unroll
+                    for (int ct = 0; ct < NCT2; ++ct) {
+                        dvacc[ct][jt] = mfma32(hi[ct], bkk, dvacc[ct][jt]);
+                        dvacc[ct][jt] = mfma32(lo[ct], bkk, dvacc[ct][jt]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                const int jj = 16 * jt + row;
+                if (t0 + jj < t_end) {
+#pragma unroll
+                    for (int ct = 0; ct < NCT2; ++ct)
+                        *reinterpret_cast<h4*>(dvb + (int64_t)(t0 + jj) * v_stride + w * DS + 16 * ct + 4 * G) = to_h4(dvacc[ct][jt]);
+                }
+            }
+
+            // carried sums
+#pragma unroll
+            for (int is = 0; is < 2; ++is) {
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct) {
+                    h8 gf = col8(Gs, LDV, is * 32, 16 * ct, lane);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) RT[ct][kt] = mfma32(gf, qf[kt][is], RT[ct][kt]);
+                }
+#pragma unroll
+                for (int kt = 0; kt < NKT2; ++kt) {
+                    h8 qa = col8(Qs, LDQ, is * 32, 16 * kt, lane);
+#pragma unroll
+                    for (int ct = 0; ct < NCT2; ++ct) RR[kt][ct] = mfma32(qa, gf2[ct][is], RR[kt][ct]);
+                }
+            }
+            if (tid < KD) {
+                float sr = 0.f;
+#pragma unroll 8
+                for (int i = 0; i < C; ++i) sr += (float)Qs[i * LDQ + tid] * gzs[i];
+                rreg += sr;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace rfa

@@ -1,0 +1,169 @@
+// Device-side building blocks shared by the RFA kernels (gfx950 / CDNA4 only).
+//
+// Conventions used everywhere in this directory
+//   * a workgroup is 256 threads = 4 wavefronts of 64 lanes;
+//   * lane = 16*G + i  (G = lane/16 in 0..3, i = lane%16);
+//   * MFMA v_mfma_f32_16x16x32_f16 computes  D[m][n] += sum_r A[m][r] * B[n][r]
+//     with, per lane,  A operand = 8 halves A[m=i][r=8G..8G+7],
+//                      B operand = 8 halves B[n=i][r=8G..8G+7],
+//                      D         = 4 floats D[m=4G+e][n=i], e=0..3.
+//     (layout checked on hardware by tests/test_gpu_mfma_layout.py)
+//   * consequence used throughout: an accumulator tile D is itself a valid A or
+//     B operand for a later MFMA that contracts over D's *row* index m, with the
+//     "split" slot order  slots 0..3 <-> m = 4G+e of tile t,
+//                         slots 4..7 <-> m = 4G+e of tile t+1;
+//     the other operand is then read with the same slot order (row_split8).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rfa {
+
+typedef _Float16 half_t;
+typedef half_t h2 __attribute__((ext_vector_type(2)));
+typedef half_t h4 __attribute__((ext_vector_type(4)));
+typedef half_t h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;   // threads per workgroup
+constexpr int kChunk = 64;      // time steps per chunk
+
+__device__ __forceinline__ f4 mfma32(h8 a, h8 b, f4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f4 f4_zero() { f4 z = {0.f, 0.f, 0.f, 0.f}; return z; }
+
+// 8 consecutive halves of one LDS row: X[row][c0 + 8G .. +7]   ("natural" slot order)
+__device__ __forceinline__ h8 row8(const half_t* X, int ld, int row, int c0, int G) {
+    return *reinterpret_cast<const h8*>(X + row * ld + c0 + 8 * G);
+}
+
+// "split" slot order: X[row][c0 + 4G + e] (e=0..3) then X[row][c0 + 16 + 4G + e]
+__device__ __forceinline__ h8 row_split8(const half_t* X, int ld, int row, int c0, int G) {
+    const half_t* p = X + row * ld + c0 + 4 * G;
+    h4 a = *reinterpret_cast<const h4*>(p);
+    h4 b = *reinterpret_cast<const h4*>(p + 16);
+    h8 r;
+    r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
+    r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
+    return r;
+}
+
+// LDS transposing read (ds_read_b64_tr_b16).  Within each group of 16 lanes the
+// hardware returns  out[lane i][e] = in[lane 4e + i/4][i%4]; with the address
+// pattern below lane (G,i) receives the column fragment
+//     X[r0 + 4G' + e][c0 + i],  e = 0..3,   where r0 already includes 4G' .
+__device__ __forceinline__ h4 tr_read4(const half_t* p) {
+    typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 fp16x4;
+    typedef __attribute__((address_space(3))) fp16x4 lds_fp16x4;
+    fp16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_fp16x4*)(p));
+    h4 r;
+    r[0] = (half_t)v[0]; r[1] = (half_t)v[1]; r[2] = (half_t)v[2]; r[3] = (half_t)v[3];
+    return r;
+}
+
+// Column fragment in natural slot order: X[r0 + 8G + e][c0 + i], e = 0..7, from a
+// row-major LDS array (ld in halves, multiple of 4).  This is how an operand whose
+// contraction index is the *row* index of X is fed to the MFMA without keeping a
+// transposed copy of X.
+__device__ __forceinline__ h8 col8(const half_t* X, int ld, int r0, int c0, int lane) {
+    const int s = lane & 15, G = lane >> 4;
+    const half_t* p = X + (r0 + 8 * G + (s >> 2)) * ld + c0 + 4 * (s & 3);
+    h4 a = tr_read4(p);
+    h4 b = tr_read4(p + 4 * ld);
+    h8 r;
+    r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
+    r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
+    return r;
+}
+
+// Two fp32 accumulator tiles -> one fp16 operand pair (hi + lo carries ~22 bits),
+// split slot order (see header comment).
+__device__ __forceinline__ void acc_to_operand(const f4& t0, const f4& t1, h8& hi, h8& lo) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        half_t h0 = (half_t)t0[e];
+        half_t h1 = (half_t)t1[e];
+        hi[e] = h0;
+        hi[4 + e] = h1;
+        lo[e] = (half_t)(t0[e] - (float)h0);
+        lo[4 + e] = (half_t)(t1[e] - (float)h1);
+    }
+}
+
+__device__ __forceinline__ h4 to_h4(const f4& x) {
+    h4 r;
+    r[0] = (half_t)x[0]; r[1] = (half_t)x[1]; r[2] = (half_t)x[2]; r[3] = (half_t)x[3];
+    return r;
+}
+
+__device__ __forceinline__ h4 h4_zero() {
+    h4 r; r[0] = (half_t)0.f; r[1] = (half_t)0.f; r[2] = (half_t)0.f; r[3] = (half_t)0.f; return r;
+}
+
+// sum over the four 16-lane groups (lanes i, i+16, i+32, i+48)
+__device__ __forceinline__ float sum_over_groups(float x) {
+    x += __shfl_xor(x, 16, 64);
+    x += __shfl_xor(x, 32, 64);
+    return x;
+}
+
+// ---------------------------------------------------------------------------
+// chunk movement: a chunk is 64 consecutive time steps of one (batch, head)
+// sequence, F halves per step; in HBM consecutive steps are `row_stride` halves
+// apart ([T, N, F] time-major layout).
+// ---------------------------------------------------------------------------
+template <int F>
+struct ChunkRegs {
+    static constexpr int kPieces = kChunk * F / 8 / kThreads;   // 16-byte pieces per thread
+    static_assert(kPieces >= 1, "feature width too small for 256 threads");
+    uint4 v[kPieces];
+};
+
+template <int F>
+__device__ __forceinline__ void chunk_g2r(ChunkRegs<F>& r, const half_t* __restrict__ base,
+                                          int64_t row_stride, int rows_valid, int tid) {
+    constexpr int PPR = F / 8;
+#pragma unroll
+    for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
+        const int p = tid + kThreads * it;
+        const int row = p / PPR, c8 = p % PPR;
+        if (row < rows_valid) {
+            r.v[it] = *reinterpret_cast<const uint4*>(base + (int64_t)row * row_stride + c8 * 8);
+        } else {
+            r.v[it] = make_uint4(0u, 0u, 0u, 0u);
+        }
+    }
+}
+
+template <int F>
+__device__ __forceinline__ void chunk_r2s(const ChunkRegs<F>& r, half_t* Xs, int ld, int tid) {
+    constexpr int PPR = F / 8;
+#pragma unroll
+    for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
+        const int p = tid + kThreads * it;
+        const int row = p / PPR, c8 = p % PPR;
+        *reinterpret_cast<uint4*>(Xs + row * ld + c8 * 8) = r.v[it];
+    }
+}
+
+// same, each row multiplied by scale[piece] (fp32) before the store
+template <int F>
+__device__ __forceinline__ void chunk_r2s_scaled(const ChunkRegs<F>& r, const float* scale,
+                                                 half_t* Xs, int ld, int tid) {
+    constexpr int PPR = F / 8;
+#pragma unroll
+    for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
+        const int p = tid + kThreads * it;
+        const int row = p / PPR, c8 = p % PPR;
+        union { uint4 u; h8 h; } x;
+        x.u = r.v[it];
+        h8 y;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)x.h[e] * scale[it]);
+        *reinterpret_cast<h8*>(Xs + row * ld + c8 * 8) = y;
+    }
+}
+
+}  // namespace rfa
