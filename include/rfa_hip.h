@@ -79,6 +79,75 @@ int rfa_causal_backward(const void* q, const void* k, const void* v, const void*
  * shape (>= 1).  Environment variable RFA_HIP_NSEG overrides the heuristic. */
 int rfa_causal_num_segments(int64_t T, int64_t N);
 
+/* ---------------------------------------------------------------------------
+ * Feature map  phi(x) = scale * [sin(W x^), cos(W x^)],  x^ = x / (||x|| + 1e-3).
+ *
+ * rfa_feature_map_forward replaces random_project(x=..., random_matrices=...)
+ *   (random_feature_attention/utils.py:105-120, with _normalize :100-102); the
+ *   reference fixes scale = SCALE = 0.1 (utils.py:10,119).
+ *   x   : fp16 [R, H, d]   R = seq_len * bsz rows
+ *   w   : fp16 [H, D, d]   the matrix build_random_matrices returns (utils.py:90-97)
+ *   phi : fp16 [R, H, 2D]  sin block in columns [0, D), cos block in [D, 2D)
+ * rfa_feature_map_backward is the gradient the reference obtains from autograd
+ *   through those ATen calls: dx fp16 [R, H, d], dw fp32 [H, D, d] (summed over rows).
+ * Supported: D in {32, 64, 128}, d in {64, 128} (rfa_feature_map_supported).
+ * ------------------------------------------------------------------------- */
+int rfa_feature_map_supported(int D, int d);
+int rfa_feature_map_forward(const void* x, const void* w, void* phi, int64_t R, int H, int D, int d,
+                            float scale, void* stream);
+size_t rfa_feature_map_backward_workspace_bytes(int64_t R, int H, int D, int d);
+int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi, void* dx, float* dw,
+                             int64_t R, int H, int D, int d, float scale, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Cross attention (encoder -> decoder).  The state is fp32.
+ *
+ * rfa_cross_state replaces the two reductions of
+ *   CrossAttentionProjectLayer.project_and_reshape
+ *   (random_feature_attention/cross_attention.py:97-104):
+ *     s[b,h] = sum_s phi_k[s,b,h] (x) v[s,b,h] ;  z[b,h] = sum_s phi_k[s,b,h]
+ *   phi_k : fp16 [S, B*H, K];  v : fp16 [S, B*H, d]
+ *   key_padding_mask : bytes [B, S], non-zero = padded key (its phi_k row counts
+ *                      as zero, cross_attention.py:97-100), or NULL
+ *   s : fp32 [B*H, K, d];  z : fp32 [B*H, K]     (overwritten)
+ * rfa_cross_readout replaces CrossAttention.rfa after the feature map
+ *   (cross_attention.py:266-269):  out = (phi_q s) / max(|phi_q z|, 1)
+ *   phi_q : fp16 [T, N, K];  out : fp16 [T, N, d]
+ * The two *_backward functions are the gradients the reference obtains from
+ * autograd through those einsums:
+ *   readout: dphi_q fp16 [T, N, K], ds fp32 [N, K, d], dz fp32 [N, K] (overwritten)
+ *   state  : dphi_k fp16 [S, N, K] (zero rows at padded keys), dv fp16 [S, N, d]
+ * ------------------------------------------------------------------------- */
+int rfa_cross_state(const void* phi_k, const void* v, const uint8_t* key_padding_mask, float* s, float* z,
+                    int64_t S_len, int64_t B, int H, int K, int d, void* stream);
+int rfa_cross_readout(const void* phi_q, const float* s, const float* z, void* out, int64_t T, int64_t N,
+                      int K, int d, void* stream);
+int rfa_cross_readout_backward(const void* phi_q, const float* s, const float* z, const void* grad_attn,
+                               void* dphi_q, float* ds, float* dz, int64_t T, int64_t N, int K, int d,
+                               void* stream);
+int rfa_cross_state_backward(const void* phi_k, const void* v, const uint8_t* key_padding_mask,
+                             const float* ds, const float* dz, void* dphi_k, void* dv, int64_t S_len,
+                             int64_t B, int H, int K, int d, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Incremental decoding.  The fp32 state (s [N, K, d], z [N, K]) is updated IN
+ * PLACE; one kernel is launched per step, in order, on `stream`.
+ *
+ * rfa_incremental replaces incremental_rfa(phi_q=, phi_k=, v=, s=, z=)
+ *   (random_feature_attention/causal_attention.py:17-54), whose loop over tgt_len
+ *   is the `steps` loop here:
+ *   phi_q, phi_k : fp16 [steps, N, K];  v : fp16 [steps, N, d];  out : fp16 [steps, N, d]
+ * rfa_incremental_fused additionally evaluates the feature map of the raw projected
+ *   q, k inside the step kernel, i.e. the decode branch of CausalAttention.forward
+ *   (causal_attention.py:241-265) in one launch per token:
+ *   q, k, v : fp16 [steps, B, H, d];  w : fp16 [H, D, d];  K = 2D
+ * ------------------------------------------------------------------------- */
+int rfa_incremental(const void* phi_q, const void* phi_k, const void* v, float* s, float* z, void* out,
+                    int64_t steps, int64_t N, int K, int d, void* stream);
+int rfa_incremental_fused(const void* q, const void* k, const void* v, const void* w, float scale, float* s,
+                          float* z, void* out, int64_t steps, int64_t B, int H, int D, int d, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -39,6 +39,16 @@ SIGNATURES = {
     "rfa_causal_forward": (c_int, [c_void_p] * 4 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "rfa_causal_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
     "rfa_causal_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "rfa_feature_map_supported": (c_int, [c_int, c_int]),
+    "rfa_feature_map_forward": (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int, c_int, c_float, c_void_p]),
+    "rfa_feature_map_backward_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int]),
+    "rfa_feature_map_backward": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p]),
+    "rfa_cross_state": (c_int, [c_void_p] * 5 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
+    "rfa_cross_readout": (c_int, [c_void_p] * 4 + [c_int64, c_int64, c_int, c_int, c_void_p]),
+    "rfa_cross_readout_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_void_p]),
+    "rfa_cross_state_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
+    "rfa_incremental": (c_int, [c_void_p] * 6 + [c_int64, c_int64, c_int, c_int, c_void_p]),
+    "rfa_incremental_fused": (c_int, [c_void_p] * 4 + [c_float] + [c_void_p] * 3 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
 }
 
 _lib = None

@@ -10,6 +10,8 @@
 #include <cstring>
 
 #include "rfa_causal.h"
+#include "rfa_decode.h"
+#include "rfa_featuremap.h"
 
 namespace {
 
@@ -100,9 +102,9 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
         auto kern = rfa::k_segment_state<KD, DH>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
         hipLaunchKernelGGL(kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
-                           k, v, wsS, wsZ, T, N, p.nseg, p.seg_len);
+                           k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
-    auto kern = rfa::k_causal_fwd<KD, DH>;
+    auto kern = rfa::k_causal_fwd<KD, DH, true>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
     hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kFwdLds, st, q, k, v, out,
                        wsS, wsZ, T, N, p.nseg, p.seg_len);
@@ -125,23 +127,156 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         auto kern = rfa::k_segment_state<KD, DH>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
         hipLaunchKernelGGL(kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
-                           k, v, wsS, wsZ, T, N, p.nseg, p.seg_len);
+                           k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     {
-        auto kern = rfa::k_causal_bwd_dq<KD, DH>;
+        auto kern = rfa::k_causal_bwd_dq<KD, DH, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDqLds)) return rc;
         hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDqLds, st, q, k, v, g,
                            dq, wsS, wsZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
     }
     {
-        auto kern = rfa::k_causal_bwd_dkdv<KD, DH>;
+        auto kern = rfa::k_causal_bwd_dkdv<KD, DH, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
         hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDkLds, st, q, k, v, g,
-                           dk, dv, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
+                           dk, dv, wsR, wsr, den, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
+
+// ---- cross attention launchers ---------------------------------------------------
+// time split for kernels whose workgroups do not depend on each other
+ScanPlan make_free_plan(int64_t T, int64_t N) {
+    ScanPlan p{1, rfa::kChunk};
+    if (T <= 0 || N <= 0) return p;
+    const int64_t nchunks = (T + rfa::kChunk - 1) / rfa::kChunk;
+    int64_t want = (512 + N - 1) / N;
+    if (want > nchunks) want = nchunks;
+    if (want < 1) want = 1;
+    const int64_t cps = (nchunks + want - 1) / want;
+    p.nseg = (int)((nchunks + cps - 1) / cps);
+    p.seg_len = (int)(cps * rfa::kChunk);
+    return p;
+}
+
+template <int KD, int DH>
+int launch_cross_state(const rfa::half_t* k, const rfa::half_t* v, const uint8_t* mask, int H, float* s,
+                       float* z, int T, int N, hipStream_t st) {
+    using Cfg = rfa::CausalCfg<KD, DH>;
+    const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
+    auto kern = rfa::k_segment_state<KD, DH>;
+    if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
+    hipLaunchKernelGGL(kern, dim3(N), dim3(rfa::kThreads), Cfg::kSegStateLds, st, k, v, mask, H, s, z, T, N,
+                       1, 1, seg_len);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+template <int KD, int DH>
+int launch_cross_readout(const rfa::half_t* q, const float* s, const float* z, rfa::half_t* out, int T, int N,
+                         hipStream_t st) {
+    using Cfg = rfa::CausalCfg<KD, DH>;
+    const ScanPlan p = make_free_plan(T, N);
+    auto kern = rfa::k_causal_fwd<KD, DH, false>;
+    if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
+    hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kFwdLds, st, q,
+                       (const rfa::half_t*)nullptr, (const rfa::half_t*)nullptr, out, s, z, T, N, p.nseg,
+                       p.seg_len);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+template <int KD, int DH>
+int launch_cross_readout_bwd(const rfa::half_t* q, const float* s, const float* z, const rfa::half_t* g,
+                             rfa::half_t* dq, float* ds, float* dz, int T, int N, hipStream_t st) {
+    using Cfg = rfa::CausalCfg<KD, DH>;
+    const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
+    auto kern = rfa::k_causal_bwd_dq<KD, DH, false>;
+    if (int rc = set_lds(kern, Cfg::kBwdDqLds)) return rc;
+    hipLaunchKernelGGL(kern, dim3(N), dim3(rfa::kThreads), Cfg::kBwdDqLds, st, q, (const rfa::half_t*)nullptr,
+                       (const rfa::half_t*)nullptr, g, dq, s, z, ds, dz, (float*)nullptr, (float*)nullptr, T, N,
+                       1, seg_len);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+template <int KD, int DH>
+int launch_cross_state_bwd(const rfa::half_t* k, const rfa::half_t* v, const uint8_t* mask, int H,
+                           const float* ds, const float* dz, rfa::half_t* dk, rfa::half_t* dv, int T, int N,
+                           hipStream_t st) {
+    using Cfg = rfa::CausalCfg<KD, DH>;
+    const ScanPlan p = make_free_plan(T, N);
+    auto kern = rfa::k_causal_bwd_dkdv<KD, DH, false>;
+    if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
+    hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDkLds, st,
+                       (const rfa::half_t*)nullptr, k, v, (const rfa::half_t*)nullptr, dk, dv, ds, dz,
+                       (const float*)nullptr, (const float*)nullptr, mask, H, T, N, p.nseg, p.seg_len);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+// ---- decode launchers --------------------------------------------------------------
+template <int KD, int DH, bool FUSED>
+int launch_decode(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, const rfa::half_t* w,
+                  float scale, int H, float* s, float* z, rfa::half_t* out, int64_t steps, int64_t N,
+                  hipStream_t st) {
+    const int64_t qk_step = FUSED ? N * DH : N * KD;
+    for (int64_t t = 0; t < steps; ++t) {
+        hipLaunchKernelGGL((rfa::k_decode_step<KD, DH, FUSED>), dim3((unsigned)N), dim3(rfa::kThreads), 0, st,
+                           q + t * qk_step, k + t * qk_step, v + t * N * DH, w, scale, H, s, z, s, z,
+                           out + t * N * DH);
+    }
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+// ---- feature map launchers ---------------------------------------------------------
+int feature_bwd_blocks(int64_t R, int H) {
+    const int64_t nrb = (R + 63) / 64;
+    int64_t nblk = (1024 + H - 1) / H;
+    if (nblk > nrb) nblk = nrb;
+    if (nblk < 1) nblk = 1;
+    return (int)nblk;
+}
+
+template <int D, int DH>
+int launch_feature_fwd(const rfa::half_t* x, const rfa::half_t* w, rfa::half_t* phi, int R, int H, float scale,
+                       hipStream_t st) {
+    using Cfg = rfa::FeatureCfg<D, DH>;
+    auto kern = rfa::k_feature_map_fwd<D, DH>;
+    if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
+    hipLaunchKernelGGL(kern, dim3((R + 63) / 64, H), dim3(rfa::kThreads), Cfg::kFwdLds, st, x, w, phi, R, H, scale);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+template <int D, int DH>
+int launch_feature_bwd(const rfa::half_t* x, const rfa::half_t* w, const rfa::half_t* gphi, rfa::half_t* dx,
+                       float* dw, float* part, int R, int H, float scale, hipStream_t st) {
+    using Cfg = rfa::FeatureCfg<D, DH>;
+    const int nblk = feature_bwd_blocks(R, H);
+    auto kern = rfa::k_feature_map_bwd<D, DH>;
+    if (int rc = set_lds(kern, Cfg::kBwdLds)) return rc;
+    hipLaunchKernelGGL(kern, dim3(nblk, H), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, part, R, H, scale);
+    const int64_t elems = (int64_t)H * D * DH;
+    hipLaunchKernelGGL(rfa::k_feature_map_dw_reduce, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, st,
+                       part, dw, nblk, elems);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+// zero fill by kernel (safe to record into a HIP graph, unlike a memset node)
+__global__ void k_zero_f32(float* p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+
+void zero_f32(float* p, int64_t n, hipStream_t st) {
+    if (n > 0) hipLaunchKernelGGL(k_zero_f32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, n);
+}
+
+bool feature_shape_supported(int D, int d) { return (D == 32 || D == 64 || D == 128) && (d == 64 || d == 128); }
 
 int check_causal_dims(int64_t T, int64_t N, int K, int d) {
     if (T < 0 || N < 0 || K <= 0 || d <= 0)
@@ -282,6 +417,215 @@ int rfa_causal_backward(const void* q, const void* k, const void* v, const void*
 #define RFA_CALL_BWD(KD, DH) launch_backward<KD, DH>(qh, kh, vh, gh, dqh, dkh, dvh, (int)T, (int)N, p, ws, wl, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_BWD)
 #undef RFA_CALL_BWD
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+// ---- cross attention ---------------------------------------------------------------
+static int check_cross_dims(const char* fn, int64_t L, int64_t B, int H, int K, int d) {
+    if (L < 0 || B < 0 || H <= 0 || K <= 0 || d <= 0)
+        return fail(RFA_ERR_BAD_SHAPE, "%s: bad sizes len=%lld B=%lld H=%d K=%d d=%d", fn, (long long)L, (long long)B, H, K, d);
+    if (!rfa_shape_supported(K, d))
+        return fail(RFA_ERR_UNSUPPORTED, "%s: no kernel for feature width K=%d, head dim d=%d", fn, K, d);
+    if (L > (1 << 30) || B * H > (1 << 22) || L * B * H > (int64_t(1) << 31))
+        return fail(RFA_ERR_BAD_SHAPE, "%s: sizes exceed the supported range", fn);
+    return RFA_OK;
+}
+
+int rfa_cross_state(const void* phi_k, const void* v, const uint8_t* key_padding_mask, float* s, float* z,
+                    int64_t S_len, int64_t B, int H, int K, int d, void* stream) {
+    if (int rc = check_cross_dims("rfa_cross_state", S_len, B, H, K, d)) return rc;
+    const int64_t N = B * H;
+    if (N == 0) return RFA_OK;
+    if (!s || !z) return fail(RFA_ERR_NULL_POINTER, "rfa_cross_state: NULL state pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (S_len == 0) {   // empty source: the state is zero
+        zero_f32(s, (int64_t)N * K * d, st);
+        zero_f32(z, (int64_t)N * K, st);
+        return RFA_OK;
+    }
+    if (!phi_k || !v) return fail(RFA_ERR_NULL_POINTER, "rfa_cross_state: NULL tensor pointer");
+    if (!aligned16(phi_k) || !aligned16(v) || !aligned16(s) || !aligned16(z))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_cross_state: tensors must be 16-byte aligned");
+    auto* kh = static_cast<const rfa::half_t*>(phi_k);
+    auto* vh = static_cast<const rfa::half_t*>(v);
+#define RFA_CALL(KD, DH) launch_cross_state<KD, DH>(kh, vh, key_padding_mask, H, s, z, (int)S_len, (int)N, st)
+    RFA_DISPATCH_KD(K, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+int rfa_cross_readout(const void* phi_q, const float* s, const float* z, void* out, int64_t T, int64_t N,
+                      int K, int d, void* stream) {
+    if (int rc = check_cross_dims("rfa_cross_readout", T, N, 1, K, d)) return rc;
+    if (T == 0 || N == 0) return RFA_OK;
+    if (!phi_q || !s || !z || !out) return fail(RFA_ERR_NULL_POINTER, "rfa_cross_readout: NULL tensor pointer");
+    if (!aligned16(phi_q) || !aligned16(s) || !aligned16(z) || !aligned16(out))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_cross_readout: tensors must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* qh = static_cast<const rfa::half_t*>(phi_q);
+    auto* oh = static_cast<rfa::half_t*>(out);
+#define RFA_CALL(KD, DH) launch_cross_readout<KD, DH>(qh, s, z, oh, (int)T, (int)N, st)
+    RFA_DISPATCH_KD(K, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+int rfa_cross_readout_backward(const void* phi_q, const float* s, const float* z, const void* grad_attn,
+                               void* dphi_q, float* ds, float* dz, int64_t T, int64_t N, int K, int d,
+                               void* stream) {
+    if (int rc = check_cross_dims("rfa_cross_readout_backward", T, N, 1, K, d)) return rc;
+    if (N == 0) return RFA_OK;
+    if (!ds || !dz) return fail(RFA_ERR_NULL_POINTER, "rfa_cross_readout_backward: NULL gradient pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (T == 0) {
+        zero_f32(ds, (int64_t)N * K * d, st);
+        zero_f32(dz, (int64_t)N * K, st);
+        return RFA_OK;
+    }
+    if (!phi_q || !s || !z || !grad_attn || !dphi_q)
+        return fail(RFA_ERR_NULL_POINTER, "rfa_cross_readout_backward: NULL tensor pointer");
+    if (!aligned16(phi_q) || !aligned16(s) || !aligned16(z) || !aligned16(grad_attn) || !aligned16(dphi_q) ||
+        !aligned16(ds) || !aligned16(dz))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_cross_readout_backward: tensors must be 16-byte aligned");
+    auto* qh = static_cast<const rfa::half_t*>(phi_q);
+    auto* gh = static_cast<const rfa::half_t*>(grad_attn);
+    auto* dqh = static_cast<rfa::half_t*>(dphi_q);
+#define RFA_CALL(KD, DH) launch_cross_readout_bwd<KD, DH>(qh, s, z, gh, dqh, ds, dz, (int)T, (int)N, st)
+    RFA_DISPATCH_KD(K, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+int rfa_cross_state_backward(const void* phi_k, const void* v, const uint8_t* key_padding_mask, const float* ds,
+                             const float* dz, void* dphi_k, void* dv, int64_t S_len, int64_t B, int H, int K,
+                             int d, void* stream) {
+    if (int rc = check_cross_dims("rfa_cross_state_backward", S_len, B, H, K, d)) return rc;
+    const int64_t N = B * H;
+    if (S_len == 0 || N == 0) return RFA_OK;
+    if (!phi_k || !v || !ds || !dz || !dphi_k || !dv)
+        return fail(RFA_ERR_NULL_POINTER, "rfa_cross_state_backward: NULL tensor pointer");
+    if (!aligned16(phi_k) || !aligned16(v) || !aligned16(ds) || !aligned16(dz) || !aligned16(dphi_k) || !aligned16(dv))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_cross_state_backward: tensors must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* kh = static_cast<const rfa::half_t*>(phi_k);
+    auto* vh = static_cast<const rfa::half_t*>(v);
+    auto* dkh = static_cast<rfa::half_t*>(dphi_k);
+    auto* dvh = static_cast<rfa::half_t*>(dv);
+#define RFA_CALL(KD, DH) launch_cross_state_bwd<KD, DH>(kh, vh, key_padding_mask, H, ds, dz, dkh, dvh, (int)S_len, (int)N, st)
+    RFA_DISPATCH_KD(K, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+// ---- incremental decoding -----------------------------------------------------------
+int rfa_incremental(const void* phi_q, const void* phi_k, const void* v, float* s, float* z, void* out,
+                    int64_t steps, int64_t N, int K, int d, void* stream) {
+    if (int rc = check_cross_dims("rfa_incremental", steps, N, 1, K, d)) return rc;
+    if (steps == 0 || N == 0) return RFA_OK;
+    if (!phi_q || !phi_k || !v || !s || !z || !out) return fail(RFA_ERR_NULL_POINTER, "rfa_incremental: NULL tensor pointer");
+    if (!aligned16(phi_q) || !aligned16(phi_k) || !aligned16(v) || !aligned16(s) || !aligned16(z) || !aligned16(out))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_incremental: tensors must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* qh = static_cast<const rfa::half_t*>(phi_q);
+    auto* kh = static_cast<const rfa::half_t*>(phi_k);
+    auto* vh = static_cast<const rfa::half_t*>(v);
+    auto* oh = static_cast<rfa::half_t*>(out);
+#define RFA_CALL(KD, DH) launch_decode<KD, DH, false>(qh, kh, vh, nullptr, 0.f, 1, s, z, oh, steps, N, st)
+    RFA_DISPATCH_KD(K, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+int rfa_incremental_fused(const void* q, const void* k, const void* v, const void* w, float scale, float* s,
+                          float* z, void* out, int64_t steps, int64_t B, int H, int D, int d, void* stream) {
+    if (int rc = check_cross_dims("rfa_incremental_fused", steps, B, H, 2 * D, d)) return rc;
+    const int64_t N = B * H;
+    if (steps == 0 || N == 0) return RFA_OK;
+    if (!q || !k || !v || !w || !s || !z || !out)
+        return fail(RFA_ERR_NULL_POINTER, "rfa_incremental_fused: NULL tensor pointer");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(s) || !aligned16(z) || !aligned16(out))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_incremental_fused: tensors must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* qh = static_cast<const rfa::half_t*>(q);
+    auto* kh = static_cast<const rfa::half_t*>(k);
+    auto* vh = static_cast<const rfa::half_t*>(v);
+    auto* wh = static_cast<const rfa::half_t*>(w);
+    auto* oh = static_cast<rfa::half_t*>(out);
+    const int K = 2 * D;
+#define RFA_CALL(KD, DH) launch_decode<KD, DH, true>(qh, kh, vh, wh, scale, H, s, z, oh, steps, N, st)
+    RFA_DISPATCH_KD(K, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+// ---- feature map --------------------------------------------------------------------
+int rfa_feature_map_supported(int D, int d) { return feature_shape_supported(D, d) ? 1 : 0; }
+
+static int check_feature_dims(const char* fn, int64_t R, int H, int D, int d) {
+    if (R < 0 || H <= 0 || D <= 0 || d <= 0)
+        return fail(RFA_ERR_BAD_SHAPE, "%s: bad sizes rows=%lld H=%d D=%d d=%d", fn, (long long)R, H, D, d);
+    if (!feature_shape_supported(D, d))
+        return fail(RFA_ERR_UNSUPPORTED, "%s: no kernel for proj_dim D=%d, head dim d=%d (supported: D in {32,64,128}, d in {64,128})", fn, D, d);
+    if (R * H > (int64_t(1) << 31) || R > (int64_t(1) << 30) || H > 65535)
+        return fail(RFA_ERR_BAD_SHAPE, "%s: sizes exceed the supported range", fn);
+    return RFA_OK;
+}
+
+#define RFA_DISPATCH_FEATURE(D, d, CALL)                  \
+    if (D == 32 && d == 64) { return CALL(32, 64); }      \
+    if (D == 64 && d == 64) { return CALL(64, 64); }      \
+    if (D == 128 && d == 64) { return CALL(128, 64); }    \
+    if (D == 32 && d == 128) { return CALL(32, 128); }    \
+    if (D == 64 && d == 128) { return CALL(64, 128); }    \
+    if (D == 128 && d == 128) { return CALL(128, 128); }
+
+int rfa_feature_map_forward(const void* x, const void* w, void* phi, int64_t R, int H, int D, int d, float scale,
+                            void* stream) {
+    if (int rc = check_feature_dims("rfa_feature_map_forward", R, H, D, d)) return rc;
+    if (R == 0) return RFA_OK;
+    if (!x || !w || !phi) return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_forward: NULL tensor pointer");
+    if (!aligned16(x) || !aligned16(w) || !aligned16(phi))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_feature_map_forward: tensors must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* xh = static_cast<const rfa::half_t*>(x);
+    auto* wh = static_cast<const rfa::half_t*>(w);
+    auto* ph = static_cast<rfa::half_t*>(phi);
+#define RFA_CALL(DD, DH) launch_feature_fwd<DD, DH>(xh, wh, ph, (int)R, H, scale, st)
+    RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+size_t rfa_feature_map_backward_workspace_bytes(int64_t R, int H, int D, int d) {
+    if (R <= 0 || H <= 0 || !feature_shape_supported(D, d)) return 0;
+    return (size_t)feature_bwd_blocks(R, H) * H * D * d * 4;
+}
+
+int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi, void* dx, float* dw, int64_t R,
+                             int H, int D, int d, float scale, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+    if (int rc = check_feature_dims("rfa_feature_map_backward", R, H, D, d)) return rc;
+    if (!dw) return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward: NULL dw");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (R == 0) {
+        zero_f32(dw, (int64_t)H * D * d, st);
+        return RFA_OK;
+    }
+    if (!x || !w || !grad_phi || !dx) return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward: NULL tensor pointer");
+    if (!aligned16(x) || !aligned16(w) || !aligned16(grad_phi) || !aligned16(dx) || !aligned16(dw))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_feature_map_backward: tensors must be 16-byte aligned");
+    const size_t need = rfa_feature_map_backward_workspace_bytes(R, H, D, d);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+        return fail(RFA_ERR_WORKSPACE, "rfa_feature_map_backward: workspace of %zu bytes required, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    auto* xh = static_cast<const rfa::half_t*>(x);
+    auto* wh = static_cast<const rfa::half_t*>(w);
+    auto* gh = static_cast<const rfa::half_t*>(grad_phi);
+    auto* dxh = static_cast<rfa::half_t*>(dx);
+    float* part = static_cast<float*>(workspace);
+#define RFA_CALL(DD, DH) launch_feature_bwd<DD, DH>(xh, wh, gh, dxh, dw, part, (int)R, H, scale, st)
+    RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
+#undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
 }
 

@@ -50,12 +50,17 @@ struct CausalCfg {
 
 // ---------------------------------------------------------------------------
 // pass 0: per-segment totals  dS = K^T V (KD x DH),  dz = K^T 1
-// grid = N * (nseg - 1): the last segment's total is never consumed.
+// grid = N * nseg_out: the causal passes compute nseg_out = nseg - 1 totals per
+// sequence (the last segment's total is never consumed); cross attention computes
+// the single total of the whole source (nseg = nseg_out = 1) straight into its
+// state tensors.  pad_mask ([B, T] bytes, 1 = padded key, may be NULL) zeroes
+// phi_k rows (reference: cross_attention.py:97-100).
 // ---------------------------------------------------------------------------
 template <int KD, int DH>
 __global__ __launch_bounds__(kThreads) void k_segment_state(
-    const half_t* __restrict__ k, const half_t* __restrict__ v, float* __restrict__ wsS,
-    float* __restrict__ wsZ, int T, int N, int nseg, int seg_len) {
+    const half_t* __restrict__ k, const half_t* __restrict__ v, const uint8_t* __restrict__ pad_mask,
+    int H, float* __restrict__ wsS, float* __restrict__ wsZ, int T, int N, int nseg, int nseg_out,
+    int seg_len) {
     using Cfg = CausalCfg<KD, DH>;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, DS = Cfg::DS;
     constexpr int NKT = KD / 16, NCT = DS / 16;
@@ -66,7 +71,8 @@ __global__ __launch_bounds__(kThreads) void k_segment_state(
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
-    const int n = blockIdx.x / (nseg - 1), seg = blockIdx.x % (nseg - 1);
+    const int n = blockIdx.x / nseg_out, seg = blockIdx.x % nseg_out;
+    const uint8_t* mrow = pad_mask ? pad_mask + (int64_t)(n / H) * T : nullptr;
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
@@ -84,6 +90,7 @@ __global__ __launch_bounds__(kThreads) void k_segment_state(
     ChunkRegs<DH> rv;
     chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
     chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
+    if (mrow) chunk_mask_rows<KD>(rk, mrow + t_begin, t_end - t_begin, tid);
     for (int t0 = t_begin; t0 < t_end; t0 += C) {
         chunk_r2s<KD>(rk, Ks, LDQ, tid);
         chunk_r2s<DH>(rv, Vs, LDV, tid);
@@ -91,6 +98,7 @@ __global__ __launch_bounds__(kThreads) void k_segment_state(
         if (t0 + C < t_end) {
             chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, t_end - t0 - C, tid);
             chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, t_end - t0 - C, tid);
+            if (mrow) chunk_mask_rows<KD>(rk, mrow + t0 + C, t_end - t0 - C, tid);
         }
         h8 bv[NCT][2];
 #pragma unroll
@@ -128,7 +136,12 @@ __global__ __launch_bounds__(kThreads) void k_segment_state(
 // forward scan.  Wave w owns value columns [w*DS, (w+1)*DS) of S (all KD rows),
 // held as accumulator tiles S[kt][ct] with element (k = 16kt+4G+e, c = w*DS+16ct+i).
 // ---------------------------------------------------------------------------
-template <int KD, int DH>
+//
+// CAUSAL = false is the cross-attention readout (reference: cross_attention.py:266-269):
+// the state is the fixed total S, z of the source (wsS/wsZ hold one state per
+// sequence), there is no intra-chunk term and no update, and the denominator is
+// max(|q.z|, 1); k and v are not read.
+template <int KD, int DH, bool CAUSAL>
 __global__ __launch_bounds__(kThreads) void k_causal_fwd(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ, int T,
@@ -163,8 +176,10 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
 #pragma unroll
         for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
     float zreg = 0.f;
-    for (int s = 0; s < seg; ++s) {
-        const float* si = wsS + ((int64_t)(n * nseg + s) * KD) * DH;
+    const int n_states = CAUSAL ? seg : 1;          // states to sum
+    const int state_stride = CAUSAL ? nseg : 1;     // states stored per sequence
+    for (int s = 0; s < n_states; ++s) {
+        const float* si = wsS + ((int64_t)(n * state_stride + s) * KD) * DH;
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
@@ -172,26 +187,32 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     S[kt][ct][e] += si[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row];
-        if (tid < KD) zreg += wsZ[(int64_t)(n * nseg + s) * KD + tid];
+        if (tid < KD) zreg += wsZ[(int64_t)(n * state_stride + s) * KD + tid];
     }
 
     ChunkRegs<KD> rq, rk;
     ChunkRegs<DH> rv;
     chunk_g2r<KD>(rq, qb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
-    chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
-    chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
+    if (CAUSAL) {
+        chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
+        chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
+    }
 
     for (int t0 = t_begin; t0 < t_end; t0 += C) {
         chunk_r2s<KD>(rq, Qs, LDQ, tid);
-        chunk_r2s<KD>(rk, Ks, LDQ, tid);
-        chunk_r2s<DH>(rv, Vs, LDV, tid);
+        if (CAUSAL) {
+            chunk_r2s<KD>(rk, Ks, LDQ, tid);
+            chunk_r2s<DH>(rv, Vs, LDV, tid);
+        }
         if (tid < KD) zs[tid] = zreg;
         __syncthreads();
         if (t0 + C < t_end) {
             const int rows = t_end - t0 - C;
             chunk_g2r<KD>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-            chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-            chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+            if (CAUSAL) {
+                chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+                chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+            }
         }
 
         // ---- phase A: wave w computes rows i in [16w, 16w+16) of A (as A^T tiles, m=j, n=i)
@@ -200,7 +221,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) at[jt] = f4_zero();
 #pragma unroll
-            for (int ks = 0; ks < KD / 32; ++ks) {
+            for (int ks = 0; ks < (CAUSAL ? KD / 32 : 0); ++ks) {
                 h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt)
@@ -229,11 +250,13 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
                 }
             }
             part = sum_over_groups(part);
-            if (G == 0) dens[16 * w + row] = fmaxf(part, 1.0f);
+            if (G == 0) dens[16 * w + row] = fmaxf(CAUSAL ? part : fabsf(part), 1.0f);
+            if (CAUSAL) {
 #pragma unroll
-            for (int jt = 0; jt < 4; ++jt) {
-                h4 hv = (jt <= w) ? to_h4(at[jt]) : h4_zero();
-                *reinterpret_cast<h4*>(As + (16 * w + row) * LDA + 16 * jt + 4 * G) = hv;
+                for (int jt = 0; jt < 4; ++jt) {
+                    h4 hv = (jt <= w) ? to_h4(at[jt]) : h4_zero();
+                    *reinterpret_cast<h4*>(As + (16 * w + row) * LDA + 16 * jt + 4 * G) = hv;
+                }
             }
         }
         __syncthreads();
@@ -241,10 +264,12 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
         // ---- phase B: out^T tiles (m=c, n=i) for this wave's value columns, then state update
         {
             h8 av[NCT][2];   // V column fragments: element V[j = 32js+8G+e][c = w*DS+16ct+i]
+            if (CAUSAL) {
 #pragma unroll
-            for (int ct = 0; ct < NCT; ++ct)
+                for (int ct = 0; ct < NCT; ++ct)
 #pragma unroll
-                for (int js = 0; js < 2; ++js) av[ct][js] = col8(Vs, LDV, js * 32, w * DS + 16 * ct, lane);
+                    for (int js = 0; js < 2; ++js) av[ct][js] = col8(Vs, LDV, js * 32, w * DS + 16 * ct, lane);
+            }
 
             f4 acc[4][NCT];
 #pragma unroll
@@ -252,7 +277,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
 #pragma unroll
                 for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = f4_zero();
 #pragma unroll
-                for (int js = 0; js < 2; ++js) {
+                for (int js = 0; js < (CAUSAL ? 2 : 0); ++js) {
                     if (js == 0 || it >= 2) {
                         h8 ba = row8(As, LDA, 16 * it + row, js * 32, G);
 #pragma unroll
@@ -288,20 +313,22 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
                     }
                 }
             }
-            // S (m=k, n=c) += K^T V
+            if (CAUSAL) {
+                // S (m=k, n=c) += K^T V
 #pragma unroll
-            for (int kt = 0; kt < NKT; ++kt)
+                for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-                for (int js = 0; js < 2; ++js) {
-                    h8 ak = col8(Ks, LDQ, js * 32, 16 * kt, lane);
+                    for (int js = 0; js < 2; ++js) {
+                        h8 ak = col8(Ks, LDQ, js * 32, 16 * kt, lane);
 #pragma unroll
-                    for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, av[ct][js], S[kt][ct]);
-                }
-            if (tid < KD) {
-                float s = 0.f;
+                        for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, av[ct][js], S[kt][ct]);
+                    }
+                if (tid < KD) {
+                    float s = 0.f;
 #pragma unroll 8
-                for (int j = 0; j < C; ++j) s += (float)Ks[j * LDQ + tid];
-                zreg += s;
+                    for (int j = 0; j < C; ++j) s += (float)Ks[j * LDQ + tid];
+                    zreg += s;
+                }
             }
         }
         __syncthreads();
@@ -313,7 +340,13 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
 // dR = Q^T (G/den), dr = Q^T gz.  Wave w owns feature rows [w*KS, (w+1)*KS):
 // ST[ct][kt] / RT[ct][kt] hold element (c = 16ct+4G+e, k = w*KS+16kt+i).
 // ---------------------------------------------------------------------------
-template <int KD, int DH>
+//
+// CAUSAL = false is the backward of the cross-attention readout: the state is the
+// fixed source total (one per sequence in wsS/wsZ), den = max(|q.z|, 1),
+// gz = -e/den^2 * sign(q.z) * [|q.z| > 1], dQ = Y/den + gz z^T, and the totals
+// dR, dr written to wsR/wsr (one per sequence, nseg must be 1) are the gradients
+// of the state (dS, dz).  k and v are not read; den_ws/gz_ws are not written.
+template <int KD, int DH, bool CAUSAL>
 __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, half_t* __restrict__ dq, const float* __restrict__ wsS,
@@ -354,8 +387,10 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
 #pragma unroll
         for (int b = 0; b < NKT; ++b) { ST[a][b] = f4_zero(); RT[a][b] = f4_zero(); }
     float zreg = 0.f, rreg = 0.f;
-    for (int s = 0; s < seg; ++s) {
-        const float* si = wsS + ((int64_t)(n * nseg + s) * KD) * DH;
+    const int n_states = CAUSAL ? seg : 1;
+    const int state_stride = CAUSAL ? nseg : 1;
+    for (int s = 0; s < n_states; ++s) {
+        const float* si = wsS + ((int64_t)(n * state_stride + s) * KD) * DH;
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct)
 #pragma unroll
@@ -363,7 +398,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
                 f4 x = *reinterpret_cast<const f4*>(si + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
                 ST[ct][kt] += x;
             }
-        if (tid < KD) zreg += wsZ[(int64_t)(n * nseg + s) * KD + tid];
+        if (tid < KD) zreg += wsZ[(int64_t)(n * state_stride + s) * KD + tid];
     }
 
     ChunkRegs<KD> rq, rk;
@@ -371,24 +406,30 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
     {
         const int rows = t_end - t_begin;
         chunk_g2r<KD>(rq, qb + (int64_t)t_begin * k_stride, k_stride, rows, tid);
-        chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, rows, tid);
-        chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, rows, tid);
         chunk_g2r<DH>(rg, gb + (int64_t)t_begin * v_stride, v_stride, rows, tid);
+        if (CAUSAL) {
+            chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, rows, tid);
+            chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, rows, tid);
+        }
     }
 
     for (int t0 = t_begin; t0 < t_end; t0 += C) {
         chunk_r2s<KD>(rq, Qs, LDQ, tid);
-        chunk_r2s<KD>(rk, Ks, LDQ, tid);
-        chunk_r2s<DH>(rv, Vs, LDV, tid);
         chunk_r2s<DH>(rg, Gs, LDV, tid);
+        if (CAUSAL) {
+            chunk_r2s<KD>(rk, Ks, LDQ, tid);
+            chunk_r2s<DH>(rv, Vs, LDV, tid);
+        }
         if (tid < KD) zs[tid] = zreg;
         __syncthreads();
         if (t0 + C < t_end) {
             const int rows = t_end - t0 - C;
             chunk_g2r<KD>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-            chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-            chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
             chunk_g2r<DH>(rg, gb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+            if (CAUSAL) {
+                chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+                chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+            }
         }
 
         // ---- phase A
@@ -399,14 +440,14 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) { at[jt] = f4_zero(); xt[jt] = f4_zero(); }
 #pragma unroll
-            for (int ks = 0; ks < KD / 32; ++ks) {
+            for (int ks = 0; ks < (CAUSAL ? KD / 32 : 0); ++ks) {
                 h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt)
                     if (jt <= w) at[jt] = mfma32(row8(Ks, LDQ, 16 * jt + row, ks * 32, G), bq, at[jt]);
             }
 #pragma unroll
-            for (int cs = 0; cs < DH / 32; ++cs) {
+            for (int cs = 0; cs < (CAUSAL ? DH / 32 : 0); ++cs) {
                 h8 bg = row8(Gs, LDV, 16 * w + row, cs * 32, G);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt)
@@ -485,12 +526,17 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
         // ---- phase B: denominators and d(qz) for the 64 rows of the chunk
         if (tid < C) {
             const float dr = drs[tid];
-            const float den = fmaxf(dr, 1.0f);
+            const float den = fmaxf(CAUSAL ? dr : fabsf(dr), 1.0f);
             const float e = e1s[tid] + ((e2p[tid] + e2p[C + tid]) + (e2p[2 * C + tid] + e2p[3 * C + tid]));
-            const float gz = (dr > 1.0f) ? -e / (den * den) : 0.f;
+            float gz;
+            if (CAUSAL) {
+                gz = (dr > 1.0f) ? -e / (den * den) : 0.f;
+            } else {
+                gz = (fabsf(dr) > 1.0f) ? (dr > 0.f ? -e : e) / (den * den) : 0.f;
+            }
             dens[tid] = den;
             gzs[tid] = gz;
-            if (t0 + tid < t_end) {
+            if (CAUSAL && t0 + tid < t_end) {
                 den_ws[(int64_t)(t0 + tid) * N + n] = den;
                 gz_ws[(int64_t)(t0 + tid) * N + n] = gz;
             }
@@ -503,7 +549,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
             const float inv = 1.0f / dens[i];
             const float gzi = gzs[i];
 #pragma unroll
-            for (int jt = 0; jt < 4; ++jt) {
+            for (int jt = 0; jt < (CAUSAL ? 4 : 0); ++jt) {
                 h4 pv = h4_zero();
                 if (jt <= w) {
 #pragma unroll
@@ -531,25 +577,32 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
         // ---- phase D: dQ^T tiles (m=k, n=i), then the carried sums
         {
             h8 kf[NKT][2];   // K column fragments: K[j = 32js+8G+e][k = w*KS+16kt+i]
+            if (CAUSAL) {
 #pragma unroll
-            for (int kt = 0; kt < NKT; ++kt)
+                for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-                for (int js = 0; js < 2; ++js) kf[kt][js] = col8(Ks, LDQ, js * 32, w * KS + 16 * kt, lane);
+                    for (int js = 0; js < 2; ++js) kf[kt][js] = col8(Ks, LDQ, js * 32, w * KS + 16 * kt, lane);
+            }
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const int i = 16 * it + row;
                 const float inv = 1.0f / dens[i];
                 const float gzi = gzs[i];
-                h8 bp0 = row8(Ps, LDA, i, 0, G);
-                h8 bp1 = row8(Ps, LDA, i, 32, G);
+                h8 bp0, bp1;
+                if (CAUSAL) {
+                    bp0 = row8(Ps, LDA, i, 0, G);
+                    bp1 = row8(Ps, LDA, i, 32, G);
+                }
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt) {
                     f4 zv = *reinterpret_cast<const f4*>(zs + w * KS + 16 * kt + 4 * G);
                     f4 acc;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) acc[e] = yt[kt][it][e] * inv + gzi * zv[e];
-                    acc = mfma32(kf[kt][0], bp0, acc);
-                    if (it >= 2) acc = mfma32(kf[kt][1], bp1, acc);
+                    if (CAUSAL) {
+                        acc = mfma32(kf[kt][0], bp0, acc);
+                        if (it >= 2) acc = mfma32(kf[kt][1], bp1, acc);
+                    }
                     if (t0 + i < t_end)
                         *reinterpret_cast<h4*>(dqb + (int64_t)(t0 + i) * k_stride + w * KS + 16 * kt + 4 * G) = to_h4(acc);
                 }
@@ -562,11 +615,12 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
 #pragma unroll
                 for (int ct = 0; ct < NCT; ++ct) {
                     h8 gf = col8(Gs, LDV, js * 32, 16 * ct, lane);
-                    h8 vf = col8(Vs, LDV, js * 32, 16 * ct, lane);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) {
-                        RT[ct][kt] = mfma32(gf, qf[kt], RT[ct][kt]);
-                        ST[ct][kt] = mfma32(vf, kf[kt][js], ST[ct][kt]);
+                    for (int kt = 0; kt < NKT; ++kt) RT[ct][kt] = mfma32(gf, qf[kt], RT[ct][kt]);
+                    if (CAUSAL) {
+                        h8 vf = col8(Vs, LDV, js * 32, 16 * ct, lane);
+#pragma unroll
+                        for (int kt = 0; kt < NKT; ++kt) ST[ct][kt] = mfma32(vf, kf[kt][js], ST[ct][kt]);
                     }
                 }
             }
@@ -574,7 +628,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
                 float sz = 0.f, sr = 0.f;
 #pragma unroll 8
                 for (int j = 0; j < C; ++j) {
-                    sz += (float)Ks[j * LDQ + tid];
+                    if (CAUSAL) sz += (float)Ks[j * LDQ + tid];
                     sr += (float)Qs[j * LDQ + tid] * gzs[j];
                 }
                 zreg += sz;
@@ -584,7 +638,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
         __syncthreads();
     }
 
-    if (seg > 0) {   // totals of segment 0 are never consumed
+    if (!CAUSAL || seg > 0) {   // causal: totals of segment 0 are never consumed
         float* ro = wsR + ((int64_t)(n * nseg + seg) * KD) * DH;
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct)
@@ -600,12 +654,19 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
 // contraction: RT[ct][kt] (c = 16ct+4G+e, k = w*KS+16kt+i) contracts over c for
 // dK; RR[kt][ct] (k = 16kt+4G+e, c = w*DS+16ct+i) contracts over k for dV.
 // ---------------------------------------------------------------------------
-template <int KD, int DH>
+//
+// CAUSAL = false is the backward of the cross-attention state: R, r are the fixed
+// gradients dS, dz (one per sequence in wsR/wsr), dK = V dS^T + 1 dz^T,
+// dV = K dS; q, g, den_ws, gz_ws are not read.  pad_mask ([B, T] bytes, may be
+// NULL; H heads per batch entry) marks padded keys: their phi_k rows are read as
+// zero and their dK rows are written as zero (the gradient of masked_fill).
+template <int KD, int DH, bool CAUSAL>
 __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, half_t* __restrict__ dk, half_t* __restrict__ dv,
     const float* __restrict__ wsR, const float* __restrict__ wsr, const float* __restrict__ den_ws,
-    const float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len) {
+    const float* __restrict__ gz_ws, const uint8_t* __restrict__ pad_mask, int H, int T, int N,
+    int nseg, int seg_len) {
     using Cfg = CausalCfg<KD, DH>;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS, DS = Cfg::DS;
     constexpr int NKT = KS / 16, NCT = DH / 16;      // RT tiles
@@ -644,8 +705,11 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
 #pragma unroll
         for (int b = 0; b < NCT2; ++b) RR[a][b] = f4_zero();
     float rreg = 0.f;
-    for (int s = seg + 1; s < nseg; ++s) {
-        const float* ri = wsR + ((int64_t)(n * nseg + s) * KD) * DH;
+    const uint8_t* mrow = (!CAUSAL && pad_mask) ? pad_mask + (int64_t)(n / H) * T : nullptr;
+    const int s_first = CAUSAL ? seg + 1 : 0, s_last = CAUSAL ? nseg : 1;
+    const int state_stride = CAUSAL ? nseg : 1;
+    for (int s = s_first; s < s_last; ++s) {
+        const float* ri = wsR + ((int64_t)(n * state_stride + s) * KD) * DH;
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct)
 #pragma unroll
@@ -658,7 +722,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     RR[kt][ct][e] += ri[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row];
-        if (tid < KD) rreg += wsr[(int64_t)(n * nseg + s) * KD + tid];
+        if (tid < KD) rreg += wsr[(int64_t)(n * state_stride + s) * KD + tid];
     }
 
     ChunkRegs<KD> rq, rk;
@@ -668,33 +732,39 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
     constexpr int PPRV = DH / 8;
     auto prefetch = [&](int t0) {
         const int rows = t_end - t0;
-        chunk_g2r<KD>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
         chunk_g2r<KD>(rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
         chunk_g2r<DH>(rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
-        chunk_g2r<DH>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+        if (CAUSAL) {
+            chunk_g2r<KD>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+            chunk_g2r<DH>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
 #pragma unroll
-        for (int it = 0; it < ChunkRegs<DH>::kPieces; ++it) {
-            const int r_ = (tid + kThreads * it) / PPRV;
-            inv_den[it] = (r_ < rows) ? 1.0f / den_ws[(int64_t)(t0 + r_) * N + n] : 0.f;
+            for (int it = 0; it < ChunkRegs<DH>::kPieces; ++it) {
+                const int r_ = (tid + kThreads * it) / PPRV;
+                inv_den[it] = (r_ < rows) ? 1.0f / den_ws[(int64_t)(t0 + r_) * N + n] : 0.f;
+            }
+            gz_next = (tid < C && tid < rows) ? gz_ws[(int64_t)(t0 + tid) * N + n] : 0.f;
+        } else if (mrow) {
+            chunk_mask_rows<KD>(rk, mrow + t0, rows, tid);
         }
-        gz_next = (tid < C && tid < rows) ? gz_ws[(int64_t)(t0 + tid) * N + n] : 0.f;
     };
 
     const int n_chunks = (t_end - t_begin + C - 1) / C;
     prefetch(t_begin + (n_chunks - 1) * C);
     for (int ci = n_chunks - 1; ci >= 0; --ci) {
         const int t0 = t_begin + ci * C;
-        chunk_r2s<KD>(rq, Qs, LDQ, tid);
         chunk_r2s<KD>(rk, Ks, LDQ, tid);
         chunk_r2s<DH>(rv, Vs, LDV, tid);
-        chunk_r2s_scaled<DH>(rg, inv_den, Gs, LDV, tid);
-        if (tid < C) gzs[tid] = gz_next;
+        if (CAUSAL) {
+            chunk_r2s<KD>(rq, Qs, LDQ, tid);
+            chunk_r2s_scaled<DH>(rg, inv_den, Gs, LDV, tid);
+            if (tid < C) gzs[tid] = gz_next;
+        }
         if (tid < KD) rs[tid] = rreg;
         __syncthreads();
         if (ci > 0) prefetch(t0 - C);
 
         // ---- phase A: wave w computes columns j in [16w, 16w+16) of A and P (tiles m=i, n=j)
-        {
+        if (CAUSAL) {
             f4 a_[4], p_[4];
 #pragma unroll
             for (int it = 0; it < 4; ++it) { a_[it] = f4_zero(); p_[it] = f4_zero(); }
@@ -731,20 +801,22 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
                 *reinterpret_cast<h4*>(PTs + j * LDA + 16 * it + 4 * G) = pv;
             }
         }
-        __syncthreads();
+        if (CAUSAL) __syncthreads();
 
         // ---- phase B
         {
             h8 qf[NKT][2];    // Q column fragments for this wave's feature slice
-#pragma unroll
-            for (int kt = 0; kt < NKT; ++kt)
-#pragma unroll
-                for (int is = 0; is < 2; ++is) qf[kt][is] = col8(Qs, LDQ, is * 32, w * KS + 16 * kt, lane);
             h8 gf2[NCT2][2];  // (G/den) column fragments for this wave's value slice
+            if (CAUSAL) {
 #pragma unroll
-            for (int ct = 0; ct < NCT2; ++ct)
+                for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-                for (int is = 0; is < 2; ++is) gf2[ct][is] = col8(Gs, LDV, is * 32, w * DS + 16 * ct, lane);
+                    for (int is = 0; is < 2; ++is) qf[kt][is] = col8(Qs, LDQ, is * 32, w * KS + 16 * kt, lane);
+#pragma unroll
+                for (int ct = 0; ct < NCT2; ++ct)
+#pragma unroll
+                    for (int is = 0; is < 2; ++is) gf2[ct][is] = col8(Gs, LDV, is * 32, w * DS + 16 * ct, lane);
+            }
 
             // dK^T tiles (m=k, n=j)
             f4 dkacc[NKT][4];
@@ -754,8 +826,10 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
                     f4 acc = rv4;
-                    if (jt < 2) acc = mfma32(qf[kt][0], row8(PTs, LDA, 16 * jt + row, 0, G), acc);
-                    acc = mfma32(qf[kt][1], row8(PTs, LDA, 16 * jt + row, 32, G), acc);
+                    if (CAUSAL) {
+                        if (jt < 2) acc = mfma32(qf[kt][0], row8(PTs, LDA, 16 * jt + row, 0, G), acc);
+                        acc = mfma32(qf[kt][1], row8(PTs, LDA, 16 * jt + row, 32, G), acc);
+                    }
                     dkacc[kt][jt] = acc;
                 }
             }
@@ -778,9 +852,11 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
             for (int jt = 0; jt < 4; ++jt) {
                 const int jj = 16 * jt + row;
                 if (t0 + jj < t_end) {
+                    const bool padded = mrow && mrow[t0 + jj];
 #pragma unroll
                     for (int kt = 0; kt < NKT; ++kt)
-                        *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + w * KS + 16 * kt + 4 * G) = to_h4(dkacc[kt][jt]);
+                        *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + w * KS + 16 * kt + 4 * G) =
+                            padded ? h4_zero() : to_h4(dkacc[kt][jt]);
                 }
             }
 
@@ -791,8 +867,10 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
                     f4 acc = f4_zero();
-                    if (jt < 2) acc = mfma32(gf2[ct][0], row8(ATs, LDA, 16 * jt + row, 0, G), acc);
-                    acc = mfma32(gf2[ct][1], row8(ATs, LDA, 16 * jt + row, 32, G), acc);
+                    if (CAUSAL) {
+                        if (jt < 2) acc = mfma32(gf2[ct][0], row8(ATs, LDA, 16 * jt + row, 0, G), acc);
+                        acc = mfma32(gf2[ct][1], row8(ATs, LDA, 16 * jt + row, 32, G), acc);
+                    }
                     dvacc[ct][jt] = acc;
                 }
 #pragma unroll
@@ -822,7 +900,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
 
             // carried sums
 #pragma unroll
-            for (int is = 0; is < 2; ++is) {
+            for (int is = 0; is < (CAUSAL ? 2 : 0); ++is) {
 #pragma unroll
                 for (int ct = 0; ct < NCT; ++ct) {
                     h8 gf = col8(Gs, LDV, is * 32, 16 * ct, lane);
@@ -836,7 +914,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
                     for (int ct = 0; ct < NCT2; ++ct) RR[kt][ct] = mfma32(qa, gf2[ct][is], RR[kt][ct]);
                 }
             }
-            if (tid < KD) {
+            if (CAUSAL && tid < KD) {
                 float sr = 0.f;
 #pragma unroll 8
                 for (int i = 0; i < C; ++i) sr += (float)Qs[i * LDQ + tid] * gzs[i];

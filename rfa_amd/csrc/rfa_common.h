@@ -148,6 +148,18 @@ __device__ __forceinline__ void chunk_r2s(const ChunkRegs<F>& r, half_t* Xs, int
     }
 }
 
+// zero the rows whose mask byte is non-zero (mask already offset to the chunk's first step)
+template <int F>
+__device__ __forceinline__ void chunk_mask_rows(ChunkRegs<F>& r, const uint8_t* __restrict__ mask,
+                                                int rows_valid, int tid) {
+    constexpr int PPR = F / 8;
+#pragma unroll
+    for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
+        const int row = (tid + kThreads * it) / PPR;
+        if (row < rows_valid && mask[row]) r.v[it] = make_uint4(0u, 0u, 0u, 0u);
+    }
+}
+
 // same, each row multiplied by scale[piece] (fp32) before the store
 template <int F>
 __device__ __forceinline__ void chunk_r2s_scaled(const ChunkRegs<F>& r, const float* scale,

@@ -97,3 +97,170 @@ def backward(q: Tensor, k: Tensor, v: Tensor, grad_attn: Tensor) -> List[Tensor]
                                            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                                            T, N, K, d, ws.data_ptr(), nbytes, _stream_ptr(q.device)))
     return [dq, dk, dv]
+
+
+# ---------------------------------------------------------------------------
+# feature map
+# ---------------------------------------------------------------------------
+def feature_map_supported(D: int, d: int) -> bool:
+    return bool(_lib.load().rfa_feature_map_supported(int(D), int(d)))
+
+
+def _check_feature_args(x: Tensor, w: Tensor):
+    _check_half_cuda("x", x, 4)
+    _check_half_cuda("random_matrices", w, 3)
+    _require(w.shape[0] == x.shape[2] and w.shape[2] == x.shape[3], ValueError,
+             f"random_matrices {tuple(w.shape)} must be [num_heads, proj_dim, head_dim] for x {tuple(x.shape)}")
+    _require(x.device == w.device, RuntimeError, "x and random_matrices must be on one device")
+
+
+def feature_map_forward(x: Tensor, w: Tensor, scale: float) -> Tensor:
+    """phi [L, B, H, 2D] for x fp16 [L, B, H, d] and w fp16 [H, D, d]."""
+    _check_feature_args(x, w)
+    L, B, H, d = x.shape
+    D = w.shape[1]
+    phi = torch.empty((L, B, H, 2 * D), dtype=torch.float16, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().rfa_feature_map_forward(
+            x.data_ptr(), w.data_ptr(), phi.data_ptr(), L * B, H, D, d, float(scale), _stream_ptr(x.device)))
+    return phi
+
+
+def feature_map_backward(x: Tensor, w: Tensor, grad_phi: Tensor, scale: float):
+    """(dx fp16 [L,B,H,d], dw fp32 [H,D,d])."""
+    _check_feature_args(x, w)
+    L, B, H, d = x.shape
+    D = w.shape[1]
+    _check_half_cuda("grad_phi", grad_phi, 4)
+    _require(tuple(grad_phi.shape) == (L, B, H, 2 * D), ValueError,
+             f"grad_phi {tuple(grad_phi.shape)} must be {(L, B, H, 2 * D)}")
+    lib = _lib.load()
+    dx = torch.empty_like(x)
+    dw = torch.empty((H, D, d), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        nbytes = lib.rfa_feature_map_backward_workspace_bytes(L * B, H, D, d)
+        ws = _workspace(nbytes, x.device)
+        _lib.check(lib.rfa_feature_map_backward(
+            x.data_ptr(), w.data_ptr(), grad_phi.data_ptr(), dx.data_ptr(), dw.data_ptr(),
+            L * B, H, D, d, float(scale), ws.data_ptr(), nbytes, _stream_ptr(x.device)))
+    return dx, dw
+
+
+# ---------------------------------------------------------------------------
+# cross attention
+# ---------------------------------------------------------------------------
+def _check_f32_cuda(name: str, t: Tensor, shape):
+    _require(isinstance(t, Tensor) and t.is_cuda, RuntimeError, f"{name} must live on a HIP device")
+    _require(t.dtype == torch.float32, TypeError, f"{name} must be float32 (got {t.dtype})")
+    _require(tuple(t.shape) == tuple(shape), ValueError, f"{name} must have shape {tuple(shape)} (got {tuple(t.shape)})")
+    _require(t.is_contiguous(), ValueError, f"{name} must be contiguous")
+
+
+def _mask_arg(mask, B: int, S: int, device):
+    """key_padding_mask [B, S] (non-zero = pad) -> (uint8 tensor kept alive, pointer)."""
+    if mask is None:
+        return None, None
+    _require(tuple(mask.shape) == (B, S), ValueError, f"key_padding_mask must be [{B}, {S}] (got {tuple(mask.shape)})")
+    _require(mask.device == device, RuntimeError, "key_padding_mask must be on the tensors' device")
+    m = (mask != 0).to(torch.uint8).contiguous()
+    return m, m.data_ptr()
+
+
+def cross_state(phi_k: Tensor, v: Tensor, key_padding_mask=None):
+    """phi_k fp16 [S, B, H, K], v fp16 [S, B, H, d], mask [B, S] -> (s fp32 [B,H,K,d], z fp32 [B,H,K])."""
+    _check_half_cuda("phi_k", phi_k, 4)
+    _check_half_cuda("v", v, 4)
+    _require(phi_k.shape[:3] == v.shape[:3], ValueError, "phi_k and v must agree in [src_len, bsz, heads]")
+    S, B, H, K = phi_k.shape
+    d = v.shape[3]
+    s = torch.empty((B, H, K, d), dtype=torch.float32, device=v.device)
+    z = torch.empty((B, H, K), dtype=torch.float32, device=v.device)
+    keep, mptr = _mask_arg(key_padding_mask, B, S, v.device)
+    with torch.cuda.device(v.device):
+        _lib.check(_lib.load().rfa_cross_state(phi_k.data_ptr(), v.data_ptr(), mptr, s.data_ptr(), z.data_ptr(),
+                                               S, B, H, K, d, _stream_ptr(v.device)))
+    return s, z
+
+
+def cross_state_backward(phi_k: Tensor, v: Tensor, ds: Tensor, dz: Tensor, key_padding_mask=None):
+    _check_half_cuda("phi_k", phi_k, 4)
+    _check_half_cuda("v", v, 4)
+    S, B, H, K = phi_k.shape
+    d = v.shape[3]
+    _check_f32_cuda("ds", ds, (B, H, K, d))
+    _check_f32_cuda("dz", dz, (B, H, K))
+    dphi_k, dv = torch.empty_like(phi_k), torch.empty_like(v)
+    keep, mptr = _mask_arg(key_padding_mask, B, S, v.device)
+    with torch.cuda.device(v.device):
+        _lib.check(_lib.load().rfa_cross_state_backward(
+            phi_k.data_ptr(), v.data_ptr(), mptr, ds.data_ptr(), dz.data_ptr(), dphi_k.data_ptr(), dv.data_ptr(),
+            S, B, H, K, d, _stream_ptr(v.device)))
+    return dphi_k, dv
+
+
+def cross_readout(phi_q: Tensor, s: Tensor, z: Tensor) -> Tensor:
+    """phi_q fp16 [T, B, H, K], s fp32 [B,H,K,d], z fp32 [B,H,K] -> attn fp16 [T, B, H, d]."""
+    _check_half_cuda("phi_q", phi_q, 4)
+    T, B, H, K = phi_q.shape
+    _require(s.dim() == 4, ValueError, "s must be [bsz, heads, 2*proj_dim, head_dim]")
+    d = s.shape[3]
+    _check_f32_cuda("s", s, (B, H, K, d))
+    _check_f32_cuda("z", z, (B, H, K))
+    out = torch.empty((T, B, H, d), dtype=torch.float16, device=phi_q.device)
+    with torch.cuda.device(phi_q.device):
+        _lib.check(_lib.load().rfa_cross_readout(phi_q.data_ptr(), s.data_ptr(), z.data_ptr(), out.data_ptr(),
+                                                 T, B * H, K, d, _stream_ptr(phi_q.device)))
+    return out
+
+
+def cross_readout_backward(phi_q: Tensor, s: Tensor, z: Tensor, grad_attn: Tensor):
+    _check_half_cuda("phi_q", phi_q, 4)
+    T, B, H, K = phi_q.shape
+    d = s.shape[3]
+    _check_f32_cuda("s", s, (B, H, K, d))
+    _check_f32_cuda("z", z, (B, H, K))
+    _check_half_cuda("grad_attn", grad_attn, 4)
+    _require(tuple(grad_attn.shape) == (T, B, H, d), ValueError, "grad_attn must be [tgt_len, bsz, heads, head_dim]")
+    dphi_q = torch.empty_like(phi_q)
+    ds, dz = torch.empty_like(s), torch.empty_like(z)
+    with torch.cuda.device(phi_q.device):
+        _lib.check(_lib.load().rfa_cross_readout_backward(
+            phi_q.data_ptr(), s.data_ptr(), z.data_ptr(), grad_attn.data_ptr(), dphi_q.data_ptr(),
+            ds.data_ptr(), dz.data_ptr(), T, B * H, K, d, _stream_ptr(phi_q.device)))
+    return dphi_q, ds, dz
+
+
+# ---------------------------------------------------------------------------
+# incremental decoding (state updated in place)
+# ---------------------------------------------------------------------------
+def incremental(phi_q: Tensor, phi_k: Tensor, v: Tensor, s: Tensor, z: Tensor) -> Tensor:
+    """phi_q, phi_k fp16 [steps, N, K]; v fp16 [steps, N, d]; s fp32 [N,K,d], z fp32 [N,K] updated in place."""
+    _check_qkv(phi_q, phi_k, v)
+    steps, N, K = phi_q.shape
+    d = v.shape[2]
+    _check_f32_cuda("s", s, (N, K, d))
+    _check_f32_cuda("z", z, (N, K))
+    out = torch.empty_like(v)
+    with torch.cuda.device(v.device):
+        _lib.check(_lib.load().rfa_incremental(phi_q.data_ptr(), phi_k.data_ptr(), v.data_ptr(), s.data_ptr(),
+                                               z.data_ptr(), out.data_ptr(), steps, N, K, d, _stream_ptr(v.device)))
+    return out
+
+
+def incremental_fused(q: Tensor, k: Tensor, v: Tensor, w: Tensor, scale: float, s: Tensor, z: Tensor) -> Tensor:
+    """q, k, v fp16 [steps, B, H, d]; w fp16 [H, D, d]; s fp32 [B,H,2D,d], z fp32 [B,H,2D] updated in place."""
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_half_cuda(name, t, 4)
+    _require(q.shape == k.shape == v.shape, ValueError, "q, k, v must have one shape [steps, bsz, heads, head_dim]")
+    _check_half_cuda("random_matrices", w, 3)
+    steps, B, H, d = q.shape
+    D = w.shape[1]
+    _require(w.shape[0] == H and w.shape[2] == d, ValueError, "random_matrices must be [heads, proj_dim, head_dim]")
+    _check_f32_cuda("s", s, (B, H, 2 * D, d))
+    _check_f32_cuda("z", z, (B, H, 2 * D))
+    out = torch.empty_like(v)
+    with torch.cuda.device(v.device):
+        _lib.check(_lib.load().rfa_incremental_fused(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), w.data_ptr(), float(scale), s.data_ptr(), z.data_ptr(),
+            out.data_ptr(), steps, B, H, D, d, _stream_ptr(v.device)))
+    return out

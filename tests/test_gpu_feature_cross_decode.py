@@ -1,0 +1,165 @@
+"""GPU parity (through the C ABI) of the feature map, the cross-attention
+contractions and the decode step against the CPU oracle.
+
+Tolerances: fp16 outputs max-abs <= 2e-3 vs the fp32 oracle on identical
+fp16-rounded inputs; gradients <= 1e-2 relative Frobenius error; fp32 states
+<= 1e-3 relative.
+"""
+import pytest
+import torch
+
+from oracle import rfa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+OUT_ATOL = 2e-3
+GRAD_RTOL = 1e-2
+
+
+def _rel(a, b):
+    return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+def _randn(*shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=torch.float32)
+
+
+# ------------------------------------------------------------------ feature map
+FEATURE_SHAPES = [(128, 2, 4, 64, 64), (3, 1, 2, 64, 32), (70, 3, 2, 128, 128), (1, 1, 1, 64, 128), (33, 2, 3, 128, 64)]
+
+
+@pytest.mark.parametrize("L,B,H,d,D", FEATURE_SHAPES)
+def test_feature_map_forward(L, B, H, d, D):
+    from rfa_amd import rfa_hip
+    x = (_randn(L, B, H, d, seed=10 + L) * 1.7).half()
+    x[0, 0, 0] = 0                                  # zero row: phi = [0.., 0.1..]
+    w = (_randn(H, D, d, seed=11) * 0.9).half()
+    print(f"phi fwd L={L} B={B} H={H} d={d} D={D}", flush=True)
+    got = rfa_hip.feature_map_forward(x.cuda(), w.cuda(), O.SCALE).float().cpu()
+    want = O.random_project(x.float(), w.float())
+    assert (got - want).abs().max().item() <= 3e-4     # |phi| <= 0.1: half an fp16 ulp is 3e-5
+    assert torch.equal(got[0, 0, 0, :D], torch.zeros(D))
+
+
+@pytest.mark.parametrize("L,B,H,d,D", FEATURE_SHAPES)
+def test_feature_map_backward(L, B, H, d, D):
+    from rfa_amd import rfa_hip
+    x = (_randn(L, B, H, d, seed=20 + L) * 1.3).half()
+    if L > 1:
+        x[1, 0, 0] = 0                              # ||x|| = 0 row must give dx = finite
+    w = (_randn(H, D, d, seed=21) * 0.9).half()
+    g = _randn(L, B, H, 2 * D, seed=22).half()
+    print(f"phi bwd L={L} B={B} H={H} d={d} D={D}", flush=True)
+    dx, dw = rfa_hip.feature_map_backward(x.cuda(), w.cuda(), g.cuda(), O.SCALE)
+    dx, dw = dx.float().cpu(), dw.cpu()
+    rx, rw = O.random_project_backward(x.float(), w.float(), g.float())
+    assert torch.isfinite(dx).all() and torch.isfinite(dw).all()
+    assert _rel(dx, rx) <= GRAD_RTOL, _rel(dx, rx)
+    assert _rel(dw, rw) <= GRAD_RTOL, _rel(dw, rw)
+
+
+# ------------------------------------------------------------------------ cross
+def _cross_inputs(S, T, B, H, d, D, seed, lengths=None):
+    W = O.make_w(d, D, H)
+    k = O.unit_rows(_randn(S, B, H, d, seed=seed)).half()
+    q = O.unit_rows(_randn(T, B, H, d, seed=seed + 1)).half()
+    v = _randn(S, B, H, d, seed=seed + 2).half()
+    g = _randn(T, B, H, d, seed=seed + 3).half()
+    pk = O.random_project(k.float(), W).half()
+    pq = O.random_project(q.float(), W).half()
+    mask = None
+    if lengths is not None:
+        mask = torch.zeros(B, S, dtype=torch.bool)
+        for b, L in enumerate(lengths):
+            mask[b, L:] = True
+    return pq, pk, v, g, mask
+
+
+CROSS_SHAPES = [
+    # S, T, B, H, d, D, lengths
+    (96, 40, 2, 2, 64, 64, None),
+    (130, 70, 3, 2, 64, 64, [130, 64, 7]),
+    (64, 1, 1, 1, 64, 32, [33]),
+    (200, 129, 1, 2, 128, 64, [150]),
+    (70, 65, 2, 1, 64, 128, None),
+]
+
+
+@pytest.mark.parametrize("S,T,B,H,d,D,lengths", CROSS_SHAPES)
+def test_cross_forward(S, T, B, H, d, D, lengths):
+    from rfa_amd import rfa_hip
+    pq, pk, v, g, mask = _cross_inputs(S, T, B, H, d, D, 300 + S, lengths)
+    print(f"cross fwd S={S} T={T} B={B} H={H} d={d} D={D}", flush=True)
+    s, z = rfa_hip.cross_state(pk.cuda(), v.cuda(), None if mask is None else mask.cuda())
+    rs, rz = O.cross_state(pk.float(), v.float(), None if mask is None else mask.t())
+    assert _rel(s.cpu(), rs) <= 1e-3 and _rel(z.cpu(), rz) <= 1e-3
+    out = rfa_hip.cross_readout(pq.cuda(), s, z).float().cpu()
+    want = O.cross_readout(pq.float(), rs, rz)
+    assert (out - want).abs().max().item() <= OUT_ATOL
+
+
+def test_cross_readout_negative_denominator():
+    """abs() in the denominator: flip the sign of z so that q.z < -1."""
+    from rfa_amd import rfa_hip
+    pq, pk, v, g, _ = _cross_inputs(256, 64, 1, 2, 64, 64, 400)
+    rs, rz = O.cross_state(pk.float(), v.float())
+    rz = -rz
+    assert (torch.einsum("tbhk,bhk->tbh", pq.float(), rz) < -1).any()
+    out = rfa_hip.cross_readout(pq.cuda(), rs.cuda().contiguous(), rz.cuda().contiguous()).float().cpu()
+    assert (out - O.cross_readout(pq.float(), rs, rz)).abs().max().item() <= OUT_ATOL
+    dq, ds, dz = rfa_hip.cross_readout_backward(pq.cuda(), rs.cuda().contiguous(), rz.cuda().contiguous(), g.cuda())
+    wq, ws, wz = O.cross_readout_backward(pq.float(), rs, rz, g.float())
+    assert _rel(dq.float().cpu(), wq) <= GRAD_RTOL
+    assert _rel(ds.cpu(), ws) <= GRAD_RTOL and _rel(dz.cpu(), wz) <= GRAD_RTOL
+
+
+@pytest.mark.parametrize("S,T,B,H,d,D,lengths", CROSS_SHAPES)
+def test_cross_backward(S, T, B, H, d, D, lengths):
+    from rfa_amd import rfa_hip
+    pq, pk, v, g, mask = _cross_inputs(S, T, B, H, d, D, 500 + S, lengths)
+    print(f"cross bwd S={S} T={T} B={B} H={H} d={d} D={D}", flush=True)
+    omask = None if mask is None else mask.t()
+    rs, rz = O.cross_state(pk.float(), v.float(), omask)
+    wq, wds, wdz = O.cross_readout_backward(pq.float(), rs, rz, g.float())
+    wk, wv = O.cross_state_backward(pk.float(), v.float(), wds, wdz, omask)
+    cmask = None if mask is None else mask.cuda()
+    s, z = rfa_hip.cross_state(pk.cuda(), v.cuda(), cmask)
+    dq, ds, dz = rfa_hip.cross_readout_backward(pq.cuda(), s, z, g.cuda())
+    dk, dv = rfa_hip.cross_state_backward(pk.cuda(), v.cuda(), ds, dz, cmask)
+    for name, got, want in (("dq", dq, wq), ("ds", ds, wds), ("dz", dz, wdz), ("dk", dk, wk), ("dv", dv, wv)):
+        got = got.float().cpu()
+        assert torch.isfinite(got).all(), name
+        assert _rel(got, want) <= GRAD_RTOL, (name, _rel(got, want))
+    if mask is not None:
+        assert (dk.float().cpu()[mask.t()] == 0).all()
+
+
+# ----------------------------------------------------------------------- decode
+@pytest.mark.parametrize("B,H,d,D,prefill,steps", [(2, 4, 64, 64, 0, 5), (3, 2, 64, 64, 40, 9), (1, 2, 128, 64, 17, 4),
+                                                   (2, 1, 64, 128, 10, 3), (1, 1, 128, 128, 5, 3), (2, 2, 64, 32, 3, 4)])
+def test_incremental_matches_oracle(B, H, d, D, prefill, steps):
+    from rfa_amd import rfa_hip
+    T = prefill + steps
+    q, k, v, _ = O.make_qkv(T, B, H, d, 700 + T)
+    W = O.make_w(d, D, H)
+    N, K = B * H, 2 * D
+    pq = O.random_project(q.float(), W).half().reshape(T, N, K)
+    pk = O.random_project(k.float(), W).half().reshape(T, N, K)
+    vv = v.reshape(T, N, d)
+    want, ws, wz = O.causal_forward_loop(pq.float(), pk.float(), vv.float())
+    _, s0, z0 = O.causal_forward_loop(pq[:prefill].float(), pk[:prefill].float(), vv[:prefill].float())
+    print(f"decode B={B} H={H} d={d} D={D} prefill={prefill} steps={steps}", flush=True)
+    # feature-level entry point
+    s, z = s0.cuda().contiguous(), z0.cuda().contiguous()
+    out = rfa_hip.incremental(pq[prefill:].cuda().contiguous(), pk[prefill:].cuda().contiguous(),
+                              vv[prefill:].cuda().contiguous(), s, z).float().cpu()
+    assert (out - want[prefill:]).abs().max().item() <= OUT_ATOL
+    assert _rel(s.cpu(), ws) <= 1e-3 and _rel(z.cpu(), wz) <= 1e-3
+    # fused entry point: raw q, k plus the random matrix
+    s = s0.cuda().reshape(B, H, K, d).contiguous()
+    z = z0.cuda().reshape(B, H, K).contiguous()
+    out2 = rfa_hip.incremental_fused(q[prefill:].cuda().contiguous(), k[prefill:].cuda().contiguous(),
+                                     v[prefill:].cuda().contiguous(), W.half().cuda(), O.SCALE, s, z).float().cpu()
+    assert (out2.reshape(steps, N, d) - want[prefill:]).abs().max().item() <= OUT_ATOL
+    assert _rel(s.cpu().reshape(N, K, d), ws) <= 2e-3
