@@ -1,0 +1,253 @@
+#!/usr/bin/env python
+"""Benchmark of the RFA kernel path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one causal forward + backward over one batch of synthetic input at the
+configuration the headline metric is quoted on (seq 1024, batch 8, 8 heads,
+head_dim 64, proj_dim 64, fp16), called through the C ABI (rfa_causal_forward +
+rfa_causal_backward) with all inputs resident in HBM.  One JSON line is printed:
+the throughput of that step, the roofline of its dominant kernel (per-kernel
+durations from HIP events recorded by the library around every launch), the same
+step timed with the CPU oracle on the host cores, and -- as extra keys -- the decode,
+cross-attention and feature-map figures.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def _event_time_ms(torch, fn, iters):
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip decode / cross / feature-map figures")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: every box of this build has one GPU and the path needs no "
+                 "second one (sequences are independent); run with --gpus 1")
+
+    import torch
+    from oracle import rfa_oracle as O
+    from rfa_amd import _lib, rfa_hip
+    lib = _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    # ---------------------------------------------------------------- workload (config 2)
+    T, B, H, d, D = 1024, 8, 8, 64, 64
+    N, K = B * H, 2 * D
+    q, k, v, g = O.make_qkv(T, B, H, d, seed=1234 + 2)
+    W = O.make_w(d, D, H).half()
+    cq, ck, cv, cg = (t.to(dev).contiguous() for t in (q, k, v, g))
+    cW = W.to(dev)
+    pq = rfa_hip.feature_map_forward(cq, cW, O.SCALE).view(T, N, K)
+    pk = rfa_hip.feature_map_forward(ck, cW, O.SCALE).view(T, N, K)
+    vv, gg = cv.view(T, N, d), cg.view(T, N, d)
+    out = torch.empty_like(vv)
+    dq, dk, dv = torch.empty_like(pq), torch.empty_like(pk), torch.empty_like(vv)
+    fbytes = lib.rfa_causal_forward_workspace_bytes(T, N, K, d)
+    bbytes = lib.rfa_causal_backward_workspace_bytes(T, N, K, d)
+    ws = torch.empty(max(fbytes, bbytes, 1), dtype=torch.uint8, device=dev)
+    p = lambda t: t.data_ptr()
+
+    def step():
+        _lib.check(lib.rfa_causal_forward(p(pq), p(pk), p(vv), p(out), T, N, K, d, p(ws), fbytes, stream))
+        _lib.check(lib.rfa_causal_backward(p(pq), p(pk), p(vv), p(gg), p(dq), p(dk), p(dv), T, N, K, d,
+                                           p(ws), bbytes, stream))
+
+    for _ in range(args.warmup):
+        step()
+    ms_per_step = _event_time_ms(torch, step, args.steps)          # the timed region: exactly K steps
+    tokens = B * T
+    value = tokens / (ms_per_step * 1e-3)
+
+    # parity gate next to the timing (fp32 oracle on a slice of the batch: first 8 sequences)
+    ns = 8
+    ref = O.causal_forward_chunked(pq[:, :ns].float().cpu(), pk[:, :ns].float().cpu(), vv[:, :ns].float().cpu())
+    rq, rk, rv = O.causal_backward_chunked(pq[:, :ns].float().cpu(), pk[:, :ns].float().cpu(),
+                                           vv[:, :ns].float().cpu(), gg[:, :ns].float().cpu())
+    rel = lambda a, b: ((a.float().cpu() - b).norm() / b.norm()).item()
+    parity = {"out_max_abs": (out[:, :ns].float().cpu() - ref).abs().max().item(),
+              "dq_rel": rel(dq[:, :ns], rq), "dk_rel": rel(dk[:, :ns], rk), "dv_rel": rel(dv[:, :ns], rv)}
+    parity["ok"] = bool(parity["out_max_abs"] <= 2e-3 and max(parity["dq_rel"], parity["dk_rel"], parity["dv_rel"]) <= 1e-2)
+
+    # ---------------------------------------------------------------- per-kernel durations
+    _lib.check(lib.rfa_profile_reset())
+    _lib.check(lib.rfa_profile_enable(1))
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    _lib.check(lib.rfa_profile_enable(0))
+    totals = _lib.profile_totals()
+    kern_us = {n: 1e3 * ms / c for n, (ms, c) in totals.items()}
+    # algorithmic HBM bytes per launch: each kernel's inputs read once + outputs written once
+    per_tok = {
+        "k_segment_state": (K + d) * 2,
+        "k_causal_fwd": (2 * K + d) * 2 + d * 2,
+        "k_causal_bwd_dq": (2 * K + 2 * d) * 2 + K * 2 + 8,
+        "k_causal_bwd_dkdv": (2 * K + 2 * d) * 2 + 8 + (K + d) * 2,
+    }
+    nseg = lib.rfa_causal_num_segments(T, N)
+    units = {n_: N * T for n_ in per_tok}
+    units["k_segment_state"] = N * T * (nseg - 1) // max(nseg, 1)
+    dominant = max((n_ for n_ in kern_us if n_ in per_tok), key=lambda n_: totals[n_][0])
+    dom_bytes = per_tok[dominant] * units[dominant]
+    achieved = dom_bytes / (kern_us[dominant] * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "bytes_per_launch": dom_bytes, "avg_us": round(kern_us[dominant], 2),
+                "kernels_us": {n_: round(u, 2) for n_, u in kern_us.items()},
+                "step_algorithmic_bytes": 2176 * N * T,
+                "step_frac_of_hbm": round(2176 * N * T / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    # ---------------------------------------------------------------- CPU baseline (oracle port)
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        cores = os.cpu_count() or 1
+        cores = min(cores, 16)
+        torch.set_num_threads(cores)
+        bs = 2                                                 # sample: 2 of the 8 batch entries
+        sq, sk = pq[:, :bs * H].float().cpu(), pk[:, :bs * H].float().cpu()
+        sv, sg = vv[:, :bs * H].float().cpu(), gg[:, :bs * H].float().cpu()
+        times = []
+        for it in range(3):
+            t0 = time.perf_counter()
+            O.causal_forward_cumsum(sq, sk, sv)
+            O.causal_backward_cumsum(sq, sk, sv, sg)
+            times.append(time.perf_counter() - t0)
+        tcpu = sorted(times[1:])[0] if len(times) > 1 else times[0]
+        cpu_baseline = {"value": round(bs * T / tcpu, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+                        "sample": f"causal fwd+bwd, cumulative-sum form (rfa.py:46-103) in fp32 torch-CPU on {bs} of "
+                                  f"{B} batch entries (T={T}, {bs * H} sequences), 1 warm-up, best of 2",
+                        "speedup": round(value / (bs * T / tcpu), 1)}
+
+    result = {
+        "metric": "causal fwd+bwd tok/s @L=1024 fp16", "value": round(value, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16 in, fp32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: RFA causal self-attention fwd+bwd, seq 1024, batch 8, 8 heads, "
+                               "head_dim 64, proj_dim 64 (phi width 128), feature-level boundary RFA.apply",
+                   "T": T, "B": B, "H": H, "head_dim": d, "proj_dim": D, "segments": nseg},
+        "parity": parity, "roofline": roofline, "cpu_baseline": cpu_baseline,
+    }
+
+    if not args.no_extras:
+        result["extras"] = extras(torch, O, lib, _lib, rfa_hip, dev, stream)
+    print(json.dumps(result))
+
+
+def extras(torch, O, lib, _lib, rfa_hip, dev, stream):
+    ex = {}
+    p = lambda t: t.data_ptr()
+    # ---- decode (config 4): B64 H16 d64 D64, 2048 steps after a 512-token prefill
+    B, H, d, D, prefill, steps = 64, 16, 64, 64, 512, 2048
+    N, K = B * H, 2 * D
+    g = torch.Generator(device="cpu").manual_seed(1234 + 4)
+    W = O.make_w(d, D, H).half().to(dev)
+    unit = lambda t: t / t.norm(dim=-1, keepdim=True)
+    pk_ = unit(torch.randn(prefill, B, H, d, generator=g)).half().to(dev)
+    pv_ = torch.randn(prefill, B, H, d, generator=g).half().to(dev)
+    s0, z0 = rfa_hip.cross_state(rfa_hip.feature_map_forward(pk_, W, O.SCALE), pv_)   # prefill state = sum over 512 tokens
+    del pk_, pv_
+    chunk = 256
+    qs = unit(torch.randn(chunk, B, H, d, generator=g)).half().to(dev).repeat(steps // chunk, 1, 1, 1)
+    ks = unit(torch.randn(chunk, B, H, d, generator=g)).half().to(dev).repeat(steps // chunk, 1, 1, 1)
+    vs = torch.randn(chunk, B, H, d, generator=g).half().to(dev).repeat(steps // chunk, 1, 1, 1)
+    outs = torch.empty_like(vs)
+    s, z = s0.clone(), z0.clone()
+
+    def run_decode():
+        _lib.check(lib.rfa_incremental_fused(p(qs), p(ks), p(vs), p(W), O.SCALE, p(s), p(z), p(outs),
+                                             steps, B, H, D, d, stream))
+    run_decode()
+    s.copy_(s0); z.copy_(z0)
+    ms = _event_time_ms(torch, run_decode, 1)
+    step_bytes = 67072 * N
+    ex["decode"] = {"workload": "configs[3]: batch 64 x 16 heads, head_dim 64, proj_dim 64, 2048 steps after a "
+                                "512-token prefill, fused feature map, fp32 state in place, one launch per step",
+                    "tokens_per_s": round(B * steps / (ms * 1e-3), 1), "us_per_step": round(1e3 * ms / steps, 3),
+                    "algorithmic_bytes_per_step": step_bytes,
+                    "hbm_gbs": round(step_bytes * steps / (ms * 1e-3) / 1e9, 1),
+                    "hbm_frac": round(step_bytes * steps / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    # parity of the first steps against the oracle on 2 heads
+    s.copy_(s0); z.copy_(z0)
+    _lib.check(lib.rfa_incremental_fused(p(qs), p(ks), p(vs), p(W), O.SCALE, p(s), p(z), p(outs), 8, B, H, D, d, stream))
+    torch.cuda.synchronize()
+    Wc = W.float().cpu()[:2]
+    fq = O.random_project(qs[:8, :1, :2].float().cpu(), Wc).reshape(8, 2, K)
+    fk = O.random_project(ks[:8, :1, :2].float().cpu(), Wc).reshape(8, 2, K)
+    want, _, _ = O.causal_forward_loop(fq, fk, vs[:8, :1, :2].float().cpu().reshape(8, 2, d),
+                                       s0[:1, :2].cpu().reshape(2, K, d), z0[:1, :2].cpu().reshape(2, K))
+    ex["decode"]["parity_max_abs"] = (outs[:8, :1, :2].float().cpu().reshape(8, 2, d) - want).abs().max().item()
+    del qs, ks, vs, outs
+
+    # ---- cross attention (config 3): T256 S512 B32 H8, lengths U[256, 512]
+    Tt, S, B, H = 256, 512, 32, 8
+    N = B * H
+    g = torch.Generator(device="cpu").manual_seed(1234 + 3)
+    W = O.make_w(d, D, H).half().to(dev)
+    lens = torch.randint(256, 513, (B,), generator=g)
+    pad = (torch.arange(S)[None, :] >= lens[:, None]).to(torch.uint8).to(dev)
+    pk = rfa_hip.feature_map_forward(unit(torch.randn(S, B, H, d, generator=g)).half().to(dev), W, O.SCALE)
+    pq = rfa_hip.feature_map_forward(unit(torch.randn(Tt, B, H, d, generator=g)).half().to(dev), W, O.SCALE)
+    v = torch.randn(S, B, H, d, generator=g).half().to(dev)
+    go = torch.randn(Tt, B, H, d, generator=g).half().to(dev)
+
+    def cross_step():
+        s_, z_ = rfa_hip.cross_state(pk, v, pad)
+        rfa_hip.cross_readout(pq, s_, z_)
+        _, ds, dz = rfa_hip.cross_readout_backward(pq, s_, z_, go)
+        rfa_hip.cross_state_backward(pk, v, ds, dz, pad)
+    for _ in range(5):
+        cross_step()
+    ms = _event_time_ms(torch, cross_step, 50)
+    flops = 6 * K * d * float((lens + Tt).sum()) * H
+    ex["cross"] = {"workload": "configs[2]: tgt 256, src 512, batch 32, 8 heads, lengths U[256,512], fwd+bwd",
+                   "tgt_tokens_per_s": round(B * Tt / (ms * 1e-3), 1), "us_per_step": round(1e3 * ms, 2),
+                   "algorithmic_tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
+
+    # ---- feature map (config 2 shape): phi forward + backward for q
+    T, B, H = 1024, 8, 8
+    x = torch.randn(T, B, H, d, generator=g).half().to(dev)
+    gp = torch.randn(T, B, H, 2 * D, generator=g).half().to(dev)
+    f = lambda: rfa_hip.feature_map_forward(x, W, O.SCALE)
+    b = lambda: rfa_hip.feature_map_backward(x, W, gp, O.SCALE)
+    for _ in range(5):
+        f(); b()
+    tf, tb = _event_time_ms(torch, f, 50), _event_time_ms(torch, b, 50)
+    rows = T * B * H
+    ex["feature_map"] = {"workload": "phi of [1024, 8, 8, 64] -> [.., 128]", "fwd_us": round(1e3 * tf, 2),
+                         "bwd_us": round(1e3 * tb, 2),
+                         "fwd_hbm_gbs": round(rows * (d + 2 * D) * 2 / (tf * 1e-3) / 1e9, 1),
+                         "bwd_hbm_gbs": round(rows * (2 * d + 2 * D) * 2 / (tb * 1e-3) / 1e9, 1)}
+    return ex
+
+
+if __name__ == "__main__":
+    main()

@@ -148,6 +148,19 @@ int rfa_incremental(const void* phi_q, const void* phi_k, const void* v, float* 
 int rfa_incremental_fused(const void* q, const void* k, const void* v, const void* w, float scale, float* s,
                           float* z, void* out, int64_t steps, int64_t B, int H, int D, int d, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Per-kernel timing (no counterpart in the reference; used by bench.py).
+ * While enabled, every kernel launch of this library is bracketed by a HIP event
+ * pair on its stream.  rfa_profile_collect waits for the recorded pairs and adds
+ * their elapsed times to per-kernel totals; rfa_profile_get reads one total
+ * (index in [0, rfa_profile_kernel_count())); rfa_profile_reset clears them.
+ * ------------------------------------------------------------------------- */
+int rfa_profile_enable(int on);
+int rfa_profile_collect(void);
+int rfa_profile_reset(void);
+int rfa_profile_kernel_count(void);
+int rfa_profile_get(int index, const char** name, double* total_ms, int64_t* calls);
+
 #ifdef __cplusplus
 }
 #endif

@@ -9,7 +9,7 @@ from __future__ import annotations
 import ctypes
 import os
 import re
-from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "librfa_hip.so")
@@ -48,6 +48,11 @@ SIGNATURES = {
     "rfa_cross_readout_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_void_p]),
     "rfa_cross_state_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
     "rfa_incremental": (c_int, [c_void_p] * 6 + [c_int64, c_int64, c_int, c_int, c_void_p]),
+    "rfa_profile_enable": (c_int, [c_int]),
+    "rfa_profile_collect": (c_int, []),
+    "rfa_profile_reset": (c_int, []),
+    "rfa_profile_kernel_count": (c_int, []),
+    "rfa_profile_get": (c_int, [c_int, POINTER(c_char_p), POINTER(c_double), POINTER(c_int64)]),
     "rfa_incremental_fused": (c_int, [c_void_p] * 4 + [c_float] + [c_void_p] * 3 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
 }
 
@@ -81,3 +86,16 @@ def declared_symbols() -> list:
     with open(HEADER_PATH) as f:
         text = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
     return sorted(set(re.findall(r"\b(rfa_[a-z0-9_]+)\s*\(", text)))
+
+
+def profile_totals() -> dict:
+    """{kernel name: (total_ms, calls)} accumulated since the last rfa_profile_reset."""
+    lib = load()
+    check(lib.rfa_profile_collect())
+    out = {}
+    for i in range(lib.rfa_profile_kernel_count()):
+        name, ms, calls = c_char_p(), c_double(), c_int64()
+        check(lib.rfa_profile_get(i, name, ms, calls))
+        if calls.value:
+            out[name.value.decode()] = (ms.value, calls.value)
+    return out

@@ -1,0 +1,180 @@
+"""Causal random feature attention; mirror of random_feature_attention/causal_attention.py.
+
+Functional forms (keyword-only, as in the reference):
+  incremental_rfa   decode loop                       -> HIP step kernel, fp32 state
+  cuda_causal_rfa   training / prefill                -> HIP chunked-scan kernels via RFA.apply
+  masked_rfa        quadratic form with explicit masks -> ATen ops, as in the reference
+and the ``CausalAttention`` module with the reference's parameter names
+(q_proj, k_proj, v_proj, out_proj, sigma) and ``saved_state`` keys
+("prev_s", "prev_z").
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+from torch import Tensor, nn
+from torch.nn import Parameter
+
+from . import rfa_hip
+from .rfa import RFA
+from .utils import (EPS, SCALE, build_random_matrices, normalize_attn_weights, random_project,
+                    upgrade_state_dict_named)
+
+
+def _drop_scalar_mask(mask: Optional[Tensor]) -> Optional[Tensor]:
+    # a 0-dim tensor stands for "no mask" (reference causal_attention.py:83-84,134-135)
+    if mask is not None and mask.dim() == 0:
+        return None
+    return mask
+
+
+def incremental_rfa(*, phi_q: Tensor, phi_k: Tensor, v: Tensor, s: Optional[Tensor] = None,
+                    z: Optional[Tensor] = None, inplace: bool = False):
+    """Per-step causal RFA (reference causal_attention.py:17-54).
+
+    phi_q, phi_k: [tgt_len, bsz, heads, 2*proj_dim]; v: [tgt_len, bsz, heads, head_dim];
+    s: [bsz, heads, 2*proj_dim, head_dim]; z: [bsz, heads, 2*proj_dim] (fp32; None = zeros).
+    Returns (attn [tgt_len, bsz, heads*head_dim], s, z).  With ``inplace=False`` (the
+    reference's behaviour) the given state is left untouched and new tensors are
+    returned; ``inplace=True`` updates s and z where they are.  Inference only.
+    """
+    tgt_len, bsz, num_heads, feat = phi_q.size()
+    head_dim = v.size(-1)
+    if s is None:
+        assert z is None
+        s = torch.zeros((bsz, num_heads, feat, head_dim), device=v.device, dtype=torch.float32)
+        z = torch.zeros((bsz, num_heads, feat), device=v.device, dtype=torch.float32)
+    else:
+        assert z is not None
+        if s.dtype != torch.float32 or z.dtype != torch.float32 or not inplace:
+            s = s.to(torch.float32, copy=True)
+            z = z.to(torch.float32, copy=True)
+        s, z = s.contiguous(), z.contiguous()
+    n = bsz * num_heads
+    attn = rfa_hip.incremental(
+        phi_q.detach().to(torch.float16).contiguous().view(tgt_len, n, feat),
+        phi_k.detach().to(torch.float16).contiguous().view(tgt_len, n, feat),
+        v.detach().to(torch.float16).contiguous().view(tgt_len, n, head_dim),
+        s.view(n, feat, head_dim), z.view(n, feat))
+    return attn.to(v.dtype).view(tgt_len, bsz, num_heads * head_dim), s, z
+
+
+def masked_rfa(*, phi_q: Tensor, phi_k: Tensor, v: Tensor, key_padding_mask: Optional[Tensor] = None,
+               attn_mask: Optional[Tensor] = None) -> Tensor:
+    """Quadratic-form RFA with explicit masks (reference causal_attention.py:57-109).
+
+    Note its normaliser, |row sum|.clamp(1e-3) in fp32 (utils.py:123-130), is not the
+    clamp-at-1 of the scan path.  Runs as ATen ops on the tensors' device.
+    """
+    tgt_len, bsz, num_heads, _ = phi_q.size()
+    head_dim = v.size(-1)
+    key_padding_mask = _drop_scalar_mask(key_padding_mask)
+    weights = torch.einsum("tbhk,sbhk->bhts", phi_q, phi_k)
+    if key_padding_mask is not None:
+        assert key_padding_mask.size(0) == bsz and key_padding_mask.size(1) == tgt_len
+        weights = weights.masked_fill(key_padding_mask.to(torch.bool)[:, None, None, :], 0.0)
+    if attn_mask is not None:
+        weights = weights.masked_fill((attn_mask < 0.0)[None, None], 0.0)
+    weights = normalize_attn_weights(weights, dtype=weights.dtype)
+    attn = torch.einsum("bhts,sbhd->tbhd", weights, v)
+    return attn.contiguous().view(tgt_len, bsz, num_heads * head_dim)
+
+
+def cuda_causal_rfa(*, phi_q: Tensor, phi_k: Tensor, v: Tensor,
+                    key_padding_mask: Optional[Tensor] = None) -> Tensor:
+    """Causal RFA through the fused kernels (reference causal_attention.py:112-151).
+
+    key_padding_mask: [bsz, tgt_len], 1 = padded key, whose phi_k is zeroed.
+    Returns attn [tgt_len, bsz, heads*head_dim].
+    """
+    tgt_len, bsz, num_heads, feat = phi_q.size()
+    head_dim = v.size(-1)
+    key_padding_mask = _drop_scalar_mask(key_padding_mask)
+    if key_padding_mask is not None:
+        assert key_padding_mask.size(0) == bsz and key_padding_mask.size(1) == tgt_len
+        pad = key_padding_mask.to(torch.bool).transpose(0, 1)[:, :, None, None]
+        phi_k = phi_k.masked_fill(pad, 0.0)
+    n = bsz * num_heads
+    attn = RFA.apply(phi_q.contiguous().view(tgt_len, n, feat),
+                     phi_k.contiguous().view(tgt_len, n, feat),
+                     v.contiguous().view(tgt_len, n, head_dim))
+    return attn.contiguous().view(tgt_len, bsz, num_heads * head_dim)
+
+
+# name without the vendor prefix
+hip_causal_rfa = cuda_causal_rfa
+
+
+class CausalAttention(nn.Module):
+    """Causal random feature self-attention (reference causal_attention.py:154-280)."""
+
+    def __init__(self, *, embed_dim: int, num_heads: int, head_dim: int, proj_dim: int, tau: float = 1.0,
+                 reparam_proj: bool = True, cuda_causal_rfa: bool = True):
+        super().__init__()
+        assert head_dim * num_heads == embed_dim, "embed_dim must be divisible by num_heads"
+        self.embed_dim, self.num_heads, self.head_dim, self.proj_dim = embed_dim, num_heads, head_dim, proj_dim
+        self.reparam_proj, self.cuda_causal_rfa, self.tau = reparam_proj, cuda_causal_rfa, tau
+        self.q_proj = nn.Linear(embed_dim, embed_dim, bias=True)
+        self.k_proj = nn.Linear(embed_dim, embed_dim, bias=True)
+        self.v_proj = nn.Linear(embed_dim, embed_dim, bias=True)
+        self.out_proj = nn.Linear(embed_dim, embed_dim, bias=True)
+        if reparam_proj:
+            self.sigma = Parameter(Tensor(num_heads, 1, head_dim))
+        self.reset_parameters()
+        self.upgrade_state_dict_named = upgrade_state_dict_named
+
+    def reset_parameters(self):
+        for proj in (self.q_proj, self.k_proj, self.v_proj, self.out_proj):
+            nn.init.xavier_uniform_(proj.weight, gain=1 / math.sqrt(2))
+        if self.reparam_proj:
+            nn.init.constant_(self.sigma, 1.0)
+        if self.out_proj.bias is not None:
+            nn.init.constant_(self.out_proj.bias, 0.0)
+
+    def _heads(self, t: Tensor, tgt_len: int, bsz: int) -> Tensor:
+        return t.contiguous().view(tgt_len, bsz, self.num_heads, self.head_dim)
+
+    def forward(self, x: Tensor, random_matrices: Tensor, key_padding_mask: Optional[Tensor] = None,
+                attn_mask: Optional[Tensor] = None,
+                saved_state: Optional[Dict[str, Optional[Tensor]]] = None) -> Tensor:
+        """x: [tgt_len, bsz, embed_dim]; random_matrices: [heads, proj_dim, head_dim] -> [tgt_len, bsz, embed_dim].
+
+        With ``saved_state`` (a dict, tgt_len must be 1) one decode step is taken and the
+        state under "prev_s" / "prev_z" is advanced (reference causal_attention.py:249-265).
+        """
+        tgt_len, bsz, embed_dim = x.size()
+        assert embed_dim == self.embed_dim
+        q = self._heads(self.q_proj(x), tgt_len, bsz)
+        k = self._heads(self.k_proj(x), tgt_len, bsz)
+        v = self._heads(self.v_proj(x), tgt_len, bsz)
+        w = build_random_matrices(random_matrices=random_matrices, tau=self.tau,
+                                  sigma=self.sigma if self.reparam_proj else None,
+                                  reparam_proj=self.reparam_proj)
+        if saved_state is not None:
+            assert tgt_len == 1
+            feat = 2 * self.proj_dim
+            s, z = saved_state.get("prev_s"), saved_state.get("prev_z")
+            if s is None:
+                s = torch.zeros((bsz, self.num_heads, feat, self.head_dim), device=x.device, dtype=torch.float32)
+                z = torch.zeros((bsz, self.num_heads, feat), device=x.device, dtype=torch.float32)
+            else:
+                assert z is not None
+                s = s.to(torch.float32).contiguous()
+                z = z.to(torch.float32).contiguous()
+            # feature map + state update + readout in one kernel; state advanced in place
+            attn = rfa_hip.incremental_fused(
+                q.detach().to(torch.float16).contiguous(), k.detach().to(torch.float16).contiguous(),
+                v.detach().to(torch.float16).contiguous(), w.detach().to(torch.float16).contiguous(), SCALE, s, z)
+            attn = attn.to(x.dtype).view(tgt_len, bsz, embed_dim)
+            saved_state["prev_s"], saved_state["prev_z"] = s, z
+        else:
+            phi_q = random_project(x=q, random_matrices=w)
+            phi_k = random_project(x=k, random_matrices=w)
+            if self.cuda_causal_rfa:
+                attn = cuda_causal_rfa(phi_q=phi_q, phi_k=phi_k, v=v, key_padding_mask=key_padding_mask)
+            else:
+                attn = masked_rfa(phi_q=phi_q, phi_k=phi_k, v=v, attn_mask=attn_mask,
+                                  key_padding_mask=key_padding_mask)
+        return self.out_proj(attn)

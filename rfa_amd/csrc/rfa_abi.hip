@@ -8,6 +8,8 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <vector>
 
 #include "rfa_causal.h"
 #include "rfa_decode.h"
@@ -30,6 +32,54 @@ int fail(int code, const char* fmt, ...) {
         hipError_t e_ = (expr);                                                              \
         if (e_ != hipSuccess)                                                                \
             return fail(RFA_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));         \
+    } while (0)
+
+
+// ---- optional per-kernel timing with HIP events ------------------------------------
+namespace prof {
+enum Id { SEG_STATE, CAUSAL_FWD, CAUSAL_BWD_DQ, CAUSAL_BWD_DKDV, CROSS_READOUT, CROSS_READOUT_BWD,
+          CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, ZERO_FILL, SELFTEST, COUNT };
+const char* const kNames[COUNT] = {"k_segment_state", "k_causal_fwd", "k_causal_bwd_dq", "k_causal_bwd_dkdv",
+                                   "k_cross_readout", "k_cross_readout_bwd", "k_cross_state_bwd", "k_decode_step",
+                                   "k_feature_map_fwd", "k_feature_map_bwd", "k_feature_map_dw_reduce",
+                                   "k_zero_f32", "k_selftest"};
+struct Rec { int id; hipEvent_t a, b; };
+std::mutex mu;
+bool enabled = false;
+std::vector<Rec> recs;
+std::vector<hipEvent_t> pool;
+double total_ms[COUNT] = {};
+long long calls[COUNT] = {};
+
+hipEvent_t take_event() {
+    if (!pool.empty()) { hipEvent_t e = pool.back(); pool.pop_back(); return e; }
+    hipEvent_t e = nullptr;
+    (void)hipEventCreate(&e);
+    return e;
+}
+
+// Records an event pair around one kernel launch on `st` while profiling is on.
+struct Scope {
+    int id; hipStream_t st; hipEvent_t a = nullptr;
+    Scope(int id_, hipStream_t st_) : id(id_), st(st_) {
+        if (!enabled) return;
+        std::lock_guard<std::mutex> lk(mu);
+        a = take_event();
+        if (a) (void)hipEventRecord(a, st);
+    }
+    ~Scope() {
+        if (!a) return;
+        std::lock_guard<std::mutex> lk(mu);
+        hipEvent_t b = take_event();
+        if (b) { (void)hipEventRecord(b, st); recs.push_back({id, a, b}); } else { pool.push_back(a); }
+    }
+};
+}  // namespace prof
+
+#define RFA_LAUNCH(ID, ...)                       \
+    do {                                          \
+        prof::Scope prof_scope_(prof::ID, st);    \
+        hipLaunchKernelGGL(__VA_ARGS__);          \
     } while (0)
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -101,12 +151,12 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
     if (p.nseg > 1) {
         auto kern = rfa::k_segment_state<KD, DH>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
-        hipLaunchKernelGGL(kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
+        RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     auto kern = rfa::k_causal_fwd<KD, DH, true>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
-    hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kFwdLds, st, q, k, v, out,
+    RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kFwdLds, st, q, k, v, out,
                        wsS, wsZ, T, N, p.nseg, p.seg_len);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -126,19 +176,19 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
     if (p.nseg > 1) {
         auto kern = rfa::k_segment_state<KD, DH>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
-        hipLaunchKernelGGL(kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
+        RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     {
         auto kern = rfa::k_causal_bwd_dq<KD, DH, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDqLds)) return rc;
-        hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDqLds, st, q, k, v, g,
+        RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDqLds, st, q, k, v, g,
                            dq, wsS, wsZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
     }
     {
         auto kern = rfa::k_causal_bwd_dkdv<KD, DH, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
-        hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDkLds, st, q, k, v, g,
+        RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDkLds, st, q, k, v, g,
                            dk, dv, wsR, wsr, den, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
     }
     RFA_HIP_TRY(hipGetLastError());
@@ -167,7 +217,7 @@ int launch_cross_state(const rfa::half_t* k, const rfa::half_t* v, const uint8_t
     const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
     auto kern = rfa::k_segment_state<KD, DH>;
     if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
-    hipLaunchKernelGGL(kern, dim3(N), dim3(rfa::kThreads), Cfg::kSegStateLds, st, k, v, mask, H, s, z, T, N,
+    RFA_LAUNCH(SEG_STATE, kern, dim3(N), dim3(rfa::kThreads), Cfg::kSegStateLds, st, k, v, mask, H, s, z, T, N,
                        1, 1, seg_len);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -180,7 +230,7 @@ int launch_cross_readout(const rfa::half_t* q, const float* s, const float* z, r
     const ScanPlan p = make_free_plan(T, N);
     auto kern = rfa::k_causal_fwd<KD, DH, false>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
-    hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kFwdLds, st, q,
+    RFA_LAUNCH(CROSS_READOUT, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kFwdLds, st, q,
                        (const rfa::half_t*)nullptr, (const rfa::half_t*)nullptr, out, s, z, T, N, p.nseg,
                        p.seg_len);
     RFA_HIP_TRY(hipGetLastError());
@@ -194,7 +244,7 @@ int launch_cross_readout_bwd(const rfa::half_t* q, const float* s, const float* 
     const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
     auto kern = rfa::k_causal_bwd_dq<KD, DH, false>;
     if (int rc = set_lds(kern, Cfg::kBwdDqLds)) return rc;
-    hipLaunchKernelGGL(kern, dim3(N), dim3(rfa::kThreads), Cfg::kBwdDqLds, st, q, (const rfa::half_t*)nullptr,
+    RFA_LAUNCH(CROSS_READOUT_BWD, kern, dim3(N), dim3(rfa::kThreads), Cfg::kBwdDqLds, st, q, (const rfa::half_t*)nullptr,
                        (const rfa::half_t*)nullptr, g, dq, s, z, ds, dz, (float*)nullptr, (float*)nullptr, T, N,
                        1, seg_len);
     RFA_HIP_TRY(hipGetLastError());
@@ -209,7 +259,7 @@ int launch_cross_state_bwd(const rfa::half_t* k, const rfa::half_t* v, const uin
     const ScanPlan p = make_free_plan(T, N);
     auto kern = rfa::k_causal_bwd_dkdv<KD, DH, false>;
     if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
-    hipLaunchKernelGGL(kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDkLds, st,
+    RFA_LAUNCH(CROSS_STATE_BWD, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDkLds, st,
                        (const rfa::half_t*)nullptr, k, v, (const rfa::half_t*)nullptr, dk, dv, ds, dz,
                        (const float*)nullptr, (const float*)nullptr, mask, H, T, N, p.nseg, p.seg_len);
     RFA_HIP_TRY(hipGetLastError());
@@ -223,7 +273,7 @@ int launch_decode(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t*
                   hipStream_t st) {
     const int64_t qk_step = FUSED ? N * DH : N * KD;
     for (int64_t t = 0; t < steps; ++t) {
-        hipLaunchKernelGGL((rfa::k_decode_step<KD, DH, FUSED>), dim3((unsigned)N), dim3(rfa::kThreads), 0, st,
+        RFA_LAUNCH(DECODE_STEP, (rfa::k_decode_step<KD, DH, FUSED>), dim3((unsigned)N), dim3(rfa::kThreads), 0, st,
                            q + t * qk_step, k + t * qk_step, v + t * N * DH, w, scale, H, s, z, s, z,
                            out + t * N * DH);
     }
@@ -246,7 +296,7 @@ int launch_feature_fwd(const rfa::half_t* x, const rfa::half_t* w, rfa::half_t* 
     using Cfg = rfa::FeatureCfg<D, DH>;
     auto kern = rfa::k_feature_map_fwd<D, DH>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
-    hipLaunchKernelGGL(kern, dim3((R + 63) / 64, H), dim3(rfa::kThreads), Cfg::kFwdLds, st, x, w, phi, R, H, scale);
+    RFA_LAUNCH(FEATURE_FWD, kern, dim3((R + 63) / 64, H), dim3(rfa::kThreads), Cfg::kFwdLds, st, x, w, phi, R, H, scale);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -258,9 +308,9 @@ int launch_feature_bwd(const rfa::half_t* x, const rfa::half_t* w, const rfa::ha
     const int nblk = feature_bwd_blocks(R, H);
     auto kern = rfa::k_feature_map_bwd<D, DH>;
     if (int rc = set_lds(kern, Cfg::kBwdLds)) return rc;
-    hipLaunchKernelGGL(kern, dim3(nblk, H), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, part, R, H, scale);
+    RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, part, R, H, scale);
     const int64_t elems = (int64_t)H * D * DH;
-    hipLaunchKernelGGL(rfa::k_feature_map_dw_reduce, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, st,
+    RFA_LAUNCH(FEATURE_DW_REDUCE, rfa::k_feature_map_dw_reduce, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, st,
                        part, dw, nblk, elems);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -273,7 +323,7 @@ __global__ void k_zero_f32(float* p, int64_t n) {
 }
 
 void zero_f32(float* p, int64_t n, hipStream_t st) {
-    if (n > 0) hipLaunchKernelGGL(k_zero_f32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, n);
+    if (n > 0) RFA_LAUNCH(ZERO_FILL, k_zero_f32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, n);
 }
 
 bool feature_shape_supported(int D, int d) { return (D == 32 || D == 64 || D == 128) && (d == 64 || d == 128); }
@@ -338,7 +388,7 @@ int rfa_selftest_layout(void* stream) {
     int hbad = 0;
     hipError_t e = hipMemcpyAsync(dbad, &hbad, sizeof(int), hipMemcpyHostToDevice, st);
     if (e == hipSuccess) {
-        hipLaunchKernelGGL(k_selftest, dim3(1), dim3(64), 0, st, dbad);
+        RFA_LAUNCH(SELFTEST, k_selftest, dim3(1), dim3(64), 0, st, dbad);
         e = hipMemcpyAsync(&hbad, dbad, sizeof(int), hipMemcpyDeviceToHost, st);
     }
     if (e == hipSuccess) e = hipStreamSynchronize(st);
@@ -627,6 +677,47 @@ int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi,
     RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+// ---- profiling ----------------------------------------------------------------------
+int rfa_profile_enable(int on) {
+    std::lock_guard<std::mutex> lk(prof::mu);
+    prof::enabled = on != 0;
+    return RFA_OK;
+}
+
+int rfa_profile_collect(void) {
+    std::lock_guard<std::mutex> lk(prof::mu);
+    for (auto& r : prof::recs) {
+        hipError_t e = hipEventSynchronize(r.b);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, r.a, r.b);
+        if (e != hipSuccess) return fail(RFA_ERR_HIP, "rfa_profile_collect: %s", hipGetErrorString(e));
+        prof::total_ms[r.id] += ms;
+        prof::calls[r.id] += 1;
+        prof::pool.push_back(r.a);
+        prof::pool.push_back(r.b);
+    }
+    prof::recs.clear();
+    return RFA_OK;
+}
+
+int rfa_profile_reset(void) {
+    if (int rc = rfa_profile_collect()) return rc;
+    std::lock_guard<std::mutex> lk(prof::mu);
+    for (int i = 0; i < prof::COUNT; ++i) { prof::total_ms[i] = 0.0; prof::calls[i] = 0; }
+    return RFA_OK;
+}
+
+int rfa_profile_kernel_count(void) { return prof::COUNT; }
+
+int rfa_profile_get(int index, const char** name, double* total_ms, int64_t* calls) {
+    if (index < 0 || index >= prof::COUNT) return fail(RFA_ERR_BAD_SHAPE, "rfa_profile_get: index %d out of range", index);
+    std::lock_guard<std::mutex> lk(prof::mu);
+    if (name) *name = prof::kNames[index];
+    if (total_ms) *total_ms = prof::total_ms[index];
+    if (calls) *calls = prof::calls[index];
+    return RFA_OK;
 }
 
 }  // extern "C"

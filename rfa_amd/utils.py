@@ -1,0 +1,137 @@
+"""Feature map and helpers; mirror of random_feature_attention/utils.py.
+
+``random_project`` runs the fused HIP feature-map kernel (forward and backward)
+instead of the reference's chain of ATen ops.  Inputs are computed in fp16 (the
+kernels' input type); other floating dtypes are rounded to fp16 on the way in
+and the result is returned in the caller's dtype.
+"""
+from __future__ import annotations
+
+import os
+from typing import List, NamedTuple, Optional, Tuple
+
+import numpy as np
+import torch
+from torch import Tensor
+
+from . import rfa_hip
+
+EPS = 1.0      # reference utils.py:9
+SCALE = 0.1    # reference utils.py:10
+RANDOM_MATRICES_PATH = os.path.join(os.path.dirname(__file__), "../random_matrices")
+
+
+class CrossAttentionState(NamedTuple):
+    """reference utils.py:14-18; s and z are fp32 here."""
+    s: Tensor
+    z: Tensor
+    random_matrices: Tensor
+    tau: float
+
+
+def upgrade_state_dict_named(state_dict, name):
+    """Checkpoint-upgrade hook the reference modules store (causal_attention.py:187,
+    cross_attention.py:44,243) but never define; parameter names are unchanged here,
+    so there is nothing to upgrade."""
+    return state_dict
+
+
+def get_rfa_attr(args):
+    """Defaults of the model flags (reference utils.py:20-28)."""
+    args.use_rfa = getattr(args, "use_rfa", False)
+    args.use_linfa = args.use_rfa      # attribute name the reference sets (utils.py:21)
+    args.cross_proj_dim = getattr(args, "cross_proj_dim", 64)
+    args.causal_proj_dim = getattr(args, "causal_proj_dim", 64)
+    args.cross_tau = getattr(args, "cross_tau", 1.0)
+    args.causal_tau = getattr(args, "causal_tau", 1.0)
+    args.reparam_proj = getattr(args, "reparam_proj", True)
+    args.cuda_causal_rfa = getattr(args, "cuda_causal_rfa", True)
+    return args
+
+
+def add_rfa_args(parser):
+    """Model flags (reference utils.py:31-46)."""
+    parser.add_argument("--use-rfa", action="store_true", help="use random feature attention")
+    parser.add_argument("--cross-proj-dim", type=int, metavar="N", help="projection size for cross rfa")
+    parser.add_argument("--causal-proj-dim", type=int, metavar="N", help="projection size for causal rfa")
+    parser.add_argument("--cross-tau", type=float, metavar="D", help="tau for cross rfa")
+    parser.add_argument("--causal-tau", type=float, metavar="D", help="tau for causal rfa")
+    parser.add_argument("--reparam-proj", action="store_true", help="reparameterize the random matrices")
+    parser.add_argument("--cuda-causal-rfa", action="store_true", help="use the fused kernel for causal rfa")
+    return parser
+
+
+def load_random_matrices(*, head_dim: int, proj_dim: int, dtype: torch.dtype = torch.half) -> Tensor:
+    """[num_random_matrices, proj_dim, head_dim] as a frozen Parameter (reference utils.py:49-59).
+
+    Reads ``random_matrices/{head_dim}_{proj_dim}.npy`` when it exists; otherwise the
+    matrices are generated in memory by the same recipe that wrote that file
+    (construct_random_matrices.py: Gaussian features, numpy seed 31415, 500 matrices).
+    """
+    path = os.path.join(RANDOM_MATRICES_PATH, f"{head_dim}_{proj_dim}.npy")
+    if os.path.exists(path):
+        mats = np.load(path)
+    else:
+        from .construct_random_matrices import construct_random_matrices, rrf
+        mats = construct_random_matrices(rrf, 500, head_dim=head_dim, proj_dim=proj_dim, seed=31415)
+    return torch.nn.Parameter(torch.tensor(mats, dtype=dtype), requires_grad=False)
+
+
+def sample_random_matrices(*, num_layers: int, num_heads: int, random_matrices: Tensor,
+                           is_training: bool = True):
+    """reference utils.py:62-87: training draws num_layers*num_heads distinct matrices and
+    returns one [num_heads, proj_dim, head_dim] stack per layer; evaluation returns the
+    first num_heads matrices (shared by all layers)."""
+    if is_training:
+        picks = np.random.choice(random_matrices.size(0), size=num_layers * num_heads, replace=False)
+        chosen = random_matrices[picks]
+        return [chosen[i * num_heads:(i + 1) * num_heads] for i in range(num_layers)]
+    return random_matrices[list(range(num_heads))]
+
+
+def build_random_matrices(random_matrices: Tensor, tau: float, sigma: Optional[Tensor] = None,
+                          reparam_proj: bool = False) -> Tensor:
+    """W' = (sigma * W if reparam_proj) / tau (reference utils.py:90-97)."""
+    if reparam_proj:
+        random_matrices = sigma * random_matrices
+    return random_matrices / tau
+
+
+def _normalize(x: Tensor) -> Tuple[Tensor, Tensor]:
+    """(x / (||x|| + 1e-3), ||x||) (reference utils.py:100-102)."""
+    norm = torch.linalg.vector_norm(x, ord=2, dim=-1, keepdim=True)
+    return x / (norm + 1e-3), norm
+
+
+class _FeatureMap(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x: Tensor, w: Tensor, scale: float) -> Tensor:
+        ctx.in_dtypes = (x.dtype, w.dtype)
+        ctx.scale = scale
+        xh = x.to(torch.float16).contiguous()
+        wh = w.to(torch.float16).contiguous()
+        ctx.save_for_backward(xh, wh)
+        return rfa_hip.feature_map_forward(xh, wh, scale).to(x.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_phi: Tensor):
+        xh, wh = ctx.saved_tensors
+        dx, dw = rfa_hip.feature_map_backward(xh, wh, grad_phi.to(torch.float16).contiguous(), ctx.scale)
+        return dx.to(ctx.in_dtypes[0]), dw.to(ctx.in_dtypes[1]), None
+
+
+def random_project(*, x: Tensor, random_matrices: Tensor, scale: float = SCALE) -> Tensor:
+    """phi(x) = scale * [sin(W x^), cos(W x^)] (reference utils.py:105-120).
+
+    x: [seq_len, bsz, num_heads, head_dim]; random_matrices: [num_heads, proj_dim, head_dim]
+    -> [seq_len, bsz, num_heads, 2 * proj_dim].  ``scale`` defaults to the reference's
+    constant 0.1; pass proj_dim ** -0.5 for the variance-normalised map.
+    """
+    return _FeatureMap.apply(x, random_matrices, scale)
+
+
+def normalize_attn_weights(x: Tensor, dim: int = -1, dtype: torch.dtype = torch.float32) -> Tensor:
+    """x / |sum(x)|.clamp(1e-3) in fp32 (reference utils.py:123-130)."""
+    x = x.to(torch.float32)
+    denom = x.sum(dim=dim, keepdim=True).abs().clamp(1e-3)
+    return (x / denom).to(dtype)

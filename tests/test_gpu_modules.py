@@ -1,0 +1,163 @@
+"""GPU tests of the host-side mirror of the reference API (autograd Functions and
+nn.Modules) against the oracle chain evaluated in fp32 on the CPU."""
+import pytest
+import torch
+
+from oracle import rfa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(a, b):
+    return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+def _randn(*shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=torch.float32)
+
+
+def test_rfa_apply_autograd_matches_oracle_grad_check_recipe():
+    """The recipe of the reference's grad_check.py (T=100, 5 sequences, K=128, d=64,
+    U(-.5,.5) inputs L2-normalised, seed 3) through RFA.apply + autograd."""
+    from rfa_amd import RFA
+    torch.manual_seed(3)
+    T, N, K, d = 100, 5, 128, 64
+    nrm = lambda t: t / t.norm(p=2, dim=-1, keepdim=True)
+    q, k, v = (nrm(torch.rand(T, N, n) - .5).half() for n in (K, K, d))
+    g = nrm(torch.rand(T, N, d)).half()
+    cq, ck, cv = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = RFA.apply(cq, ck, cv)
+    out.backward(g.cuda())
+    ref = O.causal_forward_cumsum(q.float(), k.float(), v.float())
+    rq, rk, rv = O.causal_backward_cumsum(q.float(), k.float(), v.float(), g.float())
+    # the reference's own pass rule: squared difference below 1e-4 everywhere
+    assert ((out.float().cpu() - ref) ** 2 < 1e-4).all()
+    for got, want in ((cq.grad, rq), (ck.grad, rk), (cv.grad, rv)):
+        assert ((got.float().cpu() - want) ** 2 < 1e-4).all()
+        assert _rel(got.float().cpu(), want) < 1e-2
+    # static-method spellings used by the reference's callers
+    assert torch.equal(RFA.forward_cuda(cq.detach(), ck.detach(), cv.detach()), out.detach())
+
+
+def test_functional_chain_with_padding_mask_and_grads():
+    """random_project -> cuda_causal_rfa with a key padding mask, gradients down to the
+    raw q, k, v and the random matrix."""
+    from rfa_amd.causal_attention import cuda_causal_rfa
+    from rfa_amd.utils import random_project
+    T, B, H, d, D = 150, 2, 2, 64, 64
+    q, k, v, g = (_randn(T, B, H, d, seed=s).half() for s in (1, 2, 3, 4))
+    W = (_randn(H, D, d, seed=5)).half()
+    mask = torch.zeros(B, T, dtype=torch.uint8)
+    mask[0, 100:] = 1
+    mask[1, :3] = 1
+    cq, ck, cv, cW = (t.cuda().requires_grad_(True) for t in (q, k, v, W))
+    attn = cuda_causal_rfa(phi_q=random_project(x=cq, random_matrices=cW),
+                           phi_k=random_project(x=ck, random_matrices=cW), v=cv,
+                           key_padding_mask=mask.cuda())
+    attn.backward(g.reshape(T, B, H * d).cuda())
+    fq, fk, fv, fW = (t.float().requires_grad_(True) for t in (q, k, v, W))
+    pq, pk = O.random_project(fq, fW), O.random_project(fk, fW)
+    pk = pk.masked_fill(mask.bool().t()[:, :, None, None], 0.0)
+    ref = O.causal_forward_chunked(pq.reshape(T, B * H, 2 * D), pk.reshape(T, B * H, 2 * D), fv.reshape(T, B * H, d))
+    ref.backward(g.float().reshape(T, B * H, d))
+    assert (attn.float().cpu().reshape(T, B * H, d) - ref.detach()).abs().max() <= 2e-3
+    for name, got, want in (("dq", cq.grad, fq.grad), ("dk", ck.grad, fk.grad), ("dv", cv.grad, fv.grad), ("dW", cW.grad, fW.grad)):
+        assert _rel(got.float().cpu(), want) <= 2e-2, (name, _rel(got.float().cpu(), want))
+
+
+def test_causal_module_decode_equals_training_forward():
+    from rfa_amd import CausalAttention
+    torch.manual_seed(0)
+    T, B, E, H, d, D = 40, 3, 128, 2, 64, 64
+    m = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half().eval()
+    with torch.no_grad():
+        m.sigma.copy_(1.0 + 0.1 * torch.randn_like(m.sigma))
+    x = torch.randn(T, B, E).cuda().half()
+    W = O.make_w(d, D, H).cuda().half()
+    with torch.no_grad():
+        full = m(x, W)
+        state = {}
+        rows = [m(x[t:t + 1], W, saved_state=state) for t in range(T)]
+    assert state["prev_s"].dtype == torch.float32 and tuple(state["prev_s"].shape) == (B, H, 2 * D, d)
+    assert tuple(state["prev_z"].shape) == (B, H, 2 * D)
+    step = torch.cat(rows, 0)
+    assert (step.float() - full.float()).abs().max().item() <= 4e-3
+    # quadratic fallback agrees wherever the denominators are equal (den >= 1 from a few steps on)
+    m.cuda_causal_rfa = False
+    with torch.no_grad():
+        quad = m(x, W, attn_mask=torch.triu(torch.full((T, T), float("-inf")), 1).cuda())
+    assert (quad[8:].float() - full[8:].float()).abs().max().item() <= 2e-2
+
+
+def test_causal_module_training_step_runs_and_matches_oracle():
+    from rfa_amd import CausalAttention
+    torch.manual_seed(1)
+    T, B, E, H, d, D = 96, 2, 128, 2, 64, 64
+    m = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half()
+    x = torch.randn(T, B, E).cuda().half().requires_grad_(True)
+    W = O.make_w(d, D, H).cuda().half()
+    y = m(x, W)
+    y.float().square().mean().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
+    # oracle chain in fp32 with the same weights
+    mf = {k_: v_.detach().float().cpu() for k_, v_ in m.state_dict().items()}
+    xf = x.detach().float().cpu()
+    lin = lambda n: xf @ mf[n + ".weight"].t() + mf[n + ".bias"]
+    q, k, v = (lin(n).reshape(T, B, H, d) for n in ("q_proj", "k_proj", "v_proj"))
+    Wp = O.build_random_matrices(W.float().cpu(), 1.0, mf["sigma"], True)
+    pq, pk = O.random_project(q, Wp), O.random_project(k, Wp)
+    att = O.causal_forward_chunked(pq.reshape(T, B * H, 2 * D), pk.reshape(T, B * H, 2 * D), v.reshape(T, B * H, d))
+    want = att.reshape(T, B, E) @ mf["out_proj.weight"].t() + mf["out_proj.bias"]
+    assert (y.detach().float().cpu() - want).abs().max().item() <= 1e-2
+
+
+def test_cross_modules_forward_backward_match_oracle():
+    from rfa_amd import CrossAttention, CrossAttentionProject
+    torch.manual_seed(2)
+    S, T, B, E, H, d, D, Lyr = 70, 33, 2, 128, 2, 64, 64, 2
+    proj = CrossAttentionProject(num_layers=Lyr, embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half().eval()
+    att = CrossAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half()
+    enc = torch.randn(S, B, E).cuda().half().requires_grad_(True)
+    qry = torch.randn(T, B, E).cuda().half().requires_grad_(True)
+    pad = torch.zeros(B, S, dtype=torch.bool)
+    pad[1, 50:] = True
+    states = proj(encoder_output=enc, key_padding_mask=pad.cuda())
+    assert len(states) == Lyr and states[0].s.dtype == torch.float32
+    assert tuple(states[0].s.shape) == (B, H, 2 * D, d) and tuple(states[0].z.shape) == (B, H, 2 * D)
+    y = att(qry, states[1])
+    g = torch.randn(T, B, E).cuda().half()
+    y.backward(g)
+    # oracle in fp32
+    L1 = proj.layers[1]
+    f = lambda t: t.detach().float().cpu()
+    encf, qryf = f(enc).requires_grad_(True), f(qry).requires_grad_(True)
+    k = (encf @ f(L1.k_proj.weight).t() + f(L1.k_proj.bias)).reshape(S, B, H, d)
+    v = (encf @ f(L1.v_proj.weight).t() + f(L1.v_proj.bias)).reshape(S, B, H, d)
+    Wp = O.build_random_matrices(f(proj.random_matrices_eval), 1.0, f(L1.sigma), True)
+    s, z = O.cross_state(O.random_project(k, Wp), v, pad.t())
+    q = (qryf @ f(att.q_proj.weight).t() + f(att.q_proj.bias)).reshape(T, B, H, d)
+    o = O.cross_readout(O.random_project(q, Wp), s, z).reshape(T, B, E)
+    want = o @ f(att.out_proj.weight).t() + f(att.out_proj.bias)
+    want.backward(f(g))
+    assert _rel(f(states[1].s), s.detach()) <= 5e-3
+    assert (f(y) - want.detach()).abs().max().item() <= 1e-2
+    assert _rel(f(enc.grad), encf.grad) <= 3e-2
+    assert _rel(f(qry.grad), qryf.grad) <= 3e-2
+
+
+def test_incremental_rfa_out_of_place_and_inplace():
+    from rfa_amd.causal_attention import incremental_rfa
+    T, B, H, K, d = 3, 2, 2, 128, 64
+    pq, pk = (0.1 * _randn(T, B, H, K, seed=8)).half().cuda(), (0.1 * _randn(T, B, H, K, seed=9)).half().cuda()
+    v = _randn(T, B, H, d, seed=10).half().cuda()
+    a1, s1, z1 = incremental_rfa(phi_q=pq[:2], phi_k=pk[:2], v=v[:2])
+    s1c, z1c = s1.clone(), z1.clone()
+    a2, s2, z2 = incremental_rfa(phi_q=pq[2:], phi_k=pk[2:], v=v[2:], s=s1, z=z1)
+    assert torch.equal(s1, s1c) and torch.equal(z1, z1c) and s2.data_ptr() != s1.data_ptr()
+    a3, s3, z3 = incremental_rfa(phi_q=pq[2:], phi_k=pk[2:], v=v[2:], s=s1, z=z1, inplace=True)
+    assert s3.data_ptr() == s1.data_ptr() and torch.equal(s3, s2) and torch.equal(a2, a3)
+    want, ws, wz = O.causal_forward_loop(pq.float().cpu().reshape(T, B * H, K), pk.float().cpu().reshape(T, B * H, K),
+                                         v.float().cpu().reshape(T, B * H, d))
+    got = torch.cat([a1, a2], 0).float().cpu().reshape(T, B * H, d)
+    assert (got - want).abs().max().item() <= 2e-3

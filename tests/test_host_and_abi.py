@@ -1,0 +1,165 @@
+"""CPU-only tests: the C-ABI library loads and exports every declared symbol,
+argument validation happens before any GPU work, and the host-side mirror of the
+reference API has the reference's names, defaults and parameter layout."""
+import argparse
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from rfa_amd import _lib
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _lib.declared_symbols()
+    assert len(declared) >= 19
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert set(declared) == set(_lib.SIGNATURES)
+    assert lib.rfa_version() >= 100
+
+
+def test_shape_support_and_workspace_queries():
+    lib = _lib.load()
+    assert lib.rfa_shape_supported(128, 64) == 1 and lib.rfa_shape_supported(256, 128) == 1
+    assert lib.rfa_shape_supported(100, 64) == 0 and lib.rfa_shape_supported(128, 48) == 0
+    assert lib.rfa_feature_map_supported(64, 64) == 1 and lib.rfa_feature_map_supported(48, 64) == 0
+    assert lib.rfa_causal_num_segments(1024, 64) >= 1
+    assert lib.rfa_causal_num_segments(64, 1) == 1          # one chunk cannot be split
+    assert lib.rfa_causal_forward_workspace_bytes(0, 4, 128, 64) == 0
+    fw = lib.rfa_causal_forward_workspace_bytes(1024, 64, 128, 64)
+    bw = lib.rfa_causal_backward_workspace_bytes(1024, 64, 128, 64)
+    assert bw > fw >= 0 and bw >= 2 * 1024 * 64 * 4
+    assert lib.rfa_feature_map_backward_workspace_bytes(8192, 8, 64, 64) >= 8 * 64 * 64 * 4
+
+
+def test_errors_are_reported_before_any_gpu_work():
+    lib = _lib.load()
+    rc = lib.rfa_causal_forward(None, None, None, None, 16, 2, 100, 64, None, 0, None)
+    assert rc == -3 and b"K=100" in lib.rfa_last_error()
+    rc = lib.rfa_causal_forward(None, None, None, None, 16, 2, 128, 64, None, 0, None)
+    assert rc == -1
+    rc = lib.rfa_causal_forward(None, None, None, None, -1, 2, 128, 64, None, 0, None)
+    assert rc == -2
+    buf = ctypes.create_string_buffer(64)
+    odd = ctypes.addressof(buf) + 1
+    rc = lib.rfa_causal_forward(odd, odd, odd, odd, 16, 2, 128, 64, None, 0, None)
+    assert rc == -4
+    al = (ctypes.addressof(buf) + 15) & ~15
+    rc = lib.rfa_causal_backward(al, al, al, al, al, al, al, 16, 2, 128, 64, None, 0, None)
+    assert rc == -5 and b"workspace" in lib.rfa_last_error()
+    assert lib.rfa_causal_forward(None, None, None, None, 0, 2, 128, 64, None, 0, None) == 0   # empty input
+    assert lib.rfa_feature_map_forward(None, None, None, 4, 2, 48, 64, 0.1, None) == -3
+    assert lib.rfa_incremental(None, None, None, None, None, None, 1, 2, 128, 64, None) == -1
+    with pytest.raises(_lib.RfaHipError):
+        _lib.check(-3)
+
+
+def test_host_wrappers_reject_cpu_and_wrong_dtype():
+    from rfa_amd import RFA, rfa_hip
+    q = torch.zeros(4, 2, 128, dtype=torch.float16)
+    v = torch.zeros(4, 2, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        rfa_hip.forward(q, q, v)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        RFA.apply(q, q, v)
+    with pytest.raises(RuntimeError):
+        rfa_hip.feature_map_forward(torch.zeros(2, 1, 2, 64, dtype=torch.float16), torch.zeros(2, 64, 64, dtype=torch.float16), 0.1)
+
+
+def test_formula_statements_match_oracle_on_cpu():
+    """RFA.forward_torch / backward_torch / reverse_cumsum are kept as API; they are
+    plain formulas and must agree with the oracle."""
+    from oracle import rfa_oracle as O
+    from rfa_amd.rfa import RFA, reverse_cumsum, rfa_debug
+    g = torch.Generator().manual_seed(0)
+    q, k = (0.1 * torch.randn(9, 2, 8, generator=g, dtype=torch.float64) for _ in range(2))
+    k = k.abs()
+    v, go = (torch.randn(9, 2, 4, generator=g, dtype=torch.float64) for _ in range(2))
+    assert torch.allclose(RFA.forward_torch(q, k, v), O.causal_forward_loop(q, k, v)[0], atol=1e-12)
+    assert torch.allclose(rfa_debug(q, k, v), O.causal_forward_quadratic(q, k, v), atol=1e-12)
+    for a, b in zip(RFA.backward_torch(q, k, v, go), O.causal_backward_chunked(q, k, v, go, chunk=4)):
+        assert torch.allclose(a, b, atol=1e-11)
+    x = torch.arange(6.0).reshape(3, 2)
+    assert torch.equal(reverse_cumsum(x, 0), torch.tensor([[6.0, 9.0], [6.0, 8.0], [4.0, 5.0]]))
+
+
+def test_module_parameter_names_and_defaults():
+    from rfa_amd import CausalAttention, CrossAttention, CrossAttentionProject, CrossAttentionState
+    from rfa_amd.utils import EPS, SCALE, add_rfa_args, get_rfa_attr
+    assert EPS == 1.0 and SCALE == 0.1
+    m = CausalAttention(embed_dim=128, num_heads=2, head_dim=64, proj_dim=64)
+    assert sorted(m.state_dict()) == sorted(
+        [f"{p}.{w}" for p in ("q_proj", "k_proj", "v_proj", "out_proj") for w in ("weight", "bias")] + ["sigma"])
+    assert tuple(m.sigma.shape) == (2, 1, 64) and torch.all(m.sigma == 1) and torch.all(m.out_proj.bias == 0)
+    assert m.tau == 1.0 and m.reparam_proj and m.cuda_causal_rfa and callable(m.upgrade_state_dict_named)
+    assert "sigma" not in CausalAttention(embed_dim=128, num_heads=2, head_dim=64, proj_dim=64,
+                                          reparam_proj=False).state_dict()
+    c = CrossAttention(embed_dim=128, num_heads=2, head_dim=64, proj_dim=64)
+    assert sorted(c.state_dict()) == ["out_proj.bias", "out_proj.weight", "q_proj.bias", "q_proj.weight"]
+    assert torch.all(c.q_proj.bias == 0)
+    p = CrossAttentionProject(num_layers=3, embed_dim=128, num_heads=2, head_dim=64, proj_dim=32)
+    keys = set(p.state_dict())
+    assert {"layers.0.k_proj.weight", "layers.2.v_proj.bias", "layers.1.sigma", "random_matrices",
+            "random_matrices_eval"} <= keys
+    assert tuple(p.random_matrices.shape) == (500, 32, 64) and p.random_matrices.dtype == torch.float16
+    assert tuple(p.random_matrices_eval.shape) == (2, 32, 64) and not p.random_matrices_eval.requires_grad
+    assert CrossAttentionState._fields == ("s", "z", "random_matrices", "tau")
+    args = get_rfa_attr(argparse.Namespace())
+    assert (args.cross_proj_dim, args.causal_proj_dim, args.cross_tau, args.causal_tau) == (64, 64, 1.0, 1.0)
+    assert args.reparam_proj and args.cuda_causal_rfa and not args.use_rfa
+    ns = add_rfa_args(argparse.ArgumentParser()).parse_args(["--use-rfa", "--causal-proj-dim", "128"])
+    assert ns.use_rfa and ns.causal_proj_dim == 128
+
+
+def test_sample_and_build_random_matrices():
+    from rfa_amd.utils import build_random_matrices, sample_random_matrices
+    mats = torch.arange(20 * 2 * 3, dtype=torch.float32).reshape(20, 2, 3)
+    np.random.seed(0)
+    per_layer = sample_random_matrices(num_layers=3, num_heads=4, random_matrices=mats, is_training=True)
+    assert len(per_layer) == 3 and all(tuple(m.shape) == (4, 2, 3) for m in per_layer)
+    firsts = torch.cat(per_layer)[:, 0, 0]
+    assert len(set(firsts.tolist())) == 12                    # drawn without replacement
+    assert torch.equal(sample_random_matrices(num_layers=3, num_heads=4, random_matrices=mats, is_training=False), mats[:4])
+    W = torch.ones(2, 3, 4)
+    sigma = torch.tensor([[[1.0, 2.0, 3.0, 4.0]], [[5.0, 6.0, 7.0, 8.0]]])
+    out = build_random_matrices(W, 2.0, sigma, True)
+    assert torch.equal(out[1, 2], torch.tensor([2.5, 3.0, 3.5, 4.0]))
+    assert torch.equal(build_random_matrices(W, 4.0), W / 4.0)
+
+
+def test_masked_rfa_quadratic_form_on_cpu():
+    """masked_rfa is ATen-only (as in the reference); check its normaliser and masks."""
+    from rfa_amd.causal_attention import masked_rfa
+    g = torch.Generator().manual_seed(1)
+    T, B, H, K, d = 6, 2, 1, 8, 4
+    pq, pk = (torch.rand(T, B, H, K, generator=g) for _ in range(2))
+    v = torch.randn(T, B, H, d, generator=g)
+    causal = torch.triu(torch.full((T, T), float("-inf")), 1)
+    pad = torch.zeros(B, T, dtype=torch.uint8)
+    pad[1, 4:] = 1
+    out = masked_rfa(phi_q=pq, phi_k=pk, v=v, key_padding_mask=pad, attn_mask=causal)
+    assert tuple(out.shape) == (T, B, H * d)
+    for b in range(B):
+        for t in range(T):
+            keys = [s for s in range(t + 1) if not pad[b, s]]
+            wts = torch.stack([(pq[t, b, 0] * pk[s, b, 0]).sum() for s in keys])
+            want = (wts[:, None] * torch.stack([v[s, b, 0] for s in keys])).sum(0) / wts.sum().abs().clamp(1e-3)
+            assert torch.allclose(out[t, b], want, atol=1e-5)
+    assert torch.equal(masked_rfa(phi_q=pq, phi_k=pk, v=v, key_padding_mask=torch.tensor(0), attn_mask=causal),
+                       masked_rfa(phi_q=pq, phi_k=pk, v=v, attn_mask=causal))
+
+
+def test_random_matrix_generators():
+    from rfa_amd.construct_random_matrices import construct_random_matrices, orf, rrf, softmax_kernel_error
+    a = construct_random_matrices(rrf, 3, head_dim=8, proj_dim=16, seed=31415)
+    b = construct_random_matrices(rrf, 3, head_dim=8, proj_dim=16, seed=31415)
+    assert a.shape == (3, 16, 8) and np.array_equal(a, b)
+    np.random.seed(1)
+    o = orf(head_dim=16, proj_dim=16)
+    unit = o / np.linalg.norm(o, axis=1, keepdims=True)
+    assert np.allclose(unit @ unit.T, np.eye(16), atol=1e-10)      # orthogonal directions
+    np.random.seed(2)
+    assert softmax_kernel_error(16, 2048, rrf(head_dim=16, proj_dim=2048), iters=5) < 0.15
