@@ -149,7 +149,7 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
     float* wsZ = reinterpret_cast<float*>(ws + wl.Z);
     if (p.nseg > 1) {
-        auto kern = rfa::k_segment_state<KD, DH>;
+        auto kern = rfa::k_segment_state<KD, DH, true>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, T, N, p.nseg, p.nseg - 1, p.seg_len);
@@ -174,7 +174,7 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
     float* den = reinterpret_cast<float*>(ws + wl.den);
     float* gz = reinterpret_cast<float*>(ws + wl.gz);
     if (p.nseg > 1) {
-        auto kern = rfa::k_segment_state<KD, DH>;
+        auto kern = rfa::k_segment_state<KD, DH, false>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, T, N, p.nseg, p.nseg - 1, p.seg_len);
@@ -215,7 +215,7 @@ int launch_cross_state(const rfa::half_t* k, const rfa::half_t* v, const uint8_t
                        float* z, int T, int N, hipStream_t st) {
     using Cfg = rfa::CausalCfg<KD, DH>;
     const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
-    auto kern = rfa::k_segment_state<KD, DH>;
+    auto kern = rfa::k_segment_state<KD, DH, false>;
     if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
     RFA_LAUNCH(SEG_STATE, kern, dim3(N), dim3(rfa::kThreads), Cfg::kSegStateLds, st, k, v, mask, H, s, z, T, N,
                        1, 1, seg_len);
@@ -372,6 +372,20 @@ __global__ void k_selftest(int* bad) {
 extern "C" {
 
 int rfa_version(void) { return 100; }
+
+#ifdef RFA_PHASE_TIMING
+// tuning builds only: out[32] receives the accumulated phase cycle counters; reset != 0 clears them
+int rfa_debug_phase_ticks(unsigned long long* out, int reset) {
+    if (reset) {
+        unsigned long long z[32] = {};
+        RFA_HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(rfa::g_phase_ticks), z, sizeof(z)));
+        return RFA_OK;
+    }
+    RFA_HIP_TRY(hipDeviceSynchronize());
+    RFA_HIP_TRY(hipMemcpyFromSymbol(out, HIP_SYMBOL(rfa::g_phase_ticks), 32 * sizeof(unsigned long long)));
+    return RFA_OK;
+}
+#endif
 
 const char* rfa_last_error(void) { return g_err; }
 

@@ -35,8 +35,8 @@ template <int KD, int DH>
 struct CausalCfg {
     static_assert(KD % 64 == 0 && DH % 64 == 0, "KD and DH must be multiples of 64");
     static constexpr int C = kChunk;
-    static constexpr int LDQ = KD + 16;   // +16 halves: conflict-free transposing reads
-    static constexpr int LDV = DH + 16;
+    static constexpr int LDQ = KD + lds_pad(KD);
+    static constexpr int LDV = DH + lds_pad(DH);
     static constexpr int LDA = C + 8;
     static constexpr int DS = DH / 4;     // value columns owned by one wave
     static constexpr int KS = KD / 4;     // feature rows owned by one wave
@@ -56,14 +56,21 @@ struct CausalCfg {
 // state tensors.  pad_mask ([B, T] bytes, 1 = padded key, may be NULL) zeroes
 // phi_k rows (reference: cross_attention.py:97-100).
 // ---------------------------------------------------------------------------
-template <int KD, int DH>
+//
+// FRAG selects the layout of the totals in wsS: false = row-major [KD][DH] per
+// (sequence, segment) (read by the backward sweep and by cross attention);
+// true = accumulator-fragment order [wave][kt][ct][lane][4], which the forward
+// scan, owning the same tiles, reads back with one 16-byte load per tile.
+// z is accumulated on the MFMA too: z tile (m=k) = K^T 1 with an all-ones operand;
+// wave w owns the feature tiles kt in [w*NKTW, (w+1)*NKTW).
+template <int KD, int DH, bool FRAG>
 __global__ __launch_bounds__(kThreads) void k_segment_state(
     const half_t* __restrict__ k, const half_t* __restrict__ v, const uint8_t* __restrict__ pad_mask,
     int H, float* __restrict__ wsS, float* __restrict__ wsZ, int T, int N, int nseg, int nseg_out,
     int seg_len) {
     using Cfg = CausalCfg<KD, DH>;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, DS = Cfg::DS;
-    constexpr int NKT = KD / 16, NCT = DS / 16;
+    constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / 4;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Ks = reinterpret_cast<half_t*>(smem_raw);
     half_t* Vs = Ks + C * LDQ;
@@ -84,7 +91,10 @@ __global__ __launch_bounds__(kThreads) void k_segment_state(
     for (int a = 0; a < NKT; ++a)
 #pragma unroll
         for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
-    float zreg = 0.f;
+    f4 zacc[NKTW];
+#pragma unroll
+    for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
+    const h8 ones = h8_ones();
 
     ChunkRegs<KD> rk;
     ChunkRegs<DH> rv;
@@ -113,23 +123,34 @@ __global__ __launch_bounds__(kThreads) void k_segment_state(
 #pragma unroll
                 for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, bv[ct][js], S[kt][ct]);
             }
-        if (tid < KD) {
-            float s = 0.f;
-#pragma unroll 8
-            for (int j = 0; j < C; ++j) s += (float)Ks[j * LDQ + tid];
-            zreg += s;
-        }
+#pragma unroll
+        for (int a = 0; a < NKTW; ++a)
+#pragma unroll
+            for (int js = 0; js < 2; ++js)
+                zacc[a] = mfma32(col8(Ks, LDQ, js * 32, 16 * (w * NKTW + a), lane), ones, zacc[a]);
         __syncthreads();
     }
     float* so = wsS + ((int64_t)(n * nseg + seg) * KD) * DH;
+    if (FRAG) {
+        f4* sf = reinterpret_cast<f4*>(so) + (int64_t)w * NKT * NCT * 64;
 #pragma unroll
-    for (int kt = 0; kt < NKT; ++kt)
+        for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-        for (int ct = 0; ct < NCT; ++ct)
+            for (int ct = 0; ct < NCT; ++ct) sf[(kt * NCT + ct) * 64 + lane] = S[kt][ct];
+    } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                so[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row] = S[kt][ct][e];
-    if (tid < KD) wsZ[(int64_t)(n * nseg + seg) * KD + tid] = zreg;
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    so[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row] = S[kt][ct][e];
+    }
+    if (row == 0) {
+#pragma unroll
+        for (int a = 0; a < NKTW; ++a)
+            *reinterpret_cast<f4*>(wsZ + (int64_t)(n * nseg + seg) * KD + 16 * (w * NKTW + a) + 4 * G) = zacc[a];
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -148,7 +169,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
     int N, int nseg, int seg_len) {
     using Cfg = CausalCfg<KD, DH>;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = Cfg::DS;
-    constexpr int NKT = KD / 16, NCT = DS / 16;
+    constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / 4;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
     half_t* Ks = Qs + C * LDQ;
@@ -169,27 +190,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
     const half_t* vb = v + (int64_t)n * DH;
     half_t* ob = out + (int64_t)n * DH;
 
-    // carried state = sum of the totals of all earlier segments
-    f4 S[NKT][NCT];
-#pragma unroll
-    for (int a = 0; a < NKT; ++a)
-#pragma unroll
-        for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
-    float zreg = 0.f;
-    const int n_states = CAUSAL ? seg : 1;          // states to sum
-    const int state_stride = CAUSAL ? nseg : 1;     // states stored per sequence
-    for (int s = 0; s < n_states; ++s) {
-        const float* si = wsS + ((int64_t)(n * state_stride + s) * KD) * DH;
-#pragma unroll
-        for (int kt = 0; kt < NKT; ++kt)
-#pragma unroll
-            for (int ct = 0; ct < NCT; ++ct)
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    S[kt][ct][e] += si[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row];
-        if (tid < KD) zreg += wsZ[(int64_t)(n * state_stride + s) * KD + tid];
-    }
-
+    RFA_TICK_INIT();
     ChunkRegs<KD> rq, rk;
     ChunkRegs<DH> rv;
     chunk_g2r<KD>(rq, qb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
@@ -198,14 +199,55 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
         chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
     }
 
+    // carried state = sum of the totals of all earlier segments (causal: stored in
+    // fragment order by k_segment_state<FRAG=true>; cross: one row-major state)
+    f4 S[NKT][NCT];
+#pragma unroll
+    for (int a = 0; a < NKT; ++a)
+#pragma unroll
+        for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
+    f4 zacc[NKTW];      // z for feature tiles kt = w*NKTW + a, element k = 16kt + 4G + e
+#pragma unroll
+    for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
+    const h8 ones = h8_ones();
+    const int n_states = CAUSAL ? seg : 1;          // states to sum
+    const int state_stride = CAUSAL ? nseg : 1;     // states stored per sequence
+    for (int s = 0; s < n_states; ++s) {
+        const float* si = wsS + ((int64_t)(n * state_stride + s) * KD) * DH;
+        if (CAUSAL) {
+            const f4* sf = reinterpret_cast<const f4*>(si) + (int64_t)w * NKT * NCT * 64;
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct) S[kt][ct] += sf[(kt * NCT + ct) * 64 + lane];
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        S[kt][ct][e] += si[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row];
+        }
+#pragma unroll
+        for (int a = 0; a < NKTW; ++a)
+            zacc[a] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * state_stride + s) * KD + 16 * (w * NKTW + a) + 4 * G);
+    }
+
+    RFA_TICK(0);
     for (int t0 = t_begin; t0 < t_end; t0 += C) {
         chunk_r2s<KD>(rq, Qs, LDQ, tid);
         if (CAUSAL) {
             chunk_r2s<KD>(rk, Ks, LDQ, tid);
             chunk_r2s<DH>(rv, Vs, LDV, tid);
         }
-        if (tid < KD) zs[tid] = zreg;
+        if (row == 0) {
+#pragma unroll
+            for (int a = 0; a < NKTW; ++a) *reinterpret_cast<f4*>(zs + 16 * (w * NKTW + a) + 4 * G) = zacc[a];
+        }
+        RFA_TICK(1);
         __syncthreads();
+        RFA_TICK(2);
         if (t0 + C < t_end) {
             const int rows = t_end - t0 - C;
             chunk_g2r<KD>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
@@ -215,6 +257,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
             }
         }
 
+        RFA_TICK(3);
         // ---- phase A: wave w computes rows i in [16w, 16w+16) of A (as A^T tiles, m=j, n=i)
         {
             f4 at[4];
@@ -224,20 +267,21 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
             for (int ks = 0; ks < (CAUSAL ? KD / 32 : 0); ++ks) {
                 h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt)
-                    if (jt <= w) at[jt] = mfma32(row8(Ks, LDQ, 16 * jt + row, ks * 32, G), bq, at[jt]);
+                for (int jt = 0; jt < 4; ++jt)   // all four tiles: branch-free, wave 3 needs them anyway
+                    at[jt] = mfma32(row8(Ks, LDQ, 16 * jt + row, ks * 32, G), bq, at[jt]);
             }
             float part = 0.f;
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) {
-                if (jt == w) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (4 * G + e > row) at[jt][e] = 0.f;   // keep j <= i
+                for (int e = 0; e < 4; ++e) {   // keep j <= i
+                    const bool keep = (jt < w) || (jt == w && 4 * G + e <= row);
+                    at[jt][e] = keep ? at[jt][e] : 0.f;
                 }
-                if (jt <= w) part += at[jt][0] + at[jt][1] + at[jt][2] + at[jt][3];
+                part += at[jt][0] + at[jt][1] + at[jt][2] + at[jt][3];
             }
             // + q_i . z  (this lane covers features [G*KD/4, (G+1)*KD/4))
+            f4 qz4 = f4_zero();
 #pragma unroll
             for (int kk = 0; kk < KD / 4; kk += 8) {
                 h8 qv = *reinterpret_cast<const h8*>(Qs + (16 * w + row) * LDQ + G * (KD / 4) + kk);
@@ -245,21 +289,22 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
                 f4 z1 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk + 4);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    part += (float)qv[e] * z0[e];
-                    part += (float)qv[4 + e] * z1[e];
+                    qz4[e] += (float)qv[e] * z0[e];
+                    qz4[e] += (float)qv[4 + e] * z1[e];
                 }
             }
+            part += (qz4[0] + qz4[1]) + (qz4[2] + qz4[3]);
             part = sum_over_groups(part);
             if (G == 0) dens[16 * w + row] = fmaxf(CAUSAL ? part : fabsf(part), 1.0f);
             if (CAUSAL) {
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt) {
-                    h4 hv = (jt <= w) ? to_h4(at[jt]) : h4_zero();
-                    *reinterpret_cast<h4*>(As + (16 * w + row) * LDA + 16 * jt + 4 * G) = hv;
-                }
+                for (int jt = 0; jt < 4; ++jt)
+                    *reinterpret_cast<h4*>(As + (16 * w + row) * LDA + 16 * jt + 4 * G) = to_h4(at[jt]);
             }
         }
+        RFA_TICK(4);
         __syncthreads();
+        RFA_TICK(5);
 
         // ---- phase B: out^T tiles (m=c, n=i) for this wave's value columns, then state update
         {
@@ -271,6 +316,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
                     for (int js = 0; js < 2; ++js) av[ct][js] = col8(Vs, LDV, js * 32, w * DS + 16 * ct, lane);
             }
 
+            RFA_TICK(6);
             f4 acc[4][NCT];
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
@@ -294,12 +340,12 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
                 for (int it = 0; it < 4; ++it) {
                     h8 bq = row_split8(Qs, LDQ, 16 * it + row, ks * 32, G);
 #pragma unroll
-                    for (int ct = 0; ct < NCT; ++ct) {
-                        acc[it][ct] = mfma32(hi[ct], bq, acc[it][ct]);
-                        acc[it][ct] = mfma32(lo[ct], bq, acc[it][ct]);
-                    }
+                    for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = mfma32(hi[ct], bq, acc[it][ct]);
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = mfma32(lo[ct], bq, acc[it][ct]);
                 }
             }
+            RFA_TICK(7);
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const int i = 16 * it + row;
@@ -313,6 +359,7 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
                     }
                 }
             }
+            RFA_TICK(8);
             if (CAUSAL) {
                 // S (m=k, n=c) += K^T V
 #pragma unroll
@@ -323,15 +370,16 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
 #pragma unroll
                         for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, av[ct][js], S[kt][ct]);
                     }
-                if (tid < KD) {
-                    float s = 0.f;
-#pragma unroll 8
-                    for (int j = 0; j < C; ++j) s += (float)Ks[j * LDQ + tid];
-                    zreg += s;
-                }
+#pragma unroll
+                for (int a = 0; a < NKTW; ++a)
+#pragma unroll
+                    for (int js = 0; js < 2; ++js)
+                        zacc[a] = mfma32(col8(Ks, LDQ, js * 32, 16 * (w * NKTW + a), lane), ones, zacc[a]);
             }
         }
+        RFA_TICK(9);
         __syncthreads();
+        RFA_TICK(10);
     }
 }
 
@@ -386,7 +434,11 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
     for (int a = 0; a < NCT; ++a)
 #pragma unroll
         for (int b = 0; b < NKT; ++b) { ST[a][b] = f4_zero(); RT[a][b] = f4_zero(); }
-    float zreg = 0.f, rreg = 0.f;
+    // z and dr for this wave's feature slice, as MFMA tiles (m=k): element k = w*KS + 16kt + 4G + e
+    f4 zacc[NKT], racc[NKT];
+#pragma unroll
+    for (int b = 0; b < NKT; ++b) { zacc[b] = f4_zero(); racc[b] = f4_zero(); }
+    const h8 ones = h8_ones();
     const int n_states = CAUSAL ? seg : 1;
     const int state_stride = CAUSAL ? nseg : 1;
     for (int s = 0; s < n_states; ++s) {
@@ -398,7 +450,9 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
                 f4 x = *reinterpret_cast<const f4*>(si + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
                 ST[ct][kt] += x;
             }
-        if (tid < KD) zreg += wsZ[(int64_t)(n * state_stride + s) * KD + tid];
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+            zacc[kt] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * state_stride + s) * KD + w * KS + 16 * kt + 4 * G);
     }
 
     ChunkRegs<KD> rq, rk;
@@ -420,7 +474,10 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
             chunk_r2s<KD>(rk, Ks, LDQ, tid);
             chunk_r2s<DH>(rv, Vs, LDV, tid);
         }
-        if (tid < KD) zs[tid] = zreg;
+        if (row == 0) {
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) *reinterpret_cast<f4*>(zs + w * KS + 16 * kt + 4 * G) = zacc[kt];
+        }
         __syncthreads();
         if (t0 + C < t_end) {
             const int rows = t_end - t0 - C;
@@ -443,32 +500,28 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
             for (int ks = 0; ks < (CAUSAL ? KD / 32 : 0); ++ks) {
                 h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt)
-                    if (jt <= w) at[jt] = mfma32(row8(Ks, LDQ, 16 * jt + row, ks * 32, G), bq, at[jt]);
+                for (int jt = 0; jt < 4; ++jt)   // all four tiles, branch-free
+                    at[jt] = mfma32(row8(Ks, LDQ, 16 * jt + row, ks * 32, G), bq, at[jt]);
             }
 #pragma unroll
             for (int cs = 0; cs < (CAUSAL ? DH / 32 : 0); ++cs) {
                 h8 bg = row8(Gs, LDV, 16 * w + row, cs * 32, G);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt)
-                    if (jt <= w) xt[jt] = mfma32(row8(Vs, LDV, 16 * jt + row, cs * 32, G), bg, xt[jt]);
+                    xt[jt] = mfma32(row8(Vs, LDV, 16 * jt + row, cs * 32, G), bg, xt[jt]);
             }
             float part_d = 0.f, part_e = 0.f;
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) {
-                if (jt == w) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (4 * G + e > row) at[jt][e] = 0.f;
-                }
-                if (jt <= w) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        part_d += at[jt][e];
-                        part_e += at[jt][e] * xt[jt][e];
-                    }
+                for (int e = 0; e < 4; ++e) {   // keep j <= i
+                    const bool keep = (jt < w) || (jt == w && 4 * G + e <= row);
+                    at[jt][e] = keep ? at[jt][e] : 0.f;
+                    part_d += at[jt][e];
+                    part_e += at[jt][e] * xt[jt][e];
                 }
             }
+            f4 qz4 = f4_zero();
 #pragma unroll
             for (int kk = 0; kk < KD / 4; kk += 8) {
                 h8 qv = *reinterpret_cast<const h8*>(Qs + (16 * w + row) * LDQ + G * (KD / 4) + kk);
@@ -476,10 +529,11 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
                 f4 z1 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk + 4);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    part_d += (float)qv[e] * z0[e];
-                    part_d += (float)qv[4 + e] * z1[e];
+                    qz4[e] += (float)qv[e] * z0[e];
+                    qz4[e] += (float)qv[4 + e] * z1[e];
                 }
             }
+            part_d += (qz4[0] + qz4[1]) + (qz4[2] + qz4[3]);
             part_d = sum_over_groups(part_d);
             part_e = sum_over_groups(part_e);
             if (G == 0) {
@@ -500,10 +554,9 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
                 for (int it = 0; it < 4; ++it) {
                     h8 bg = row_split8(Gs, LDV, 16 * it + row, cs * 32, G);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) {
-                        yt[kt][it] = mfma32(hi[kt], bg, yt[kt][it]);
-                        yt[kt][it] = mfma32(lo[kt], bg, yt[kt][it]);
-                    }
+                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(hi[kt], bg, yt[kt][it]);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(lo[kt], bg, yt[kt][it]);
                 }
             }
             float e2[4] = {0.f, 0.f, 0.f, 0.f};
@@ -550,13 +603,11 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
             const float gzi = gzs[i];
 #pragma unroll
             for (int jt = 0; jt < (CAUSAL ? 4 : 0); ++jt) {
-                h4 pv = h4_zero();
-                if (jt <= w) {
+                h4 pv;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int j = 16 * jt + 4 * G + e;
-                        pv[e] = (j <= i) ? (half_t)(xt[jt][e] * inv + gzi) : (half_t)0.f;
-                    }
+                for (int e = 0; e < 4; ++e) {
+                    const int j = 16 * jt + 4 * G + e;
+                    pv[e] = (j <= i) ? (half_t)(xt[jt][e] * inv + gzi) : (half_t)0.f;
                 }
                 *reinterpret_cast<h4*>(Ps + i * LDA + 16 * jt + 4 * G) = pv;
             }
@@ -612,6 +663,17 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
                 h8 qf[NKT];   // Q column fragments
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt) qf[kt] = col8(Qs, LDQ, js * 32, w * KS + 16 * kt, lane);
+                // dr (m=k) += Q^T gz, z (m=k) += K^T 1: the vector operand is the same for all n
+                h8 ghi, glo;
+                f8_to_operand(*reinterpret_cast<const f4*>(gzs + js * 32 + 8 * G),
+                              *reinterpret_cast<const f4*>(gzs + js * 32 + 8 * G + 4), ghi, glo);
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) {
+                    racc[kt] = mfma32(qf[kt], ghi, racc[kt]);
+                    if (CAUSAL) zacc[kt] = mfma32(kf[kt][js], ones, zacc[kt]);
+                }
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt], glo, racc[kt]);
 #pragma unroll
                 for (int ct = 0; ct < NCT; ++ct) {
                     h8 gf = col8(Gs, LDV, js * 32, 16 * ct, lane);
@@ -624,16 +686,6 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
                     }
                 }
             }
-            if (tid < KD) {
-                float sz = 0.f, sr = 0.f;
-#pragma unroll 8
-                for (int j = 0; j < C; ++j) {
-                    if (CAUSAL) sz += (float)Ks[j * LDQ + tid];
-                    sr += (float)Qs[j * LDQ + tid] * gzs[j];
-                }
-                zreg += sz;
-                rreg += sr;
-            }
         }
         __syncthreads();
     }
@@ -645,7 +697,11 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
 #pragma unroll
             for (int kt = 0; kt < NKT; ++kt)
                 *reinterpret_cast<f4*>(ro + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G) = RT[ct][kt];
-        if (tid < KD) wsr[(int64_t)(n * nseg + seg) * KD + tid] = rreg;
+        if (row == 0) {
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+                *reinterpret_cast<f4*>(wsr + (int64_t)(n * nseg + seg) * KD + w * KS + 16 * kt + 4 * G) = racc[kt];
+        }
     }
 }
 
@@ -704,7 +760,9 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
     for (int a = 0; a < NKT2; ++a)
 #pragma unroll
         for (int b = 0; b < NCT2; ++b) RR[a][b] = f4_zero();
-    float rreg = 0.f;
+    f4 racc[NKT];     // r for this wave's feature slice (m=k tiles): k = w*KS + 16kt + 4G + e
+#pragma unroll
+    for (int b = 0; b < NKT; ++b) racc[b] = f4_zero();
     const uint8_t* mrow = (!CAUSAL && pad_mask) ? pad_mask + (int64_t)(n / H) * T : nullptr;
     const int s_first = CAUSAL ? seg + 1 : 0, s_last = CAUSAL ? nseg : 1;
     const int state_stride = CAUSAL ? nseg : 1;
@@ -722,7 +780,9 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     RR[kt][ct][e] += ri[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row];
-        if (tid < KD) rreg += wsr[(int64_t)(n * state_stride + s) * KD + tid];
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+            racc[kt] += *reinterpret_cast<const f4*>(wsr + (int64_t)(n * state_stride + s) * KD + w * KS + 16 * kt + 4 * G);
     }
 
     ChunkRegs<KD> rq, rk;
@@ -759,7 +819,10 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
             chunk_r2s_scaled<DH>(rg, inv_den, Gs, LDV, tid);
             if (tid < C) gzs[tid] = gz_next;
         }
-        if (tid < KD) rs[tid] = rreg;
+        if (row == 0) {
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) *reinterpret_cast<f4*>(rs + w * KS + 16 * kt + 4 * G) = racc[kt];
+        }
         __syncthreads();
         if (ci > 0) prefetch(t0 - C);
 
@@ -772,30 +835,26 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
             for (int ks = 0; ks < KD / 32; ++ks) {
                 h8 bk = row8(Ks, LDQ, 16 * w + row, ks * 32, G);
 #pragma unroll
-                for (int it = 0; it < 4; ++it)
-                    if (it >= w) a_[it] = mfma32(row8(Qs, LDQ, 16 * it + row, ks * 32, G), bk, a_[it]);
+                for (int it = 0; it < 4; ++it)   // all four tiles, branch-free
+                    a_[it] = mfma32(row8(Qs, LDQ, 16 * it + row, ks * 32, G), bk, a_[it]);
             }
 #pragma unroll
             for (int cs = 0; cs < DH / 32; ++cs) {
                 h8 bv = row8(Vs, LDV, 16 * w + row, cs * 32, G);
 #pragma unroll
                 for (int it = 0; it < 4; ++it)
-                    if (it >= w) p_[it] = mfma32(row8(Gs, LDV, 16 * it + row, cs * 32, G), bv, p_[it]);
+                    p_[it] = mfma32(row8(Gs, LDV, 16 * it + row, cs * 32, G), bv, p_[it]);
             }
             const int j = 16 * w + row;
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
-                h4 av = h4_zero(), pv = h4_zero();
-                if (it >= w) {
-                    f4 gzv = *reinterpret_cast<const f4*>(gzs + 16 * it + 4 * G);
+                h4 av, pv;
+                f4 gzv = *reinterpret_cast<const f4*>(gzs + 16 * it + 4 * G);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int i = 16 * it + 4 * G + e;
-                        if (i >= j) {
-                            av[e] = (half_t)a_[it][e];
-                            pv[e] = (half_t)(p_[it][e] + gzv[e]);
-                        }
-                    }
+                for (int e = 0; e < 4; ++e) {
+                    const int i = 16 * it + 4 * G + e;
+                    av[e] = (i >= j) ? (half_t)a_[it][e] : (half_t)0.f;
+                    pv[e] = (i >= j) ? (half_t)(p_[it][e] + gzv[e]) : (half_t)0.f;
                 }
                 *reinterpret_cast<h4*>(ATs + j * LDA + 16 * it + 4 * G) = av;
                 *reinterpret_cast<h4*>(PTs + j * LDA + 16 * it + 4 * G) = pv;
@@ -842,10 +901,9 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
                 for (int jt = 0; jt < 4; ++jt) {
                     h8 bvv = row_split8(Vs, LDV, 16 * jt + row, cs * 32, G);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) {
-                        dkacc[kt][jt] = mfma32(hi[kt], bvv, dkacc[kt][jt]);
-                        dkacc[kt][jt] = mfma32(lo[kt], bvv, dkacc[kt][jt]);
-                    }
+                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(hi[kt], bvv, dkacc[kt][jt]);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(lo[kt], bvv, dkacc[kt][jt]);
                 }
             }
 #pragma unroll
@@ -882,10 +940,9 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
                 for (int jt = 0; jt < 4; ++jt) {
                     h8 bkk = row_split8(Ks, LDQ, 16 * jt + row, ks * 32, G);
 #pragma unroll
-                    for (int ct = 0; ct < NCT2; ++ct) {
-                        dvacc[ct][jt] = mfma32(hi[ct], bkk, dvacc[ct][jt]);
-                        dvacc[ct][jt] = mfma32(lo[ct], bkk, dvacc[ct][jt]);
-                    }
+                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(hi[ct], bkk, dvacc[ct][jt]);
+#pragma unroll
+                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(lo[ct], bkk, dvacc[ct][jt]);
                 }
             }
 #pragma unroll
@@ -901,6 +958,13 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
             // carried sums
 #pragma unroll
             for (int is = 0; is < (CAUSAL ? 2 : 0); ++is) {
+                h8 ghi, glo;   // r (m=k) += Q^T gz
+                f8_to_operand(*reinterpret_cast<const f4*>(gzs + is * 32 + 8 * G),
+                              *reinterpret_cast<const f4*>(gzs + is * 32 + 8 * G + 4), ghi, glo);
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt][is], ghi, racc[kt]);
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt][is], glo, racc[kt]);
 #pragma unroll
                 for (int ct = 0; ct < NCT; ++ct) {
                     h8 gf = col8(Gs, LDV, is * 32, 16 * ct, lane);
@@ -913,12 +977,6 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
 #pragma unroll
                     for (int ct = 0; ct < NCT2; ++ct) RR[kt][ct] = mfma32(qa, gf2[ct][is], RR[kt][ct]);
                 }
-            }
-            if (CAUSAL && tid < KD) {
-                float sr = 0.f;
-#pragma unroll 8
-                for (int i = 0; i < C; ++i) sr += (float)Qs[i * LDQ + tid] * gzs[i];
-                rreg += sr;
             }
         }
         __syncthreads();

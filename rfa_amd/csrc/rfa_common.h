@@ -25,6 +25,31 @@ typedef half_t h4 __attribute__((ext_vector_type(4)));
 typedef half_t h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 
+// Phase timing for kernel tuning: compile with -DRFA_PHASE_TIMING to make thread 0 of
+// one workgroup add the core-clock cycles spent between consecutive RFA_TICK marks to
+// g_phase_ticks (read back with rfa_debug_phase_ticks).  Compiled out otherwise.
+#ifdef RFA_PHASE_TIMING
+__device__ unsigned long long g_phase_ticks[32];
+#define RFA_TICK_INIT() long long tick_last_ = clock64()
+#define RFA_TICK(i)                                                                        \
+    do {                                                                                   \
+        if (blockIdx.x == RFA_PHASE_TIMING && threadIdx.x == 0) {                          \
+            const long long now_ = clock64();                                              \
+            atomicAdd(&g_phase_ticks[i], (unsigned long long)(now_ - tick_last_));         \
+            tick_last_ = now_;                                                             \
+        }                                                                                  \
+    } while (0)
+#else
+#define RFA_TICK_INIT() do { } while (0)
+#define RFA_TICK(i) do { } while (0)
+#endif
+
+// Row padding (in halves) of an LDS array with F halves per row.  With 64 banks of 4
+// bytes the row stride in dwords must be 4*odd mod 64 for conflict-free 16-byte row
+// reads and leave 8-dword gaps between 4 consecutive rows for the transposing reads:
+// stride = 12 (mod 64) dwords for F = 128, 256 and 36 for F = 64.
+constexpr int lds_pad(int F) { return (F % 128 == 0) ? 24 : 8; }
+
 constexpr int kThreads = 256;   // threads per workgroup
 constexpr int kChunk = 64;      // time steps per chunk
 
@@ -44,10 +69,7 @@ __device__ __forceinline__ h8 row_split8(const half_t* X, int ld, int row, int c
     const half_t* p = X + row * ld + c0 + 4 * G;
     h4 a = *reinterpret_cast<const h4*>(p);
     h4 b = *reinterpret_cast<const h4*>(p + 16);
-    h8 r;
-    r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
-    r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
-    return r;
+    return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
 // LDS transposing read (ds_read_b64_tr_b16).  Within each group of 16 lanes the
@@ -57,10 +79,9 @@ __device__ __forceinline__ h8 row_split8(const half_t* X, int ld, int row, int c
 __device__ __forceinline__ h4 tr_read4(const half_t* p) {
     typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 fp16x4;
     typedef __attribute__((address_space(3))) fp16x4 lds_fp16x4;
-    fp16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_fp16x4*)(p));
-    h4 r;
-    r[0] = (half_t)v[0]; r[1] = (half_t)v[1]; r[2] = (half_t)v[2]; r[3] = (half_t)v[3];
-    return r;
+    union { fp16x4 v; h4 h; } u;
+    u.v = __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_fp16x4*)(p));
+    return u.h;
 }
 
 // Column fragment in natural slot order: X[r0 + 8G + e][c0 + i], e = 0..7, from a
@@ -72,10 +93,7 @@ __device__ __forceinline__ h8 col8(const half_t* X, int ld, int r0, int c0, int 
     const half_t* p = X + (r0 + 8 * G + (s >> 2)) * ld + c0 + 4 * (s & 3);
     h4 a = tr_read4(p);
     h4 b = tr_read4(p + 4 * ld);
-    h8 r;
-    r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
-    r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
-    return r;
+    return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
 // Two fp32 accumulator tiles -> one fp16 operand pair (hi + lo carries ~22 bits),
@@ -102,6 +120,26 @@ __device__ __forceinline__ h4 h4_zero() {
     h4 r; r[0] = (half_t)0.f; r[1] = (half_t)0.f; r[2] = (half_t)0.f; r[3] = (half_t)0.f; return r;
 }
 
+__device__ __forceinline__ h8 h8_ones() {
+    h8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (half_t)1.0f;
+    return r;
+}
+
+// eight fp32 values (two f4) -> fp16 operand pair hi + lo, natural slot order
+__device__ __forceinline__ void f8_to_operand(const f4& a, const f4& b, h8& hi, h8& lo) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        half_t h0 = (half_t)a[e];
+        half_t h1 = (half_t)b[e];
+        hi[e] = h0;
+        hi[4 + e] = h1;
+        lo[e] = (half_t)(a[e] - (float)h0);
+        lo[4 + e] = (half_t)(b[e] - (float)h1);
+    }
+}
+
 // sum over the four 16-lane groups (lanes i, i+16, i+32, i+48)
 __device__ __forceinline__ float sum_over_groups(float x) {
     x += __shfl_xor(x, 16, 64);
@@ -125,6 +163,15 @@ template <int F>
 __device__ __forceinline__ void chunk_g2r(ChunkRegs<F>& r, const half_t* __restrict__ base,
                                           int64_t row_stride, int rows_valid, int tid) {
     constexpr int PPR = F / 8;
+    if (rows_valid >= kChunk) {   // full chunk (uniform): no per-lane predication
+#pragma unroll
+        for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
+            const int p = tid + kThreads * it;
+            const int row = p / PPR, c8 = p % PPR;
+            r.v[it] = *reinterpret_cast<const uint4*>(base + (int64_t)row * row_stride + c8 * 8);
+        }
+        return;
+    }
 #pragma unroll
     for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
         const int p = tid + kThreads * it;

@@ -17,8 +17,8 @@ namespace rfa {
 template <int D, int DH>
 struct FeatureCfg {
     static_assert(D % 32 == 0 && DH % 64 == 0, "D multiple of 32, DH multiple of 64");
-    static constexpr int LDW = DH + 16;
-    static constexpr int LDU = D + 16;
+    static constexpr int LDW = DH + lds_pad(DH);
+    static constexpr int LDU = D + lds_pad(D);
     static constexpr size_t kFwdLds = (size_t)D * LDW * 2;
     static constexpr size_t kBwdLds = (size_t)(D * LDW + 64 * LDW + 64 * LDU) * 2;
 };
