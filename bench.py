@@ -25,6 +25,16 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch at the bench configuration, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
+# passes summarised in profiles/bench_cfg2_hbm_traffic.md (counters scaled on the 512 MiB copy).
+MEASURED_TRAFFIC_BYTES = {
+    "k_segment_state": 25359084,
+    "k_causal_fwd": 63281112,
+    "k_causal_bwd_dq": 87573852,
+    "k_causal_bwd_dkdv": 89580074,
+    "k_decode_step": 68890060,
+}
+
 
 def _event_time_ms(torch, fn, iters):
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -119,7 +129,8 @@ def main():
     dom_bytes = per_tok[dominant] * units[dominant]
     achieved = dom_bytes / (kern_us[dominant] * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
                 "bytes_per_launch": dom_bytes, "avg_us": round(kern_us[dominant], 2),
                 "kernels_us": {n_: round(u, 2) for n_, u in kern_us.items()},
                 "step_algorithmic_bytes": 2176 * N * T,
@@ -246,6 +257,17 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream):
                          "bwd_us": round(1e3 * tb, 2),
                          "fwd_hbm_gbs": round(rows * (d + 2 * D) * 2 / (tf * 1e-3) / 1e9, 1),
                          "bwd_hbm_gbs": round(rows * (2 * d + 2 * D) * 2 / (tb * 1e-3) / 1e9, 1)}
+    # ---- plain device copy of 512 MiB (larger than the 256 MiB last-level cache): the HBM
+    # bandwidth a trivial kernel reaches here, and the known-size dispatch against which the
+    # rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled
+    src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    cp = lambda: torch.bitwise_not(src, out=dst)      # an elementwise kernel, not a DMA copy
+    for _ in range(2):
+        cp()
+    tc = _event_time_ms(torch, cp, 5)
+    ex["hbm_copy"] = {"bytes_read": 512 << 20, "bytes_written": 512 << 20,
+                      "gbs": round(2 * (512 << 20) / (tc * 1e-3) / 1e9, 1)}
     return ex
 
 

@@ -3,6 +3,7 @@
 #include "../../include/rfa_hip.h"
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdio>
@@ -58,29 +59,27 @@ hipEvent_t take_event() {
     return e;
 }
 
-// Records an event pair around one kernel launch on `st` while profiling is on.
-struct Scope {
-    int id; hipStream_t st; hipEvent_t a = nullptr;
-    Scope(int id_, hipStream_t st_) : id(id_), st(st_) {
-        if (!enabled) return;
+// One kernel launch.  While profiling is on the launch carries a start/stop event pair
+// that takes the kernel's own begin and end timestamps (hipExtLaunchKernelGGL), i.e. the
+// same interval a kernel trace reports, without the launch latency around it.
+template <typename F, typename... Args>
+void launch(int id, F kern, dim3 grid, dim3 block, size_t lds, hipStream_t st, Args... args) {
+    if (enabled) {
         std::lock_guard<std::mutex> lk(mu);
-        a = take_event();
-        if (a) (void)hipEventRecord(a, st);
+        hipEvent_t a = take_event(), b = take_event();
+        if (a && b) {
+            hipExtLaunchKernelGGL(kern, grid, block, (uint32_t)lds, st, a, b, 0, args...);
+            recs.push_back({id, a, b});
+            return;
+        }
+        if (a) pool.push_back(a);
+        if (b) pool.push_back(b);
     }
-    ~Scope() {
-        if (!a) return;
-        std::lock_guard<std::mutex> lk(mu);
-        hipEvent_t b = take_event();
-        if (b) { (void)hipEventRecord(b, st); recs.push_back({id, a, b}); } else { pool.push_back(a); }
-    }
-};
+    hipLaunchKernelGGL(kern, grid, block, lds, st, args...);
+}
 }  // namespace prof
 
-#define RFA_LAUNCH(ID, ...)                       \
-    do {                                          \
-        prof::Scope prof_scope_(prof::ID, st);    \
-        hipLaunchKernelGGL(__VA_ARGS__);          \
-    } while (0)
+#define RFA_LAUNCH(ID, ...) prof::launch(prof::ID, __VA_ARGS__)
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -284,7 +283,7 @@ int launch_decode(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t*
 // ---- feature map launchers ---------------------------------------------------------
 int feature_bwd_blocks(int64_t R, int H) {
     const int64_t nrb = (R + 63) / 64;
-    int64_t nblk = (1024 + H - 1) / H;
+    int64_t nblk = (256 + H - 1) / H;   // about one workgroup per CU; few partial sums to reduce
     if (nblk > nrb) nblk = nrb;
     if (nblk < 1) nblk = 1;
     return (int)nblk;

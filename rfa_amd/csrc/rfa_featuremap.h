@@ -220,9 +220,16 @@ __global__ void k_feature_map_dw_reduce(const float* __restrict__ part, float* _
                                         int64_t elems) {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= elems) return;
-    float s = 0.f;
-    for (int b = 0; b < nblk; ++b) s += part[(int64_t)b * elems + e];
-    dw[e] = s;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;   // independent chains: the loads overlap
+    int b = 0;
+    for (; b + 4 <= nblk; b += 4) {
+        s0 += part[(int64_t)b * elems + e];
+        s1 += part[(int64_t)(b + 1) * elems + e];
+        s2 += part[(int64_t)(b + 2) * elems + e];
+        s3 += part[(int64_t)(b + 3) * elems + e];
+    }
+    for (; b < nblk; ++b) s0 += part[(int64_t)b * elems + e];
+    dw[e] = (s0 + s1) + (s2 + s3);
 }
 
 }  // namespace rfa
