@@ -1,0 +1,133 @@
+"""Full-size GPU tests at the benchmark configurations: oracle comparison on a few
+sequences (the CPU oracle would take minutes on all of them) plus size-independent
+properties on everything -- bit-exact independence of sequences, run-to-run determinism,
+the prefix property, and decode/prefill hand-off."""
+import pytest
+import torch
+
+from oracle import rfa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(a, b):
+    return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+def _features_gpu(T, B, H, d, D, seed):
+    from rfa_amd import rfa_hip
+    g = torch.Generator().manual_seed(seed)
+    unit = lambda t: t / t.norm(dim=-1, keepdim=True)
+    W = O.make_w(d, D, H).half().cuda()
+    q = unit(torch.randn(T, B, H, d, generator=g)).half().cuda()
+    k = unit(torch.randn(T, B, H, d, generator=g)).half().cuda()
+    v = torch.randn(T, B, H, d, generator=g).half().cuda()
+    go = torch.randn(T, B, H, d, generator=g).half().cuda()
+    pq = rfa_hip.feature_map_forward(q, W, O.SCALE).view(T, B * H, 2 * D)
+    pk = rfa_hip.feature_map_forward(k, W, O.SCALE).view(T, B * H, 2 * D)
+    return pq, pk, v.view(T, B * H, d), go.view(T, B * H, d)
+
+
+@pytest.mark.parametrize("name,T,B,H,d,D,n_check", [
+    ("config2", 1024, 8, 8, 64, 64, 4),
+    ("config5", 16384, 2, 16, 128, 128, 1),
+])
+def test_causal_full_size(name, T, B, H, d, D, n_check):
+    from rfa_amd import rfa_hip
+    print(f"{name}: causal fwd+bwd T={T} N={B*H} K={2*D} d={d}", flush=True)
+    pq, pk, v, g = _features_gpu(T, B, H, d, D, seed=1234 + T)
+    N = B * H
+    out = rfa_hip.forward(pq, pk, v)
+    dq, dk, dv = rfa_hip.backward(pq, pk, v, g)
+    assert all(torch.isfinite(t.float()).all() for t in (out, dq, dk, dv))
+    # oracle on the first and last n_check sequences
+    for sl in (slice(0, n_check), slice(N - n_check, N)):
+        cq, ck, cv, cg = (t[:, sl].float().cpu() for t in (pq, pk, v, g))
+        ref = O.causal_forward_chunked(cq, ck, cv)
+        assert (out[:, sl].float().cpu() - ref).abs().max().item() <= 2e-3
+        rq, rk, rv = O.causal_backward_chunked(cq, ck, cv, cg)
+        for nm, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+            assert _rel(got[:, sl].float().cpu(), want) <= 1e-2, (nm, _rel(got[:, sl].float().cpu(), want))
+    # determinism: a second run is bit-identical
+    assert torch.equal(rfa_hip.forward(pq, pk, v), out)
+    assert all(torch.equal(a, b) for a, b in zip(rfa_hip.backward(pq, pk, v, g), (dq, dk, dv)))
+    # sequences are independent: reversing their order reverses the results bit for bit
+    flip = lambda t: t.flip(1).contiguous()
+    assert torch.equal(rfa_hip.forward(flip(pq), flip(pk), flip(v)), flip(out))
+    fq, fk, fv = rfa_hip.backward(flip(pq), flip(pk), flip(v), flip(g))
+    assert torch.equal(fq, flip(dq)) and torch.equal(fk, flip(dk)) and torch.equal(fv, flip(dv))
+    # prefix property: the first T/2 + 7 steps do not depend on what follows
+    Tp = T // 2 + 7
+    part = rfa_hip.forward(pq[:Tp].contiguous(), pk[:Tp].contiguous(), v[:Tp].contiguous())
+    assert (part.float() - out[:Tp].float()).abs().max().item() <= 2e-3
+    # zero upstream gradient -> zero gradients
+    zq, zk, zv = rfa_hip.backward(pq, pk, v, torch.zeros_like(g))
+    assert not zq.any() and not zk.any() and not zv.any()
+
+
+def test_cross_full_size_config3():
+    from rfa_amd import rfa_hip
+    Tt, S, B, H, d, D = 256, 512, 32, 8, 64, 64
+    print("config3: cross fwd+bwd", flush=True)
+    g = torch.Generator().manual_seed(1234 + 3)
+    unit = lambda t: t / t.norm(dim=-1, keepdim=True)
+    W = O.make_w(d, D, H).half()
+    lens = torch.randint(256, 513, (B,), generator=g)
+    pad = torch.arange(S)[None, :] >= lens[:, None]
+    k = unit(torch.randn(S, B, H, d, generator=g)).half()
+    q = unit(torch.randn(Tt, B, H, d, generator=g)).half()
+    v = torch.randn(S, B, H, d, generator=g).half()
+    go = torch.randn(Tt, B, H, d, generator=g).half()
+    pk = rfa_hip.feature_map_forward(k.cuda(), W.cuda(), O.SCALE)
+    pq = rfa_hip.feature_map_forward(q.cuda(), W.cuda(), O.SCALE)
+    s, z = rfa_hip.cross_state(pk, v.cuda(), pad.cuda())
+    out = rfa_hip.cross_readout(pq, s, z)
+    dq, ds, dz = rfa_hip.cross_readout_backward(pq, s, z, go.cuda())
+    dk, dv = rfa_hip.cross_state_backward(pk, v.cuda(), ds, dz, pad.cuda())
+    fpk, fpq = pk.float().cpu(), pq.float().cpu()
+    rs, rz = O.cross_state(fpk, v.float(), pad.t())
+    assert _rel(s.cpu(), rs) <= 1e-3 and _rel(z.cpu(), rz) <= 1e-3
+    assert (out.float().cpu() - O.cross_readout(fpq, rs, rz)).abs().max().item() <= 2e-3
+    wq, wds, wdz = O.cross_readout_backward(fpq, rs, rz, go.float())
+    wk, wv = O.cross_state_backward(fpk, v.float(), wds, wdz, pad.t())
+    for nm, got, want in (("dq", dq, wq), ("ds", ds, wds), ("dz", dz, wdz), ("dk", dk, wk), ("dv", dv, wv)):
+        assert _rel(got.float().cpu(), want) <= 1e-2, (nm, _rel(got.float().cpu(), want))
+    # masking == truncation: batch entry b only sees its first lens[b] source steps
+    b = int(torch.argmin(lens))
+    L = int(lens[b])
+    s1, z1 = rfa_hip.cross_state(pk[:L, b:b + 1].contiguous(), v[:L, b:b + 1].cuda().contiguous())
+    assert torch.allclose(s1[0], s[b], rtol=1e-5, atol=1e-6) and torch.allclose(z1[0], z[b], rtol=1e-5, atol=1e-6)
+    assert not dk.float().cpu()[pad.t()].any()
+
+
+def test_decode_full_size_config4():
+    """512-token prefill through the scan kernels' state, then 2048 fused decode steps; the
+    outputs must equal the causal forward over the whole 2560-step sequence."""
+    from rfa_amd import rfa_hip
+    B, H, d, D, prefill, steps = 64, 16, 64, 64, 512, 2048
+    N, K, T = B * H, 2 * D, prefill + steps
+    print("config4: decode", flush=True)
+    g = torch.Generator().manual_seed(1234 + 4)
+    unit = lambda t: t / t.norm(dim=-1, keepdim=True)
+    W = O.make_w(d, D, H).half().cuda()
+    # the same 256-step block of inputs is cycled (keeps host memory small)
+    blk = 256
+    q = unit(torch.randn(blk, B, H, d, generator=g)).half().cuda().repeat(T // blk, 1, 1, 1)
+    k = unit(torch.randn(blk, B, H, d, generator=g)).half().cuda().repeat(T // blk, 1, 1, 1)
+    v = torch.randn(blk, B, H, d, generator=g).half().cuda().repeat(T // blk, 1, 1, 1)
+    pq = rfa_hip.feature_map_forward(q, W, O.SCALE)
+    pk = rfa_hip.feature_map_forward(k, W, O.SCALE)
+    full = rfa_hip.forward(pq.view(T, N, K), pk.view(T, N, K), v.view(T, N, d))      # scan over all 2560 steps
+    s, z = rfa_hip.cross_state(pk[:prefill].contiguous(), v[:prefill].contiguous())  # state after the prefill
+    dec = rfa_hip.incremental_fused(q[prefill:].contiguous(), k[prefill:].contiguous(), v[prefill:].contiguous(),
+                                    W, O.SCALE, s, z)
+    assert (dec.view(steps, N, d).float() - full[prefill:].float()).abs().max().item() <= 2e-3
+    s_all, z_all = rfa_hip.cross_state(pk, v)
+    # (the fused step evaluates phi in fp32, the scan reads fp16-rounded phi)
+    assert _rel(s, s_all) <= 1e-3 and _rel(z, z_all) <= 1e-3
+    # oracle on two heads, all 2560 steps
+    sl = slice(0, 2)
+    want, ws, wz = O.causal_forward_loop(pq.view(T, N, K)[:, sl].float().cpu(), pk.view(T, N, K)[:, sl].float().cpu(),
+                                         v.view(T, N, d)[:, sl].float().cpu())
+    assert (dec.view(steps, N, d)[:, sl].float().cpu() - want[prefill:]).abs().max().item() <= 2e-3
+    assert _rel(s.view(N, K, d)[sl].cpu(), ws) <= 1e-3
