@@ -5,8 +5,8 @@
 
 A "step" is one causal forward + backward over one batch of synthetic input at the
 configuration the headline metric is quoted on (seq 1024, batch 8, 8 heads,
-head_dim 64, proj_dim 64, fp16), called through the C ABI (rfa_causal_forward +
-rfa_causal_backward) with all inputs resident in HBM.  One JSON line is printed:
+head_dim 64, proj_dim 64, fp16), called through the C ABI (rfa_causal_forward_save +
+rfa_causal_backward_saved, the pair RFA.apply(...).backward(...) runs) with all inputs resident in HBM.  One JSON line is printed:
 the throughput of that step, the roofline of its dominant kernel (per-kernel
 durations from HIP events recorded by the library around every launch), the same
 step timed with the CPU oracle on the host cores, and -- as extra keys -- the decode,
@@ -85,10 +85,15 @@ def main():
     ws = torch.empty(max(fbytes, bbytes, 1), dtype=torch.uint8, device=dev)
     p = lambda t: t.data_ptr()
 
+    sbytes = lib.rfa_causal_saved_state_bytes(T, N, K, d)
+    saved = torch.empty(max(sbytes, 1), dtype=torch.uint8, device=dev)
+
     def step():
-        _lib.check(lib.rfa_causal_forward(p(pq), p(pk), p(vv), p(out), T, N, K, d, p(ws), fbytes, stream))
-        _lib.check(lib.rfa_causal_backward(p(pq), p(pk), p(vv), p(gg), p(dq), p(dk), p(dv), T, N, K, d,
-                                           p(ws), bbytes, stream))
+        # what RFA.apply(...).backward(grad) runs: the forward hands its segment totals to the backward
+        _lib.check(lib.rfa_causal_forward_save(p(pq), p(pk), p(vv), p(out), p(saved), sbytes, T, N, K, d,
+                                               p(ws), fbytes, stream))
+        _lib.check(lib.rfa_causal_backward_saved(p(pq), p(pk), p(vv), p(gg), p(saved), sbytes, p(dq), p(dk), p(dv),
+                                                 T, N, K, d, p(ws), bbytes, stream))
 
     for _ in range(args.warmup):
         step()

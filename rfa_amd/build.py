@@ -23,6 +23,9 @@ HIPCC_FLAGS = [
     "-ffp-contract=fast",
     # keep the compiler from forming packed fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA accumulators in VGPRs: the state tiles are re-read as operands every chunk,
+    # AGPR residency would cost a v_accvgpr move per element per use
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
 
 

@@ -143,15 +143,17 @@ int set_lds(Kern kern, size_t bytes) {
 
 template <int KD, int DH>
 int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, rfa::half_t* out,
-                   int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, hipStream_t st) {
+                   int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, float* savedS, float* savedZ,
+                   hipStream_t st) {
     using Cfg = rfa::CausalCfg<KD, DH>;
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
-    float* wsZ = reinterpret_cast<float*>(ws + wl.Z);
+    // with a saved-state buffer the z totals are written there directly (z has one layout)
+    float* wsZ = savedZ ? savedZ : reinterpret_cast<float*>(ws + wl.Z);
     if (p.nseg > 1) {
         auto kern = rfa::k_segment_state<KD, DH, true>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
-                           k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, T, N, p.nseg, p.nseg - 1, p.seg_len);
+                           k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, savedS, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     auto kern = rfa::k_causal_fwd<KD, DH, true>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
@@ -164,7 +166,8 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
 template <int KD, int DH>
 int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v,
                     const rfa::half_t* g, rfa::half_t* dq, rfa::half_t* dk, rfa::half_t* dv, int T, int N,
-                    const ScanPlan& p, char* ws, const Workspace& wl, hipStream_t st) {
+                    const ScanPlan& p, char* ws, const Workspace& wl, const float* savedS, const float* savedZ,
+                    hipStream_t st) {
     using Cfg = rfa::CausalCfg<KD, DH>;
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
     float* wsZ = reinterpret_cast<float*>(ws + wl.Z);
@@ -172,17 +175,22 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
     float* wsr = reinterpret_cast<float*>(ws + wl.r);
     float* den = reinterpret_cast<float*>(ws + wl.den);
     float* gz = reinterpret_cast<float*>(ws + wl.gz);
-    if (p.nseg > 1) {
+    const float* inS = wsS;
+    const float* inZ = wsZ;
+    if (savedS) {          // segment totals handed over by the forward pass
+        inS = savedS;
+        inZ = savedZ;
+    } else if (p.nseg > 1) {
         auto kern = rfa::k_segment_state<KD, DH, false>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
-                           k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, T, N, p.nseg, p.nseg - 1, p.seg_len);
+                           k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     {
         auto kern = rfa::k_causal_bwd_dq<KD, DH, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDqLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDqLds, st, q, k, v, g,
-                           dq, wsS, wsZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
+                           dq, inS, inZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
     }
     {
         auto kern = rfa::k_causal_bwd_dkdv<KD, DH, true>;
@@ -216,8 +224,8 @@ int launch_cross_state(const rfa::half_t* k, const rfa::half_t* v, const uint8_t
     const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
     auto kern = rfa::k_segment_state<KD, DH, false>;
     if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
-    RFA_LAUNCH(SEG_STATE, kern, dim3(N), dim3(rfa::kThreads), Cfg::kSegStateLds, st, k, v, mask, H, s, z, T, N,
-                       1, 1, seg_len);
+    RFA_LAUNCH(SEG_STATE, kern, dim3(N), dim3(rfa::kThreads), Cfg::kSegStateLds, st, k, v, mask, H, s, z,
+               (float*)nullptr, T, N, 1, 1, seg_len);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -429,10 +437,50 @@ size_t rfa_causal_backward_workspace_bytes(int64_t T, int64_t N, int K, int d) {
     if (K == 128 && d == 128) { return CALL(128, 128); }              \
     if (K == 256 && d == 128) { return CALL(256, 128); }
 
+// bytes of the segment totals (row-major S then z) for the saved-state buffer
+static size_t saved_state_bytes(int64_t T, int64_t N, int K, int d, size_t* z_offset) {
+    const ScanPlan p = make_plan(T, N);
+    const size_t s_bytes = align_up((size_t)N * p.nseg * K * d * 4);
+    if (z_offset) *z_offset = s_bytes;
+    return s_bytes + align_up((size_t)N * p.nseg * K * 4);
+}
+
+size_t rfa_causal_saved_state_bytes(int64_t T, int64_t N, int K, int d) {
+    if (T <= 0 || N <= 0 || !rfa_shape_supported(K, d)) return 0;
+    return saved_state_bytes(T, N, K, d, nullptr);
+}
+
+static int causal_forward_impl(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
+                               int K, int d, void* saved, size_t saved_bytes, bool want_saved, void* workspace,
+                               size_t workspace_bytes, void* stream);
+
 int rfa_causal_forward(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
                        int K, int d, void* workspace, size_t workspace_bytes, void* stream) {
+    return causal_forward_impl(q, k, v, out, T, N, K, d, nullptr, 0, false, workspace, workspace_bytes, stream);
+}
+
+int rfa_causal_forward_save(const void* q, const void* k, const void* v, void* out, void* saved,
+                            size_t saved_bytes, int64_t T, int64_t N, int K, int d, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+    return causal_forward_impl(q, k, v, out, T, N, K, d, saved, saved_bytes, true, workspace, workspace_bytes, stream);
+}
+
+static int causal_forward_impl(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
+                               int K, int d, void* saved, size_t saved_bytes, bool want_saved, void* workspace,
+                               size_t workspace_bytes, void* stream) {
     if (int rc = check_causal_dims(T, N, K, d)) return rc;
     if (T == 0 || N == 0) return RFA_OK;
+    float* savedS = nullptr;
+    float* savedZ = nullptr;
+    if (want_saved) {
+        size_t zoff = 0;
+        const size_t need = saved_state_bytes(T, N, K, d, &zoff);
+        if (!saved || saved_bytes < need || !aligned16(saved))
+            return fail(RFA_ERR_WORKSPACE, "rfa_causal_forward_save: saved-state buffer of %zu bytes required, got %zu",
+                        need, saved ? saved_bytes : (size_t)0);
+        savedS = static_cast<float*>(saved);
+        savedZ = reinterpret_cast<float*>(static_cast<char*>(saved) + zoff);
+    }
     if (!q || !k || !v || !out) return fail(RFA_ERR_NULL_POINTER, "rfa_causal_forward: NULL tensor pointer");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
         return fail(RFA_ERR_ALIGNMENT, "rfa_causal_forward: tensors must be 16-byte aligned");
@@ -447,17 +495,48 @@ int rfa_causal_forward(const void* q, const void* k, const void* v, void* out, i
     auto* vh = static_cast<const rfa::half_t*>(v);
     auto* oh = static_cast<rfa::half_t*>(out);
     char* ws = static_cast<char*>(workspace);
-#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, st)
+#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedS, savedZ, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_FWD)
 #undef RFA_CALL_FWD
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
 }
 
+static int causal_backward_impl(const void* q, const void* k, const void* v, const void* grad_attn, void* dq,
+                                void* dk, void* dv, int64_t T, int64_t N, int K, int d, const void* saved,
+                                size_t saved_bytes, bool have_saved, void* workspace, size_t workspace_bytes,
+                                void* stream);
+
 int rfa_causal_backward(const void* q, const void* k, const void* v, const void* grad_attn, void* dq,
                         void* dk, void* dv, int64_t T, int64_t N, int K, int d, void* workspace,
                         size_t workspace_bytes, void* stream) {
+    return causal_backward_impl(q, k, v, grad_attn, dq, dk, dv, T, N, K, d, nullptr, 0, false, workspace,
+                                workspace_bytes, stream);
+}
+
+int rfa_causal_backward_saved(const void* q, const void* k, const void* v, const void* grad_attn,
+                              const void* saved, size_t saved_bytes, void* dq, void* dk, void* dv, int64_t T,
+                              int64_t N, int K, int d, void* workspace, size_t workspace_bytes, void* stream) {
+    return causal_backward_impl(q, k, v, grad_attn, dq, dk, dv, T, N, K, d, saved, saved_bytes, true, workspace,
+                                workspace_bytes, stream);
+}
+
+static int causal_backward_impl(const void* q, const void* k, const void* v, const void* grad_attn, void* dq,
+                                void* dk, void* dv, int64_t T, int64_t N, int K, int d, const void* saved,
+                                size_t saved_bytes, bool have_saved, void* workspace, size_t workspace_bytes,
+                                void* stream) {
     if (int rc = check_causal_dims(T, N, K, d)) return rc;
     if (T == 0 || N == 0) return RFA_OK;
+    const float* savedS = nullptr;
+    const float* savedZ = nullptr;
+    if (have_saved) {
+        size_t zoff = 0;
+        const size_t need = saved_state_bytes(T, N, K, d, &zoff);
+        if (!saved || saved_bytes < need || !aligned16(saved))
+            return fail(RFA_ERR_WORKSPACE, "rfa_causal_backward_saved: saved-state buffer of %zu bytes required, got %zu",
+                        need, saved ? saved_bytes : (size_t)0);
+        savedS = static_cast<const float*>(saved);
+        savedZ = reinterpret_cast<const float*>(static_cast<const char*>(saved) + zoff);
+    }
     if (!q || !k || !v || !grad_attn || !dq || !dk || !dv)
         return fail(RFA_ERR_NULL_POINTER, "rfa_causal_backward: NULL tensor pointer");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(grad_attn) || !aligned16(dq) ||
@@ -477,7 +556,7 @@ int rfa_causal_backward(const void* q, const void* k, const void* v, const void*
     auto* dkh = static_cast<rfa::half_t*>(dk);
     auto* dvh = static_cast<rfa::half_t*>(dv);
     char* ws = static_cast<char*>(workspace);
-#define RFA_CALL_BWD(KD, DH) launch_backward<KD, DH>(qh, kh, vh, gh, dqh, dkh, dvh, (int)T, (int)N, p, ws, wl, st)
+#define RFA_CALL_BWD(KD, DH) launch_backward<KD, DH>(qh, kh, vh, gh, dqh, dkh, dvh, (int)T, (int)N, p, ws, wl, savedS, savedZ, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_BWD)
 #undef RFA_CALL_BWD
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");

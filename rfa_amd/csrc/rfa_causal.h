@@ -63,11 +63,13 @@ struct CausalCfg {
 // scan, owning the same tiles, reads back with one 16-byte load per tile.
 // z is accumulated on the MFMA too: z tile (m=k) = K^T 1 with an all-ones operand;
 // wave w owns the feature tiles kt in [w*NKTW, (w+1)*NKTW).
+// row_copy (FRAG only, may be NULL) receives a second, row-major copy of the totals: the
+// forward pass of a training step hands it to the backward pass, which then skips this pass.
 template <int KD, int DH, bool FRAG>
 __global__ __launch_bounds__(kThreads) void k_segment_state(
     const half_t* __restrict__ k, const half_t* __restrict__ v, const uint8_t* __restrict__ pad_mask,
-    int H, float* __restrict__ wsS, float* __restrict__ wsZ, int T, int N, int nseg, int nseg_out,
-    int seg_len) {
+    int H, float* __restrict__ wsS, float* __restrict__ wsZ, float* __restrict__ row_copy, int T, int N,
+    int nseg, int nseg_out, int seg_len) {
     using Cfg = CausalCfg<KD, DH>;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, DS = Cfg::DS;
     constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / 4;
@@ -137,7 +139,9 @@ __global__ __launch_bounds__(kThreads) void k_segment_state(
         for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
             for (int ct = 0; ct < NCT; ++ct) sf[(kt * NCT + ct) * 64 + lane] = S[kt][ct];
-    } else {
+    }
+    if (!FRAG || row_copy) {
+        if (FRAG) so = row_copy + ((int64_t)(n * nseg + seg) * KD) * DH;
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll

@@ -77,15 +77,20 @@ class RFA(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q: Tensor, k: Tensor, v: Tensor) -> Tensor:
-        """attn [tgt_len, bsz*heads, head_dim]; saves (q, k, v) like rfa.py:124."""
+        """attn [tgt_len, bsz*heads, head_dim]; saves (q, k, v) like rfa.py:124 (plus the segment totals)."""
         ctx.in_dtypes = (q.dtype, k.dtype, v.dtype)
         q, k, v = _as_kernel_input(q), _as_kernel_input(k), _as_kernel_input(v)
-        ctx.save_for_backward(q, k, v)
-        return rfa_hip.forward(q, k, v).to(ctx.in_dtypes[2])
+        if any(ctx.needs_input_grad):
+            # also keep the per-segment state totals so that backward need not rebuild them
+            attn, seg_totals = rfa_hip.forward_save(q, k, v)
+            ctx.save_for_backward(q, k, v, seg_totals)
+        else:
+            attn = rfa_hip.forward(q, k, v)
+        return attn.to(ctx.in_dtypes[2])
 
     @staticmethod
     def backward(ctx, grad_attn: Tensor):
-        q, k, v = ctx.saved_tensors
-        gq, gk, gv = rfa_hip.backward(q, k, v, _as_kernel_input(grad_attn))
+        q, k, v, seg_totals = ctx.saved_tensors
+        gq, gk, gv = rfa_hip.backward_saved(q, k, v, _as_kernel_input(grad_attn), seg_totals)
         dq, dk, dv = ctx.in_dtypes
         return gq.to(dq), gk.to(dk), gv.to(dv)

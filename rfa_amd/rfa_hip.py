@@ -77,6 +77,46 @@ def forward(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
     return out
 
 
+def forward_save(q: Tensor, k: Tensor, v: Tensor):
+    """(attn, saved): forward that also returns the per-segment state totals for backward_saved."""
+    _check_qkv(q, k, v)
+    lib = _lib.load()
+    T, N, K = q.shape
+    d = v.shape[2]
+    out = torch.empty_like(v)
+    with torch.cuda.device(q.device):
+        nbytes = lib.rfa_causal_forward_workspace_bytes(T, N, K, d)
+        sbytes = lib.rfa_causal_saved_state_bytes(T, N, K, d)
+        ws = _workspace(nbytes, q.device)
+        saved = _workspace(sbytes, q.device)
+        _lib.check(lib.rfa_causal_forward_save(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                               saved.data_ptr(), sbytes, T, N, K, d, ws.data_ptr(), nbytes,
+                                               _stream_ptr(q.device)))
+    return out, saved
+
+
+def backward_saved(q: Tensor, k: Tensor, v: Tensor, grad_attn: Tensor, saved: Tensor) -> List[Tensor]:
+    """backward() that reuses the segment totals returned by forward_save for the same q, k, v."""
+    _check_qkv(q, k, v)
+    _check_half_cuda("grad_attn", grad_attn, 3)
+    _require(grad_attn.shape == v.shape, ValueError,
+             f"grad_attn {tuple(grad_attn.shape)} must match v {tuple(v.shape)}")
+    _require(saved.is_cuda and saved.dtype == torch.uint8 and saved.is_contiguous(), TypeError,
+             "saved must be the byte buffer returned by forward_save")
+    lib = _lib.load()
+    T, N, K = q.shape
+    d = v.shape[2]
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    with torch.cuda.device(q.device):
+        nbytes = lib.rfa_causal_backward_workspace_bytes(T, N, K, d)
+        ws = _workspace(nbytes, q.device)
+        _lib.check(lib.rfa_causal_backward_saved(q.data_ptr(), k.data_ptr(), v.data_ptr(), grad_attn.data_ptr(),
+                                                 saved.data_ptr(), saved.numel(), dq.data_ptr(), dk.data_ptr(),
+                                                 dv.data_ptr(), T, N, K, d, ws.data_ptr(), nbytes,
+                                                 _stream_ptr(q.device)))
+    return [dq, dk, dv]
+
+
 def backward(q: Tensor, k: Tensor, v: Tensor, grad_attn: Tensor) -> List[Tensor]:
     """[grad_q, grad_k, grad_v] of causal RFA.
 

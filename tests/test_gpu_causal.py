@@ -84,3 +84,15 @@ def test_backward_matches_oracle(T, B, H, d, D):
 def test_selftest_layout():
     from rfa_amd import rfa_hip
     rfa_hip.selftest_layout()
+
+
+@pytest.mark.parametrize("T,B,H,d,D", [(640, 1, 2, 64, 64), (100, 2, 1, 64, 64), (1024, 2, 8, 64, 64), (300, 1, 2, 128, 64)])
+def test_saved_state_pair_equals_plain_pair(T, B, H, d, D):
+    """forward_save / backward_saved hand the segment totals from forward to backward; the
+    results must be bit-identical to the plain forward / backward pair."""
+    from rfa_amd import rfa_hip
+    pq, pk, v, g = (t.cuda() for t in _features(T, B, H, d, D, seed=3000 + T))
+    out, saved = rfa_hip.forward_save(pq, pk, v)
+    assert torch.equal(out, rfa_hip.forward(pq, pk, v))
+    for a, b in zip(rfa_hip.backward_saved(pq, pk, v, g, saved), rfa_hip.backward(pq, pk, v, g)):
+        assert torch.equal(a, b)
