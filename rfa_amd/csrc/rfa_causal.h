@@ -803,8 +803,9 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
             chunk_g2r<DH>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
 #pragma unroll
             for (int it = 0; it < ChunkRegs<DH>::kPieces; ++it) {
+                // raw den only: dividing here would wait for the loads issued just above
                 const int r_ = (tid + kThreads * it) / PPRV;
-                inv_den[it] = (r_ < rows) ? 1.0f / den_ws[(int64_t)(t0 + r_) * N + n] : 0.f;
+                inv_den[it] = (r_ < rows) ? den_ws[(int64_t)(t0 + r_) * N + n] : 0.f;
             }
             gz_next = (tid < C && tid < rows) ? gz_ws[(int64_t)(t0 + tid) * N + n] : 0.f;
         } else if (mrow) {
@@ -820,6 +821,9 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
         chunk_r2s<DH>(rv, Vs, LDV, tid);
         if (CAUSAL) {
             chunk_r2s<KD>(rq, Qs, LDQ, tid);
+#pragma unroll
+            for (int it = 0; it < ChunkRegs<DH>::kPieces; ++it)
+                inv_den[it] = inv_den[it] > 0.f ? 1.0f / inv_den[it] : 0.f;   // den >= 1 on valid rows
             chunk_r2s_scaled<DH>(rg, inv_den, Gs, LDV, tid);
             if (tid < C) gzs[tid] = gz_next;
         }
