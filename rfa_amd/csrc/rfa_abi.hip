@@ -134,6 +134,10 @@ Workspace layout_workspace(int64_t T, int64_t N, int K, int d, const ScanPlan& p
     return w;
 }
 
+// wavefronts per workgroup of the scan kernels: 8 where the per-wave share of the fp32
+// state would not fit the register file with 4 (K >= 128 with d = 128)
+constexpr int causal_waves(int KD, int DH) { return (DH >= 128 && KD >= 128) ? 8 : 4; }
+
 template <typename Kern>
 int set_lds(Kern kern, size_t bytes) {
     RFA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -145,19 +149,20 @@ template <int KD, int DH>
 int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, rfa::half_t* out,
                    int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, float* savedS, float* savedZ,
                    hipStream_t st) {
-    using Cfg = rfa::CausalCfg<KD, DH>;
+    constexpr int NW = causal_waves(KD, DH);
+    using Cfg = rfa::CausalCfg<KD, DH, NW>;
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
     // with a saved-state buffer the z totals are written there directly (z has one layout)
     float* wsZ = savedZ ? savedZ : reinterpret_cast<float*>(ws + wl.Z);
     if (p.nseg > 1) {
-        auto kern = rfa::k_segment_state<KD, DH, true>;
+        auto kern = rfa::k_segment_state<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
-        RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
+        RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(64 * NW), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, savedS, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
-    auto kern = rfa::k_causal_fwd<KD, DH, true>;
+    auto kern = rfa::k_causal_fwd<KD, DH, NW, true>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
-    RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kFwdLds, st, q, k, v, out,
+    RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q, k, v, out,
                        wsS, wsZ, T, N, p.nseg, p.seg_len);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -168,7 +173,8 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
                     const rfa::half_t* g, rfa::half_t* dq, rfa::half_t* dk, rfa::half_t* dv, int T, int N,
                     const ScanPlan& p, char* ws, const Workspace& wl, const float* savedS, const float* savedZ,
                     hipStream_t st) {
-    using Cfg = rfa::CausalCfg<KD, DH>;
+    constexpr int NW = causal_waves(KD, DH);
+    using Cfg = rfa::CausalCfg<KD, DH, NW>;
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
     float* wsZ = reinterpret_cast<float*>(ws + wl.Z);
     float* wsR = reinterpret_cast<float*>(ws + wl.R);
@@ -181,21 +187,21 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         inS = savedS;
         inZ = savedZ;
     } else if (p.nseg > 1) {
-        auto kern = rfa::k_segment_state<KD, DH, false>;
+        auto kern = rfa::k_segment_state<KD, DH, NW, false>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
-        RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(rfa::kThreads), Cfg::kSegStateLds, st,
+        RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(64 * NW), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     {
-        auto kern = rfa::k_causal_bwd_dq<KD, DH, true>;
+        auto kern = rfa::k_causal_bwd_dq<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDqLds)) return rc;
-        RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDqLds, st, q, k, v, g,
+        RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDqLds, st, q, k, v, g,
                            dq, inS, inZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
     }
     {
-        auto kern = rfa::k_causal_bwd_dkdv<KD, DH, true>;
+        auto kern = rfa::k_causal_bwd_dkdv<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
-        RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDkLds, st, q, k, v, g,
+        RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDkLds, st, q, k, v, g,
                            dk, dv, wsR, wsr, den, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
     }
     RFA_HIP_TRY(hipGetLastError());
@@ -220,11 +226,12 @@ ScanPlan make_free_plan(int64_t T, int64_t N) {
 template <int KD, int DH>
 int launch_cross_state(const rfa::half_t* k, const rfa::half_t* v, const uint8_t* mask, int H, float* s,
                        float* z, int T, int N, hipStream_t st) {
-    using Cfg = rfa::CausalCfg<KD, DH>;
+    constexpr int NW = causal_waves(KD, DH);
+    using Cfg = rfa::CausalCfg<KD, DH, NW>;
     const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
-    auto kern = rfa::k_segment_state<KD, DH, false>;
+    auto kern = rfa::k_segment_state<KD, DH, NW, false>;
     if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
-    RFA_LAUNCH(SEG_STATE, kern, dim3(N), dim3(rfa::kThreads), Cfg::kSegStateLds, st, k, v, mask, H, s, z,
+    RFA_LAUNCH(SEG_STATE, kern, dim3(N), dim3(64 * NW), Cfg::kSegStateLds, st, k, v, mask, H, s, z,
                (float*)nullptr, T, N, 1, 1, seg_len);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -233,11 +240,12 @@ int launch_cross_state(const rfa::half_t* k, const rfa::half_t* v, const uint8_t
 template <int KD, int DH>
 int launch_cross_readout(const rfa::half_t* q, const float* s, const float* z, rfa::half_t* out, int T, int N,
                          hipStream_t st) {
-    using Cfg = rfa::CausalCfg<KD, DH>;
+    constexpr int NW = causal_waves(KD, DH);
+    using Cfg = rfa::CausalCfg<KD, DH, NW>;
     const ScanPlan p = make_free_plan(T, N);
-    auto kern = rfa::k_causal_fwd<KD, DH, false>;
+    auto kern = rfa::k_causal_fwd<KD, DH, NW, false>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
-    RFA_LAUNCH(CROSS_READOUT, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kFwdLds, st, q,
+    RFA_LAUNCH(CROSS_READOUT, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q,
                        (const rfa::half_t*)nullptr, (const rfa::half_t*)nullptr, out, s, z, T, N, p.nseg,
                        p.seg_len);
     RFA_HIP_TRY(hipGetLastError());
@@ -247,11 +255,12 @@ int launch_cross_readout(const rfa::half_t* q, const float* s, const float* z, r
 template <int KD, int DH>
 int launch_cross_readout_bwd(const rfa::half_t* q, const float* s, const float* z, const rfa::half_t* g,
                              rfa::half_t* dq, float* ds, float* dz, int T, int N, hipStream_t st) {
-    using Cfg = rfa::CausalCfg<KD, DH>;
+    constexpr int NW = causal_waves(KD, DH);
+    using Cfg = rfa::CausalCfg<KD, DH, NW>;
     const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
-    auto kern = rfa::k_causal_bwd_dq<KD, DH, false>;
+    auto kern = rfa::k_causal_bwd_dq<KD, DH, NW, false>;
     if (int rc = set_lds(kern, Cfg::kBwdDqLds)) return rc;
-    RFA_LAUNCH(CROSS_READOUT_BWD, kern, dim3(N), dim3(rfa::kThreads), Cfg::kBwdDqLds, st, q, (const rfa::half_t*)nullptr,
+    RFA_LAUNCH(CROSS_READOUT_BWD, kern, dim3(N), dim3(64 * NW), Cfg::kBwdDqLds, st, q, (const rfa::half_t*)nullptr,
                        (const rfa::half_t*)nullptr, g, dq, s, z, ds, dz, (float*)nullptr, (float*)nullptr, T, N,
                        1, seg_len);
     RFA_HIP_TRY(hipGetLastError());
@@ -262,11 +271,12 @@ template <int KD, int DH>
 int launch_cross_state_bwd(const rfa::half_t* k, const rfa::half_t* v, const uint8_t* mask, int H,
                            const float* ds, const float* dz, rfa::half_t* dk, rfa::half_t* dv, int T, int N,
                            hipStream_t st) {
-    using Cfg = rfa::CausalCfg<KD, DH>;
+    constexpr int NW = causal_waves(KD, DH);
+    using Cfg = rfa::CausalCfg<KD, DH, NW>;
     const ScanPlan p = make_free_plan(T, N);
-    auto kern = rfa::k_causal_bwd_dkdv<KD, DH, false>;
+    auto kern = rfa::k_causal_bwd_dkdv<KD, DH, NW, false>;
     if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
-    RFA_LAUNCH(CROSS_STATE_BWD, kern, dim3(N * p.nseg), dim3(rfa::kThreads), Cfg::kBwdDkLds, st,
+    RFA_LAUNCH(CROSS_STATE_BWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDkLds, st,
                        (const rfa::half_t*)nullptr, k, v, (const rfa::half_t*)nullptr, dk, dv, ds, dz,
                        (const float*)nullptr, (const float*)nullptr, mask, H, T, N, p.nseg, p.seg_len);
     RFA_HIP_TRY(hipGetLastError());

@@ -31,19 +31,27 @@
 
 namespace rfa {
 
-template <int KD, int DH>
+// NW = wavefronts per workgroup (4 or 8).  Wave w = 4*half + rb: in the tile phases it
+// works on row (column) block rb of the 64 x 64 chunk matrices and, with 8 waves, on one
+// half of that block's tiles; for the state it owns value columns [w*DS, (w+1)*DS) or
+// feature rows [w*KS, (w+1)*KS).  8 waves halve the per-wave state for the large shapes.
+template <int KD, int DH, int NW = 4>
 struct CausalCfg {
-    static_assert(KD % 64 == 0 && DH % 64 == 0, "KD and DH must be multiples of 64");
+    static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+    static_assert(KD % (16 * NW) == 0 && DH % (16 * NW) == 0, "KD and DH must be multiples of 16*NW");
+    static constexpr int NT = 64 * NW;    // threads per workgroup
+    static constexpr int NH = NW / 4;     // waves sharing one 16-row block in the tile phases
+    static constexpr int JPW = 4 / NH;    // 16 x 16 tiles of that block per wave
     static constexpr int C = kChunk;
     static constexpr int LDQ = KD + lds_pad(KD);
     static constexpr int LDV = DH + lds_pad(DH);
     static constexpr int LDA = C + 8;
-    static constexpr int DS = DH / 4;     // value columns owned by one wave
-    static constexpr int KS = KD / 4;     // feature rows owned by one wave
+    static constexpr int DS = DH / NW;    // value columns owned by one wave
+    static constexpr int KS = KD / NW;    // feature rows owned by one wave
     static constexpr size_t kSegStateLds = (size_t)(C * LDQ + C * LDV) * 2;
-    static constexpr size_t kFwdLds = (size_t)(2 * C * LDQ + C * LDV + C * LDA) * 2 + (KD + C) * 4;
+    static constexpr size_t kFwdLds = (size_t)(2 * C * LDQ + C * LDV + C * LDA) * 2 + (KD + NH * C) * 4;
     static constexpr size_t kBwdDqLds =
-        (size_t)(2 * C * LDQ + 2 * C * LDV + C * LDA) * 2 + (size_t)(KD + 8 * C) * 4;
+        (size_t)(2 * C * LDQ + 2 * C * LDV + C * LDA) * 2 + (size_t)(KD + (2 * NH + NW + 2) * C) * 4;
     static constexpr size_t kBwdDkLds =
         (size_t)(2 * C * LDQ + 2 * C * LDV + 2 * C * LDA) * 2 + (size_t)(KD + C) * 4;
 };
@@ -65,14 +73,15 @@ struct CausalCfg {
 // wave w owns the feature tiles kt in [w*NKTW, (w+1)*NKTW).
 // row_copy (FRAG only, may be NULL) receives a second, row-major copy of the totals: the
 // forward pass of a training step hands it to the backward pass, which then skips this pass.
-template <int KD, int DH, bool FRAG>
-__global__ __launch_bounds__(kThreads) void k_segment_state(
+template <int KD, int DH, int NW, bool FRAG>
+__global__ __launch_bounds__(64 * NW) void k_segment_state(
     const half_t* __restrict__ k, const half_t* __restrict__ v, const uint8_t* __restrict__ pad_mask,
     int H, float* __restrict__ wsS, float* __restrict__ wsZ, float* __restrict__ row_copy, int T, int N,
     int nseg, int nseg_out, int seg_len) {
-    using Cfg = CausalCfg<KD, DH>;
+    using Cfg = CausalCfg<KD, DH, NW>;
+    constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, DS = Cfg::DS;
-    constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / 4;
+    constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / NW;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Ks = reinterpret_cast<half_t*>(smem_raw);
     half_t* Vs = Ks + C * LDQ;
@@ -98,19 +107,19 @@ __global__ __launch_bounds__(kThreads) void k_segment_state(
     for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
     const h8 ones = h8_ones();
 
-    ChunkRegs<KD> rk;
-    ChunkRegs<DH> rv;
-    chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
-    chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
-    if (mrow) chunk_mask_rows<KD>(rk, mrow + t_begin, t_end - t_begin, tid);
+    ChunkRegs<KD, NT> rk;
+    ChunkRegs<DH, NT> rv;
+    chunk_g2r<KD, NT>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
+    chunk_g2r<DH, NT>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
+    if (mrow) chunk_mask_rows<KD, NT>(rk, mrow + t_begin, t_end - t_begin, tid);
     for (int t0 = t_begin; t0 < t_end; t0 += C) {
-        chunk_r2s<KD>(rk, Ks, LDQ, tid);
-        chunk_r2s<DH>(rv, Vs, LDV, tid);
+        chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
+        chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
         __syncthreads();
         if (t0 + C < t_end) {
-            chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, t_end - t0 - C, tid);
-            chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, t_end - t0 - C, tid);
-            if (mrow) chunk_mask_rows<KD>(rk, mrow + t0 + C, t_end - t0 - C, tid);
+            chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, t_end - t0 - C, tid);
+            chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, t_end - t0 - C, tid);
+            if (mrow) chunk_mask_rows<KD, NT>(rk, mrow + t0 + C, t_end - t0 - C, tid);
         }
         h8 bv[NCT][2];
 #pragma unroll
@@ -166,25 +175,28 @@ __global__ __launch_bounds__(kThreads) void k_segment_state(
 // the state is the fixed total S, z of the source (wsS/wsZ hold one state per
 // sequence), there is no intra-chunk term and no update, and the denominator is
 // max(|q.z|, 1); k and v are not read.
-template <int KD, int DH, bool CAUSAL>
-__global__ __launch_bounds__(kThreads) void k_causal_fwd(
+template <int KD, int DH, int NW, bool CAUSAL>
+__global__ __launch_bounds__(64 * NW) void k_causal_fwd(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ, int T,
     int N, int nseg, int seg_len) {
-    using Cfg = CausalCfg<KD, DH>;
+    using Cfg = CausalCfg<KD, DH, NW>;
+    constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = Cfg::DS;
-    constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / 4;
+    constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / NW;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
     half_t* Ks = Qs + C * LDQ;
     half_t* Vs = Ks + C * LDQ;
     half_t* As = Vs + C * LDV;
     float* zs = reinterpret_cast<float*>(As + C * LDA);
-    float* dens = zs + KD;
+    float* dparts = zs + KD;    // [NH][C] partial raw denominators
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
+    const int rb = w & 3, half = w >> 2;   // tile-phase role: 16-row block and which of its tiles
+    constexpr int JPW = Cfg::JPW, NH = Cfg::NH;
     const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
@@ -195,12 +207,12 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
     half_t* ob = out + (int64_t)n * DH;
 
     RFA_TICK_INIT();
-    ChunkRegs<KD> rq, rk;
-    ChunkRegs<DH> rv;
-    chunk_g2r<KD>(rq, qb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
+    ChunkRegs<KD, NT> rq, rk;
+    ChunkRegs<DH, NT> rv;
+    chunk_g2r<KD, NT>(rq, qb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
     if (CAUSAL) {
-        chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
-        chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
+        chunk_g2r<KD, NT>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
+        chunk_g2r<DH, NT>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
     }
 
     // carried state = sum of the totals of all earlier segments (causal: stored in
@@ -240,10 +252,10 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
 
     RFA_TICK(0);
     for (int t0 = t_begin; t0 < t_end; t0 += C) {
-        chunk_r2s<KD>(rq, Qs, LDQ, tid);
+        chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
         if (CAUSAL) {
-            chunk_r2s<KD>(rk, Ks, LDQ, tid);
-            chunk_r2s<DH>(rv, Vs, LDV, tid);
+            chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
+            chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
         }
         if (row == 0) {
 #pragma unroll
@@ -254,43 +266,48 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
         RFA_TICK(2);
         if (t0 + C < t_end) {
             const int rows = t_end - t0 - C;
-            chunk_g2r<KD>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+            chunk_g2r<KD, NT>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
             if (CAUSAL) {
-                chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-                chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+                chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+                chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
             }
         }
 
         RFA_TICK(3);
-        // ---- phase A: wave w computes rows i in [16w, 16w+16) of A (as A^T tiles, m=j, n=i)
+        // ---- phase A: rows i in [16rb, 16rb+16) of A as A^T tiles (m=j, n=i); this wave's
+        // tiles are jt = half*JPW + a (all tiles of the row, branch-free: the last row block
+        // needs them anyway)
         {
-            f4 at[4];
+            f4 at[JPW];
 #pragma unroll
-            for (int jt = 0; jt < 4; ++jt) at[jt] = f4_zero();
+            for (int a = 0; a < JPW; ++a) at[a] = f4_zero();
 #pragma unroll
             for (int ks = 0; ks < (CAUSAL ? KD / 32 : 0); ++ks) {
-                h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
+                h8 bq = row8(Qs, LDQ, 16 * rb + row, ks * 32, G);
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt)   // all four tiles: branch-free, wave 3 needs them anyway
-                    at[jt] = mfma32(row8(Ks, LDQ, 16 * jt + row, ks * 32, G), bq, at[jt]);
+                for (int a = 0; a < JPW; ++a)
+                    at[a] = mfma32(row8(Ks, LDQ, 16 * (half * JPW + a) + row, ks * 32, G), bq, at[a]);
             }
             float part = 0.f;
 #pragma unroll
-            for (int jt = 0; jt < 4; ++jt) {
+            for (int a = 0; a < JPW; ++a) {
+                const int jt = half * JPW + a;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {   // keep j <= i
-                    const bool keep = (jt < w) || (jt == w && 4 * G + e <= row);
-                    at[jt][e] = keep ? at[jt][e] : 0.f;
+                    const bool keep = (jt < rb) || (jt == rb && 4 * G + e <= row);
+                    at[a][e] = keep ? at[a][e] : 0.f;
                 }
-                part += at[jt][0] + at[jt][1] + at[jt][2] + at[jt][3];
+                part += at[a][0] + at[a][1] + at[a][2] + at[a][3];
             }
-            // + q_i . z  (this lane covers features [G*KD/4, (G+1)*KD/4))
+            // + q_i . z : this lane covers features [G*KD/4 + half*QZW, +QZW)
+            constexpr int QZW = KD / 4 / NH;
             f4 qz4 = f4_zero();
 #pragma unroll
-            for (int kk = 0; kk < KD / 4; kk += 8) {
-                h8 qv = *reinterpret_cast<const h8*>(Qs + (16 * w + row) * LDQ + G * (KD / 4) + kk);
-                f4 z0 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk);
-                f4 z1 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk + 4);
+            for (int kk = 0; kk < QZW; kk += 8) {
+                const int k0 = G * (KD / 4) + half * QZW + kk;
+                h8 qv = *reinterpret_cast<const h8*>(Qs + (16 * rb + row) * LDQ + k0);
+                f4 z0 = *reinterpret_cast<const f4*>(zs + k0);
+                f4 z1 = *reinterpret_cast<const f4*>(zs + k0 + 4);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     qz4[e] += (float)qv[e] * z0[e];
@@ -299,11 +316,11 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
             }
             part += (qz4[0] + qz4[1]) + (qz4[2] + qz4[3]);
             part = sum_over_groups(part);
-            if (G == 0) dens[16 * w + row] = fmaxf(CAUSAL ? part : fabsf(part), 1.0f);
+            if (G == 0) dparts[half * C + 16 * rb + row] = part;
             if (CAUSAL) {
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt)
-                    *reinterpret_cast<h4*>(As + (16 * w + row) * LDA + 16 * jt + 4 * G) = to_h4(at[jt]);
+                for (int a = 0; a < JPW; ++a)
+                    *reinterpret_cast<h4*>(As + (16 * rb + row) * LDA + 16 * (half * JPW + a) + 4 * G) = to_h4(at[a]);
             }
         }
         RFA_TICK(4);
@@ -353,7 +370,10 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const int i = 16 * it + row;
-                const float inv = 1.0f / dens[i];
+                float dr = dparts[i];
+#pragma unroll
+                for (int h = 1; h < NH; ++h) dr += dparts[h * C + i];
+                const float inv = 1.0f / fmaxf(CAUSAL ? dr : fabsf(dr), 1.0f);
                 if (t0 + i < t_end) {
 #pragma unroll
                     for (int ct = 0; ct < NCT; ++ct) {
@@ -398,13 +418,14 @@ __global__ __launch_bounds__(kThreads) void k_causal_fwd(
 // gz = -e/den^2 * sign(q.z) * [|q.z| > 1], dQ = Y/den + gz z^T, and the totals
 // dR, dr written to wsR/wsr (one per sequence, nseg must be 1) are the gradients
 // of the state (dS, dz).  k and v are not read; den_ws/gz_ws are not written.
-template <int KD, int DH, bool CAUSAL>
-__global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
+template <int KD, int DH, int NW, bool CAUSAL>
+__global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, half_t* __restrict__ dq, const float* __restrict__ wsS,
     const float* __restrict__ wsZ, float* __restrict__ wsR, float* __restrict__ wsr,
     float* __restrict__ den_ws, float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len) {
-    using Cfg = CausalCfg<KD, DH>;
+    using Cfg = CausalCfg<KD, DH, NW>;
+    constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS;
     constexpr int NKT = KS / 16, NCT = DH / 16;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -414,15 +435,17 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
     half_t* Gs = Vs + C * LDV;
     half_t* Ps = Gs + C * LDV;
     float* zs = reinterpret_cast<float*>(Ps + C * LDA);
-    float* drs = zs + KD;       // den_raw per row
-    float* e1s = drs + C;       // rowsum(A*X)
-    float* e2p = e1s + C;       // [4][C] per-wave partial rowsum(Q*Y)
-    float* dens = e2p + 4 * C;
+    float* drs = zs + KD;        // [NH][C] partial den_raw per row
+    float* e1s = drs + Cfg::NH * C;   // [NH][C] partial rowsum(A*X)
+    float* e2p = e1s + Cfg::NH * C;   // [NW][C] per-wave partial rowsum(Q*Y)
+    float* dens = e2p + NW * C;
     float* gzs = dens + C;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
+    const int rb = w & 3, half = w >> 2;   // tile-phase role: 16-row block and which of its tiles
+    constexpr int JPW = Cfg::JPW, NH = Cfg::NH;
     const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
@@ -459,24 +482,24 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
             zacc[kt] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * state_stride + s) * KD + w * KS + 16 * kt + 4 * G);
     }
 
-    ChunkRegs<KD> rq, rk;
-    ChunkRegs<DH> rv, rg;
+    ChunkRegs<KD, NT> rq, rk;
+    ChunkRegs<DH, NT> rv, rg;
     {
         const int rows = t_end - t_begin;
-        chunk_g2r<KD>(rq, qb + (int64_t)t_begin * k_stride, k_stride, rows, tid);
-        chunk_g2r<DH>(rg, gb + (int64_t)t_begin * v_stride, v_stride, rows, tid);
+        chunk_g2r<KD, NT>(rq, qb + (int64_t)t_begin * k_stride, k_stride, rows, tid);
+        chunk_g2r<DH, NT>(rg, gb + (int64_t)t_begin * v_stride, v_stride, rows, tid);
         if (CAUSAL) {
-            chunk_g2r<KD>(rk, kb + (int64_t)t_begin * k_stride, k_stride, rows, tid);
-            chunk_g2r<DH>(rv, vb + (int64_t)t_begin * v_stride, v_stride, rows, tid);
+            chunk_g2r<KD, NT>(rk, kb + (int64_t)t_begin * k_stride, k_stride, rows, tid);
+            chunk_g2r<DH, NT>(rv, vb + (int64_t)t_begin * v_stride, v_stride, rows, tid);
         }
     }
 
     for (int t0 = t_begin; t0 < t_end; t0 += C) {
-        chunk_r2s<KD>(rq, Qs, LDQ, tid);
-        chunk_r2s<DH>(rg, Gs, LDV, tid);
+        chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
+        chunk_r2s<DH, NT>(rg, Gs, LDV, tid);
         if (CAUSAL) {
-            chunk_r2s<KD>(rk, Ks, LDQ, tid);
-            chunk_r2s<DH>(rv, Vs, LDV, tid);
+            chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
+            chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
         }
         if (row == 0) {
 #pragma unroll
@@ -485,52 +508,55 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
         __syncthreads();
         if (t0 + C < t_end) {
             const int rows = t_end - t0 - C;
-            chunk_g2r<KD>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-            chunk_g2r<DH>(rg, gb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+            chunk_g2r<KD, NT>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+            chunk_g2r<DH, NT>(rg, gb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
             if (CAUSAL) {
-                chunk_g2r<KD>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-                chunk_g2r<DH>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+                chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+                chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
             }
         }
 
         // ---- phase A
-        f4 xt[4];           // X^T tiles (m=j, n=i) for rows i of this wave, kept for phase C
+        f4 xt[JPW];         // X^T tiles (m=j, n=i): rows i of block rb, tiles jt = half*JPW + a; kept for phase C
         f4 yt[NKT][4];      // Y^T tiles (m=k, n=i), k in this wave's slice, all i
         {
-            f4 at[4];
+            f4 at[JPW];
 #pragma unroll
-            for (int jt = 0; jt < 4; ++jt) { at[jt] = f4_zero(); xt[jt] = f4_zero(); }
+            for (int a = 0; a < JPW; ++a) { at[a] = f4_zero(); xt[a] = f4_zero(); }
 #pragma unroll
             for (int ks = 0; ks < (CAUSAL ? KD / 32 : 0); ++ks) {
-                h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
+                h8 bq = row8(Qs, LDQ, 16 * rb + row, ks * 32, G);
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt)   // all four tiles, branch-free
-                    at[jt] = mfma32(row8(Ks, LDQ, 16 * jt + row, ks * 32, G), bq, at[jt]);
+                for (int a = 0; a < JPW; ++a)   // all tiles of the row block, branch-free
+                    at[a] = mfma32(row8(Ks, LDQ, 16 * (half * JPW + a) + row, ks * 32, G), bq, at[a]);
             }
 #pragma unroll
             for (int cs = 0; cs < (CAUSAL ? DH / 32 : 0); ++cs) {
-                h8 bg = row8(Gs, LDV, 16 * w + row, cs * 32, G);
+                h8 bg = row8(Gs, LDV, 16 * rb + row, cs * 32, G);
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt)
-                    xt[jt] = mfma32(row8(Vs, LDV, 16 * jt + row, cs * 32, G), bg, xt[jt]);
+                for (int a = 0; a < JPW; ++a)
+                    xt[a] = mfma32(row8(Vs, LDV, 16 * (half * JPW + a) + row, cs * 32, G), bg, xt[a]);
             }
             float part_d = 0.f, part_e = 0.f;
 #pragma unroll
-            for (int jt = 0; jt < 4; ++jt) {
+            for (int a = 0; a < JPW; ++a) {
+                const int jt = half * JPW + a;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {   // keep j <= i
-                    const bool keep = (jt < w) || (jt == w && 4 * G + e <= row);
-                    at[jt][e] = keep ? at[jt][e] : 0.f;
-                    part_d += at[jt][e];
-                    part_e += at[jt][e] * xt[jt][e];
+                    const bool keep = (jt < rb) || (jt == rb && 4 * G + e <= row);
+                    at[a][e] = keep ? at[a][e] : 0.f;
+                    part_d += at[a][e];
+                    part_e += at[a][e] * xt[a][e];
                 }
             }
+            constexpr int QZW = KD / 4 / NH;   // this lane covers features [G*KD/4 + half*QZW, +QZW)
             f4 qz4 = f4_zero();
 #pragma unroll
-            for (int kk = 0; kk < KD / 4; kk += 8) {
-                h8 qv = *reinterpret_cast<const h8*>(Qs + (16 * w + row) * LDQ + G * (KD / 4) + kk);
-                f4 z0 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk);
-                f4 z1 = *reinterpret_cast<const f4*>(zs + G * (KD / 4) + kk + 4);
+            for (int kk = 0; kk < QZW; kk += 8) {
+                const int k0 = G * (KD / 4) + half * QZW + kk;
+                h8 qv = *reinterpret_cast<const h8*>(Qs + (16 * rb + row) * LDQ + k0);
+                f4 z0 = *reinterpret_cast<const f4*>(zs + k0);
+                f4 z1 = *reinterpret_cast<const f4*>(zs + k0 + 4);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     qz4[e] += (float)qv[e] * z0[e];
@@ -541,8 +567,8 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
             part_d = sum_over_groups(part_d);
             part_e = sum_over_groups(part_e);
             if (G == 0) {
-                drs[16 * w + row] = part_d;
-                e1s[16 * w + row] = part_e;
+                drs[half * C + 16 * rb + row] = part_d;
+                e1s[half * C + 16 * rb + row] = part_e;
             }
 
 #pragma unroll
@@ -582,9 +608,14 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
 
         // ---- phase B: denominators and d(qz) for the 64 rows of the chunk
         if (tid < C) {
-            const float dr = drs[tid];
+            float dr = drs[tid], e = e1s[tid];
+#pragma unroll
+            for (int h = 1; h < NH; ++h) { dr += drs[h * C + tid]; e += e1s[h * C + tid]; }
+            float e2sum = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) e2sum += e2p[ww * C + tid];
+            e += e2sum;
             const float den = fmaxf(CAUSAL ? dr : fabsf(dr), 1.0f);
-            const float e = e1s[tid] + ((e2p[tid] + e2p[C + tid]) + (e2p[2 * C + tid] + e2p[3 * C + tid]));
             float gz;
             if (CAUSAL) {
                 gz = (dr > 1.0f) ? -e / (den * den) : 0.f;
@@ -602,23 +633,24 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
 
         // ---- phase C: P rows of this wave; G <- G/den in place
         {
-            const int i = 16 * w + row;
+            const int i = 16 * rb + row;
             const float inv = 1.0f / dens[i];
             const float gzi = gzs[i];
 #pragma unroll
-            for (int jt = 0; jt < (CAUSAL ? 4 : 0); ++jt) {
+            for (int a = 0; a < (CAUSAL ? JPW : 0); ++a) {
+                const int jt = half * JPW + a;
                 h4 pv;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int j = 16 * jt + 4 * G + e;
-                    pv[e] = (j <= i) ? (half_t)(xt[jt][e] * inv + gzi) : (half_t)0.f;
+                    pv[e] = (j <= i) ? (half_t)(xt[a][e] * inv + gzi) : (half_t)0.f;
                 }
                 *reinterpret_cast<h4*>(Ps + i * LDA + 16 * jt + 4 * G) = pv;
             }
             constexpr int PPR = DH / 8;
 #pragma unroll
-            for (int it = 0; it < ChunkRegs<DH>::kPieces; ++it) {
-                const int p = tid + kThreads * it;
+            for (int it = 0; it < ChunkRegs<DH, NT>::kPieces; ++it) {
+                const int p = tid + NT * it;
                 const int r_ = p / PPR, c8 = p % PPR;
                 const float sc = 1.0f / dens[r_];
                 h8 x = *reinterpret_cast<const h8*>(Gs + r_ * LDV + c8 * 8);
@@ -720,14 +752,15 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dq(
 // dV = K dS; q, g, den_ws, gz_ws are not read.  pad_mask ([B, T] bytes, may be
 // NULL; H heads per batch entry) marks padded keys: their phi_k rows are read as
 // zero and their dK rows are written as zero (the gradient of masked_fill).
-template <int KD, int DH, bool CAUSAL>
-__global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
+template <int KD, int DH, int NW, bool CAUSAL>
+__global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, half_t* __restrict__ dk, half_t* __restrict__ dv,
     const float* __restrict__ wsR, const float* __restrict__ wsr, const float* __restrict__ den_ws,
     const float* __restrict__ gz_ws, const uint8_t* __restrict__ pad_mask, int H, int T, int N,
     int nseg, int seg_len) {
-    using Cfg = CausalCfg<KD, DH>;
+    using Cfg = CausalCfg<KD, DH, NW>;
+    constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS, DS = Cfg::DS;
     constexpr int NKT = KS / 16, NCT = DH / 16;      // RT tiles
     constexpr int NKT2 = KD / 16, NCT2 = DS / 16;    // RR tiles
@@ -744,6 +777,8 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
+    const int rb = w & 3, half = w >> 2;   // tile-phase role: 16-row block and which of its tiles
+    constexpr int JPW = Cfg::JPW, NH = Cfg::NH;
     const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
@@ -789,27 +824,27 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
             racc[kt] += *reinterpret_cast<const f4*>(wsr + (int64_t)(n * state_stride + s) * KD + w * KS + 16 * kt + 4 * G);
     }
 
-    ChunkRegs<KD> rq, rk;
-    ChunkRegs<DH> rv, rg;
-    float inv_den[ChunkRegs<DH>::kPieces];
+    ChunkRegs<KD, NT> rq, rk;
+    ChunkRegs<DH, NT> rv, rg;
+    float inv_den[ChunkRegs<DH, NT>::kPieces];
     float gz_next = 0.f;
     constexpr int PPRV = DH / 8;
     auto prefetch = [&](int t0) {
         const int rows = t_end - t0;
-        chunk_g2r<KD>(rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
-        chunk_g2r<DH>(rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+        chunk_g2r<KD, NT>(rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<DH, NT>(rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
         if (CAUSAL) {
-            chunk_g2r<KD>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
-            chunk_g2r<DH>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+            chunk_g2r<KD, NT>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+            chunk_g2r<DH, NT>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
 #pragma unroll
-            for (int it = 0; it < ChunkRegs<DH>::kPieces; ++it) {
+            for (int it = 0; it < ChunkRegs<DH, NT>::kPieces; ++it) {
                 // raw den only: dividing here would wait for the loads issued just above
-                const int r_ = (tid + kThreads * it) / PPRV;
+                const int r_ = (tid + NT * it) / PPRV;
                 inv_den[it] = (r_ < rows) ? den_ws[(int64_t)(t0 + r_) * N + n] : 0.f;
             }
             gz_next = (tid < C && tid < rows) ? gz_ws[(int64_t)(t0 + tid) * N + n] : 0.f;
         } else if (mrow) {
-            chunk_mask_rows<KD>(rk, mrow + t0, rows, tid);
+            chunk_mask_rows<KD, NT>(rk, mrow + t0, rows, tid);
         }
     };
 
@@ -817,14 +852,14 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
     prefetch(t_begin + (n_chunks - 1) * C);
     for (int ci = n_chunks - 1; ci >= 0; --ci) {
         const int t0 = t_begin + ci * C;
-        chunk_r2s<KD>(rk, Ks, LDQ, tid);
-        chunk_r2s<DH>(rv, Vs, LDV, tid);
+        chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
+        chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
         if (CAUSAL) {
-            chunk_r2s<KD>(rq, Qs, LDQ, tid);
+            chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
 #pragma unroll
-            for (int it = 0; it < ChunkRegs<DH>::kPieces; ++it)
+            for (int it = 0; it < ChunkRegs<DH, NT>::kPieces; ++it)
                 inv_den[it] = inv_den[it] > 0.f ? 1.0f / inv_den[it] : 0.f;   // den >= 1 on valid rows
-            chunk_r2s_scaled<DH>(rg, inv_den, Gs, LDV, tid);
+            chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
             if (tid < C) gzs[tid] = gz_next;
         }
         if (row == 0) {
@@ -834,35 +869,36 @@ __global__ __launch_bounds__(kThreads) void k_causal_bwd_dkdv(
         __syncthreads();
         if (ci > 0) prefetch(t0 - C);
 
-        // ---- phase A: wave w computes columns j in [16w, 16w+16) of A and P (tiles m=i, n=j)
+        // ---- phase A: columns j in [16rb, 16rb+16) of A and P (tiles m=i, n=j)
         if (CAUSAL) {
-            f4 a_[4], p_[4];
+            f4 a_[JPW], p_[JPW];   // tiles it = half*JPW + a of column block rb
 #pragma unroll
-            for (int it = 0; it < 4; ++it) { a_[it] = f4_zero(); p_[it] = f4_zero(); }
+            for (int a = 0; a < JPW; ++a) { a_[a] = f4_zero(); p_[a] = f4_zero(); }
 #pragma unroll
             for (int ks = 0; ks < KD / 32; ++ks) {
-                h8 bk = row8(Ks, LDQ, 16 * w + row, ks * 32, G);
+                h8 bk = row8(Ks, LDQ, 16 * rb + row, ks * 32, G);
 #pragma unroll
-                for (int it = 0; it < 4; ++it)   // all four tiles, branch-free
-                    a_[it] = mfma32(row8(Qs, LDQ, 16 * it + row, ks * 32, G), bk, a_[it]);
+                for (int a = 0; a < JPW; ++a)   // all tiles of the column block, branch-free
+                    a_[a] = mfma32(row8(Qs, LDQ, 16 * (half * JPW + a) + row, ks * 32, G), bk, a_[a]);
             }
 #pragma unroll
             for (int cs = 0; cs < DH / 32; ++cs) {
-                h8 bv = row8(Vs, LDV, 16 * w + row, cs * 32, G);
+                h8 bv = row8(Vs, LDV, 16 * rb + row, cs * 32, G);
 #pragma unroll
-                for (int it = 0; it < 4; ++it)
-                    p_[it] = mfma32(row8(Gs, LDV, 16 * it + row, cs * 32, G), bv, p_[it]);
+                for (int a = 0; a < JPW; ++a)
+                    p_[a] = mfma32(row8(Gs, LDV, 16 * (half * JPW + a) + row, cs * 32, G), bv, p_[a]);
             }
-            const int j = 16 * w + row;
+            const int j = 16 * rb + row;
 #pragma unroll
-            for (int it = 0; it < 4; ++it) {
+            for (int a = 0; a < JPW; ++a) {
+                const int it = half * JPW + a;
                 h4 av, pv;
                 f4 gzv = *reinterpret_cast<const f4*>(gzs + 16 * it + 4 * G);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int i = 16 * it + 4 * G + e;
-                    av[e] = (i >= j) ? (half_t)a_[it][e] : (half_t)0.f;
-                    pv[e] = (i >= j) ? (half_t)(p_[it][e] + gzv[e]) : (half_t)0.f;
+                    av[e] = (i >= j) ? (half_t)a_[a][e] : (half_t)0.f;
+                    pv[e] = (i >= j) ? (half_t)(p_[a][e] + gzv[e]) : (half_t)0.f;
                 }
                 *reinterpret_cast<h4*>(ATs + j * LDA + 16 * it + 4 * G) = av;
                 *reinterpret_cast<h4*>(PTs + j * LDA + 16 * it + 4 * G) = pv;

@@ -152,29 +152,29 @@ __device__ __forceinline__ float sum_over_groups(float x) {
 // sequence, F halves per step; in HBM consecutive steps are `row_stride` halves
 // apart ([T, N, F] time-major layout).
 // ---------------------------------------------------------------------------
-template <int F>
+template <int F, int NT = kThreads>
 struct ChunkRegs {
-    static constexpr int kPieces = kChunk * F / 8 / kThreads;   // 16-byte pieces per thread
-    static_assert(kPieces >= 1, "feature width too small for 256 threads");
+    static constexpr int kPieces = kChunk * F / 8 / NT;   // 16-byte pieces per thread
+    static_assert(kPieces >= 1, "feature width too small for this many threads");
     uint4 v[kPieces];
 };
 
-template <int F>
-__device__ __forceinline__ void chunk_g2r(ChunkRegs<F>& r, const half_t* __restrict__ base,
+template <int F, int NT = kThreads>
+__device__ __forceinline__ void chunk_g2r(ChunkRegs<F, NT>& r, const half_t* __restrict__ base,
                                           int64_t row_stride, int rows_valid, int tid) {
     constexpr int PPR = F / 8;
     if (rows_valid >= kChunk) {   // full chunk (uniform): no per-lane predication
 #pragma unroll
-        for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
-            const int p = tid + kThreads * it;
+        for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
+            const int p = tid + NT * it;
             const int row = p / PPR, c8 = p % PPR;
             r.v[it] = *reinterpret_cast<const uint4*>(base + (int64_t)row * row_stride + c8 * 8);
         }
         return;
     }
 #pragma unroll
-    for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
-        const int p = tid + kThreads * it;
+    for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
+        const int p = tid + NT * it;
         const int row = p / PPR, c8 = p % PPR;
         if (row < rows_valid) {
             r.v[it] = *reinterpret_cast<const uint4*>(base + (int64_t)row * row_stride + c8 * 8);
@@ -184,37 +184,37 @@ __device__ __forceinline__ void chunk_g2r(ChunkRegs<F>& r, const half_t* __restr
     }
 }
 
-template <int F>
-__device__ __forceinline__ void chunk_r2s(const ChunkRegs<F>& r, half_t* Xs, int ld, int tid) {
+template <int F, int NT = kThreads>
+__device__ __forceinline__ void chunk_r2s(const ChunkRegs<F, NT>& r, half_t* Xs, int ld, int tid) {
     constexpr int PPR = F / 8;
 #pragma unroll
-    for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
-        const int p = tid + kThreads * it;
+    for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
+        const int p = tid + NT * it;
         const int row = p / PPR, c8 = p % PPR;
         *reinterpret_cast<uint4*>(Xs + row * ld + c8 * 8) = r.v[it];
     }
 }
 
 // zero the rows whose mask byte is non-zero (mask already offset to the chunk's first step)
-template <int F>
-__device__ __forceinline__ void chunk_mask_rows(ChunkRegs<F>& r, const uint8_t* __restrict__ mask,
+template <int F, int NT = kThreads>
+__device__ __forceinline__ void chunk_mask_rows(ChunkRegs<F, NT>& r, const uint8_t* __restrict__ mask,
                                                 int rows_valid, int tid) {
     constexpr int PPR = F / 8;
 #pragma unroll
-    for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
-        const int row = (tid + kThreads * it) / PPR;
+    for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
+        const int row = (tid + NT * it) / PPR;
         if (row < rows_valid && mask[row]) r.v[it] = make_uint4(0u, 0u, 0u, 0u);
     }
 }
 
 // same, each row multiplied by scale[piece] (fp32) before the store
-template <int F>
-__device__ __forceinline__ void chunk_r2s_scaled(const ChunkRegs<F>& r, const float* scale,
+template <int F, int NT = kThreads>
+__device__ __forceinline__ void chunk_r2s_scaled(const ChunkRegs<F, NT>& r, const float* scale,
                                                  half_t* Xs, int ld, int tid) {
     constexpr int PPR = F / 8;
 #pragma unroll
-    for (int it = 0; it < ChunkRegs<F>::kPieces; ++it) {
-        const int p = tid + kThreads * it;
+    for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
+        const int p = tid + NT * it;
         const int row = p / PPR, c8 = p % PPR;
         union { uint4 u; h8 h; } x;
         x.u = r.v[it];
