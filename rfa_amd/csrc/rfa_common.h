@@ -140,6 +140,18 @@ __device__ __forceinline__ void f8_to_operand(const f4& a, const f4& b, h8& hi, 
     }
 }
 
+// sin and cos of x (radians) on the hardware transcendental unit: v_sin_f32 / v_cos_f32
+// take their argument in turns.  The argument of the feature map is u = w . x^ with
+// |u| rarely above 10; the error of x * (1/2pi) in fp32 (2^-24 relative) and of the unit
+// itself stay below 1e-6 absolute there, far inside the fp16 resolution of the outputs
+// (3e-4 relative at |phi| ~ 0.1).  About ten times fewer instructions than sincosf.
+__device__ __forceinline__ void fast_sincos(float x, float& s, float& c) {
+    float t = x * 0.15915494309189535f;
+    t = t - floorf(t);                  // v_fract: keeps the unit inside its valid range
+    s = __builtin_amdgcn_sinf(t);
+    c = __builtin_amdgcn_cosf(t);
+}
+
 // sum over the four 16-lane groups (lanes i, i+16, i+32, i+48)
 __device__ __forceinline__ float sum_over_groups(float x) {
     x += __shfl_xor(x, 16, 64);

@@ -56,7 +56,7 @@ __device__ __forceinline__ void decode_feature_map(float* phi_q, float* phi_k,
     if (part == 0) {
         const float u = dot / (sqrtf(ss) + 1e-3f);
         float s_, c_;
-        sincosf(u, &s_, &c_);
+        fast_sincos(u, s_, c_);
         float* dst = (vec == 0 ? phi_q : phi_k);
         dst[j] = scale * s_;
         dst[D + j] = scale * c_;

@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_fwd(
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             float s_, c_;
-            sincosf(acc[e] * inv, &s_, &c_);
+            fast_sincos(acc[e] * inv, s_, c_);
             sv[e] = (half_t)(scale * s_);
             cv[e] = (half_t)(scale * c_);
         }
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 float s_, c_;
-                sincosf(acc[e] * inv, &s_, &c_);
+                fast_sincos(acc[e] * inv, s_, c_);
                 du[e] = (half_t)(scale * (c_ * (float)gs[e] - s_ * (float)gc[e]) * inv);
             }
             *reinterpret_cast<h4*>(Us + lr * LDU + 16 * jt + 4 * G) = du;

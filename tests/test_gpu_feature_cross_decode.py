@@ -38,7 +38,7 @@ def test_feature_map_forward(L, B, H, d, D):
     print(f"phi fwd L={L} B={B} H={H} d={d} D={D}", flush=True)
     got = rfa_hip.feature_map_forward(x.cuda(), w.cuda(), O.SCALE).float().cpu()
     want = O.random_project(x.float(), w.float())
-    assert (got - want).abs().max().item() <= 3e-4     # |phi| <= 0.1: half an fp16 ulp is 3e-5
+    assert (got - want).abs().max().item() <= 7e-5     # |phi| <= 0.1: one fp16 ulp there is 6.1e-5
     assert torch.equal(got[0, 0, 0, :D], torch.zeros(D))
 
 
