@@ -25,7 +25,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # MFMA accumulators in VGPRs: the state tiles are re-read as operands every chunk,
     # AGPR residency would cost a v_accvgpr move per element per use
-    # "-mllvm", "-amdgpu-mfma-vgpr-form=1",
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
 
 
