@@ -137,6 +137,9 @@ Workspace layout_workspace(int64_t T, int64_t N, int K, int d, const ScanPlan& p
 // wavefronts per workgroup of the scan kernels: 8 where the per-wave share of the fp32
 // state would not fit the register file with 4 (K >= 128 with d = 128)
 constexpr int causal_waves(int KD, int DH) { return (DH >= 128 && KD >= 128) ? 8 : 4; }
+// the dQ sweep owns feature-row slices only, so it can run 8 waves (two per SIMD) whenever
+// K >= 128
+constexpr int dq_waves(int KD, int DH) { return KD >= 128 ? 8 : 4; }
 
 template <typename Kern>
 int set_lds(Kern kern, size_t bytes) {
@@ -193,9 +196,11 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     {
-        auto kern = rfa::k_causal_bwd_dq<KD, DH, NW, true>;
-        if (int rc = set_lds(kern, Cfg::kBwdDqLds)) return rc;
-        RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDqLds, st, q, k, v, g,
+        constexpr int NWQ = dq_waves(KD, DH);
+        using CfgQ = rfa::CausalCfg<KD, DH, NWQ>;
+        auto kern = rfa::k_causal_bwd_dq<KD, DH, NWQ, true>;
+        if (int rc = set_lds(kern, CfgQ::kBwdDqLds)) return rc;
+        RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqLds, st, q, k, v, g,
                            dq, inS, inZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
     }
     {

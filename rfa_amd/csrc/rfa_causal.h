@@ -38,7 +38,9 @@ namespace rfa {
 template <int KD, int DH, int NW = 4>
 struct CausalCfg {
     static_assert(NW == 4 || NW == 8, "4 or 8 waves");
-    static_assert(KD % (16 * NW) == 0 && DH % (16 * NW) == 0, "KD and DH must be multiples of 16*NW");
+    static_assert(KD % 64 == 0 && DH % 64 == 0, "KD and DH must be multiples of 64");
+    // kernels owning value-column slices need DH % (16*NW) == 0, those owning feature-row
+    // slices KD % (16*NW) == 0; each kernel asserts what it uses
     static constexpr int NT = 64 * NW;    // threads per workgroup
     static constexpr int NH = NW / 4;     // waves sharing one 16-row block in the tile phases
     static constexpr int JPW = 4 / NH;    // 16 x 16 tiles of that block per wave
@@ -82,6 +84,7 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, DS = Cfg::DS;
     constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / NW;
+    static_assert(DH % (16 * NW) == 0 && NKT % NW == 0, "shape does not split over the waves");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Ks = reinterpret_cast<half_t*>(smem_raw);
     half_t* Vs = Ks + C * LDQ;
@@ -184,6 +187,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = Cfg::DS;
     constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / NW;
+    static_assert(DH % (16 * NW) == 0 && NKT % NW == 0, "shape does not split over the waves");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
     half_t* Ks = Qs + C * LDQ;
@@ -428,6 +432,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS;
     constexpr int NKT = KS / 16, NCT = DH / 16;
+    static_assert(KD % (16 * NW) == 0, "feature rows do not split over the waves");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
     half_t* Ks = Qs + C * LDQ;
@@ -764,6 +769,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS, DS = Cfg::DS;
     constexpr int NKT = KS / 16, NCT = DH / 16;      // RT tiles
     constexpr int NKT2 = KD / 16, NCT2 = DS / 16;    // RR tiles
+    static_assert(KD % (16 * NW) == 0 && DH % (16 * NW) == 0, "shape does not split over the waves");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
     half_t* Ks = Qs + C * LDQ;
