@@ -332,7 +332,8 @@ int launch_feature_bwd(const rfa::half_t* x, const rfa::half_t* w, const rfa::ha
     if (int rc = set_lds(kern, Cfg::kBwdLds)) return rc;
     RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, part, R, H, scale);
     const int64_t elems = (int64_t)H * D * DH;
-    RFA_LAUNCH(FEATURE_DW_REDUCE, rfa::k_feature_map_dw_reduce, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, st,
+    static_assert((D * DH) % 256 == 0, "dw reduce works on blocks of 256 elements");
+    RFA_LAUNCH(FEATURE_DW_REDUCE, rfa::k_feature_map_dw_reduce, dim3((unsigned)(elems / 256)), dim3(rfa::kThreads), 0, st,
                        part, dw, nblk, elems);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;

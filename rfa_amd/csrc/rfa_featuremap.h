@@ -19,9 +19,70 @@ struct FeatureCfg {
     static_assert(D % 32 == 0 && DH % 64 == 0, "D multiple of 32, DH multiple of 64");
     static constexpr int LDW = DH + lds_pad(DH);
     static constexpr int LDU = D + lds_pad(D);
-    static constexpr size_t kFwdLds = (size_t)D * LDW * 2;
-    static constexpr size_t kBwdLds = (size_t)(D * LDW + 64 * LDW + 64 * LDU) * 2;
+    // staging rows of phi / grad_phi (2D halves): a stride of 32 bytes mod 256 spreads the
+    // 8-byte fragment writes of 16 rows over all banks
+    static constexpr int LDP = 2 * D + 16;
+    static constexpr int LDG = (2 * D > DH ? 2 * D : DH) + 16;   // backward: grad_phi rows in, dx rows out
+    static constexpr size_t kFwdLds = (size_t)(D * LDW + 64 * LDP) * 2;
+    static constexpr size_t kBwdLds = (size_t)(D * LDW + 64 * LDW + 64 * LDU + 64 * LDG) * 2;
 };
+
+// Orders this wave's earlier LDS writes before its later LDS reads of other lanes' data
+// (one wave executes its LDS instructions in order; this only stops the compiler).
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Copy this wave's 16 staged rows (F halves each, row stride ld in LDS) to global rows
+// r0 .. r0+15 of a [R, H, F] tensor at head h: every store instruction writes whole rows,
+// 16 bytes per lane.
+template <int F>
+__device__ __forceinline__ void wave_rows_s2g(const half_t* Ss, int ld, half_t* __restrict__ dst, int r0, int R,
+                                              int H, int h, int lane) {
+    constexpr int PPR = F / 8;        // 16-byte pieces per row
+    constexpr int RPI = 64 / PPR;     // rows per instruction
+    static_assert(PPR <= 64 && 64 % PPR == 0, "row too long for one wave");
+#pragma unroll
+    for (int k = 0; k < 16 / RPI; ++k) {
+        const int lr = k * RPI + lane / PPR, pc = lane % PPR;
+        const uint4 val = *reinterpret_cast<const uint4*>(Ss + lr * ld + pc * 8);
+        if (r0 + lr < R) *reinterpret_cast<uint4*>(dst + ((int64_t)(r0 + lr) * H + h) * F + pc * 8) = val;
+    }
+}
+
+// The reverse, split so that the loads can be issued one row block ahead: global rows
+// -> registers (zero beyond R) -> this wave's staging rows.
+template <int F>
+struct WaveRows {
+    static constexpr int PPR = F / 8;
+    static constexpr int RPI = 64 / PPR;
+    static_assert(PPR <= 64 && 64 % PPR == 0, "row too long for one wave");
+    uint4 v[16 / RPI];
+};
+
+template <int F>
+__device__ __forceinline__ void wave_rows_g2r(WaveRows<F>& rr, const half_t* __restrict__ src, int r0, int R, int H,
+                                              int h, int lane) {
+    constexpr int PPR = WaveRows<F>::PPR, RPI = WaveRows<F>::RPI;
+#pragma unroll
+    for (int k = 0; k < 16 / RPI; ++k) {
+        const int lr = k * RPI + lane / PPR, pc = lane % PPR;
+        rr.v[k] = make_uint4(0, 0, 0, 0);
+        if (r0 + lr < R) rr.v[k] = *reinterpret_cast<const uint4*>(src + ((int64_t)(r0 + lr) * H + h) * F + pc * 8);
+    }
+}
+
+template <int F>
+__device__ __forceinline__ void wave_rows_r2s(const WaveRows<F>& rr, half_t* Ss, int ld, int lane) {
+    constexpr int PPR = WaveRows<F>::PPR, RPI = WaveRows<F>::RPI;
+#pragma unroll
+    for (int k = 0; k < 16 / RPI; ++k) {
+        const int lr = k * RPI + lane / PPR, pc = lane % PPR;
+        *reinterpret_cast<uint4*>(Ss + lr * ld + pc * 8) = rr.v[k];
+    }
+}
 
 template <int D, int DH>
 __device__ __forceinline__ void load_w_to_lds(half_t* Ws, const half_t* __restrict__ wh, int tid) {
@@ -39,11 +100,12 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_fwd(
     const half_t* __restrict__ x, const half_t* __restrict__ w, half_t* __restrict__ phi, int R, int H,
     float scale) {
     using Cfg = FeatureCfg<D, DH>;
-    constexpr int LDW = Cfg::LDW;
+    constexpr int LDW = Cfg::LDW, LDP = Cfg::LDP;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Ws = reinterpret_cast<half_t*>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    half_t* Ps = Ws + D * LDW + wv * 16 * LDP;     // this wave's 16 output rows
     const int i = lane & 15, G = lane >> 4;
     const int h = blockIdx.y;
     const int r = blockIdx.x * 64 + 16 * wv + i;
@@ -67,7 +129,6 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_fwd(
     const float inv = 1.0f / (sqrtf(ss) + 1e-3f);
     __syncthreads();
 
-    half_t* po = phi + ((int64_t)r * H + h) * (2 * D);
 #pragma unroll
     for (int jt = 0; jt < D / 16; ++jt) {
         f4 acc = f4_zero();   // u^T tile (m = feature j, n = row)
@@ -81,11 +142,13 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_fwd(
             sv[e] = (half_t)(scale * s_);
             cv[e] = (half_t)(scale * c_);
         }
-        if (r < R) {
-            *reinterpret_cast<h4*>(po + 16 * jt + 4 * G) = sv;
-            *reinterpret_cast<h4*>(po + D + 16 * jt + 4 * G) = cv;
-        }
+        *reinterpret_cast<h4*>(Ps + i * LDP + 16 * jt + 4 * G) = sv;
+        *reinterpret_cast<h4*>(Ps + i * LDP + D + 16 * jt + 4 * G) = cv;
     }
+    // the fragment layout holds 8 bytes per lane and row: stage through LDS so that the
+    // stores to HBM cover whole 4D-byte rows
+    wave_lds_fence();
+    wave_rows_s2g<2 * D>(Ps, LDP, phi, blockIdx.x * 64 + 16 * wv, R, H, h, lane);
 }
 
 // Backward.  grid = (nblk, H); workgroup (b, h) walks row blocks b, b+nblk, ...
@@ -99,7 +162,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
     const half_t* __restrict__ x, const half_t* __restrict__ w, const half_t* __restrict__ gphi,
     half_t* __restrict__ dx, float* __restrict__ dw_part, int R, int H, float scale) {
     using Cfg = FeatureCfg<D, DH>;
-    constexpr int LDW = Cfg::LDW, LDU = Cfg::LDU;
+    constexpr int LDW = Cfg::LDW, LDU = Cfg::LDU, LDG = Cfg::LDG;
     constexpr int NCTW = DH / 64;   // c-tiles of dW owned by one wave
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Ws = reinterpret_cast<half_t*>(smem_raw);
@@ -107,8 +170,10 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
     half_t* Us = Xs + 64 * LDW;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    half_t* Gs = Us + 64 * LDU + wv * 16 * LDG;   // this wave's 16 rows: grad_phi in, dx out
     const int i = lane & 15, G = lane >> 4;
     const int h = blockIdx.y;
+    const int lr = 16 * wv + i;          // this lane's row inside a block
 
     load_w_to_lds<D, DH>(Ws, w + (int64_t)h * D * DH, tid);
 
@@ -118,41 +183,49 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
 #pragma unroll
         for (int b = 0; b < D / 16; ++b) dwacc[a][b] = f4_zero();
 
-    const int nrb = (R + 63) / 64;
-    for (int rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
-        const int lr = 16 * wv + i;          // row inside the block
+    // x rows are loaded straight into MFMA operand form (16 bytes per lane, 64-byte runs);
+    // grad_phi rows are loaded whole and re-read from LDS in fragment form
+    h8 xn[DH / 32];
+    WaveRows<2 * D> gn;
+    auto issue_loads = [&](int rb) {
         const int r = rb * 64 + lr;
+#pragma unroll
+        for (int cs = 0; cs < DH / 32; ++cs) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xn[cs][e] = (half_t)0.f;
+            if (r < R) xn[cs] = *reinterpret_cast<const h8*>(x + ((int64_t)r * H + h) * DH + cs * 32 + 8 * G);
+        }
+        wave_rows_g2r<2 * D>(gn, gphi, rb * 64 + 16 * wv, R, H, h, lane);
+    };
+
+    const int nrb = (R + 63) / 64;
+    if ((int)blockIdx.x < nrb) issue_loads(blockIdx.x);
+    for (int rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+        const int r0 = rb * 64 + 16 * wv;    // first row of this wave
         h8 xb[DH / 32];
         float ss = 0.f;
 #pragma unroll
         for (int cs = 0; cs < DH / 32; ++cs) {
-            if (r < R) {
-                xb[cs] = *reinterpret_cast<const h8*>(x + ((int64_t)r * H + h) * DH + cs * 32 + 8 * G);
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) xb[cs][e] = (half_t)0.f;
-            }
+            xb[cs] = xn[cs];
             *reinterpret_cast<h8*>(Xs + lr * LDW + cs * 32 + 8 * G) = xb[cs];
 #pragma unroll
             for (int e = 0; e < 8; ++e) ss += (float)xb[cs][e] * (float)xb[cs][e];
         }
+        wave_rows_r2s<2 * D>(gn, Gs, LDG, lane);
         ss = sum_over_groups(ss);
         const float nrm = sqrtf(ss);
         const float inv = 1.0f / (nrm + 1e-3f);
         const float coef = nrm > 0.f ? inv / nrm : 0.f;
-        __syncthreads();   // Ws (first pass), Xs visible; previous block's dW reads done
+        __syncthreads();   // Ws (first pass), Xs, Gs visible; previous block's dW reads done
+        if (rb + (int)gridDim.x < nrb) issue_loads(rb + gridDim.x);
 
-        const half_t* gp = gphi + ((int64_t)r * H + h) * (2 * D);
 #pragma unroll
         for (int jt = 0; jt < D / 16; ++jt) {
             f4 acc = f4_zero();
 #pragma unroll
             for (int cs = 0; cs < DH / 32; ++cs) acc = mfma32(row8(Ws, LDW, 16 * jt + i, cs * 32, G), xb[cs], acc);
-            h4 gs = h4_zero(), gc = h4_zero();
-            if (r < R) {
-                gs = *reinterpret_cast<const h4*>(gp + 16 * jt + 4 * G);
-                gc = *reinterpret_cast<const h4*>(gp + D + 16 * jt + 4 * G);
-            }
+            const h4 gs = *reinterpret_cast<const h4*>(Gs + i * LDG + 16 * jt + 4 * G);
+            const h4 gc = *reinterpret_cast<const h4*>(Gs + i * LDG + D + 16 * jt + 4 * G);
             h4 du;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -179,17 +252,17 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
             for (int e = 0; e < 4; ++e) xdot += acc[e] * (float)xv[e];
         }
         xdot = sum_over_groups(xdot) * coef;
-        if (r < R) {
-            half_t* dxo = dx + ((int64_t)r * H + h) * DH;
+        // dx rows: fragment layout -> this wave's staging rows -> whole-row stores
 #pragma unroll
-            for (int ct = 0; ct < DH / 16; ++ct) {
-                h4 xv = *reinterpret_cast<const h4*>(Xs + lr * LDW + 16 * ct + 4 * G);
-                h4 o;
+        for (int ct = 0; ct < DH / 16; ++ct) {
+            h4 xv = *reinterpret_cast<const h4*>(Xs + lr * LDW + 16 * ct + 4 * G);
+            h4 o;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = (half_t)(y[ct][e] - (float)xv[e] * xdot);
-                *reinterpret_cast<h4*>(dxo + 16 * ct + 4 * G) = o;
-            }
+            for (int e = 0; e < 4; ++e) o[e] = (half_t)(y[ct][e] - (float)xv[e] * xdot);
+            *reinterpret_cast<h4*>(Gs + i * LDG + 16 * ct + 4 * G) = o;
         }
+        wave_lds_fence();
+        wave_rows_s2g<DH>(Gs, LDG, dx, r0, R, H, h, lane);
 
         // dW (m = c, n = j) += X^T Us over the 64 rows of the block
 #pragma unroll
@@ -204,7 +277,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
                 for (int a = 0; a < NCTW; ++a) dwacc[a][jt] = mfma32(xa[a], ub, dwacc[a][jt]);
             }
         }
-        __syncthreads();   // all reads of Xs / Us done before the next block overwrites them
+        __syncthreads();   // all reads of Xs / Us / Gs done before the next block overwrites them
     }
 
     float* po = dw_part + ((int64_t)blockIdx.x * H + h) * D * DH;
@@ -215,21 +288,33 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
             *reinterpret_cast<f4*>(po + (16 * jt + i) * DH + 16 * (wv * NCTW + a) + 4 * G) = dwacc[a][jt];
 }
 
-// dw[e] = sum_b dw_part[b][e]
-__global__ void k_feature_map_dw_reduce(const float* __restrict__ part, float* __restrict__ dw, int nblk,
-                                        int64_t elems) {
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= elems) return;
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;   // independent chains: the loads overlap
-    int b = 0;
-    for (; b + 4 <= nblk; b += 4) {
-        s0 += part[(int64_t)b * elems + e];
-        s1 += part[(int64_t)(b + 1) * elems + e];
-        s2 += part[(int64_t)(b + 2) * elems + e];
-        s3 += part[(int64_t)(b + 3) * elems + e];
+// dw[e] = sum_b dw_part[b][e].  One workgroup of 4 waves per 256 consecutive elements
+// (64 lanes x 16 bytes); wave p sums the shares b = p, p+4, ... with all its loads in
+// flight at once, then the 4 waves are added through LDS.  elems % 256 == 0.
+__global__ __launch_bounds__(kThreads) void k_feature_map_dw_reduce(const float* __restrict__ part,
+                                                                    float* __restrict__ dw, int nblk,
+                                                                    int64_t elems) {
+    __shared__ f4 red[3][64];
+    const int lane = threadIdx.x & 63, p = threadIdx.x >> 6;
+    const int64_t e = ((int64_t)blockIdx.x * 64 + lane) * 4;
+    f4 acc = f4_zero();
+    int b = p;
+    for (; b + 28 < nblk; b += 32) {
+        f4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const f4*>(part + (int64_t)(b + 4 * u) * elems + e);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u];
     }
-    for (; b < nblk; ++b) s0 += part[(int64_t)b * elems + e];
-    dw[e] = (s0 + s1) + (s2 + s3);
+    for (; b < nblk; b += 4) acc += *reinterpret_cast<const f4*>(part + (int64_t)b * elems + e);
+    if (p > 0) red[p - 1][lane] = acc;
+    __syncthreads();
+    if (p == 0) {
+        acc += red[0][lane];
+        acc += red[1][lane];
+        acc += red[2][lane];
+        *reinterpret_cast<f4*>(dw + e) = acc;
+    }
 }
 
 }  // namespace rfa
