@@ -28,11 +28,11 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the bench configuration, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
 # passes summarised in profiles/bench_cfg2_hbm_traffic.md (counters scaled on the 512 MiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "k_segment_state": 25359084,
-    "k_causal_fwd": 63281112,
-    "k_causal_bwd_dq": 87573852,
-    "k_causal_bwd_dkdv": 89580074,
-    "k_decode_step": 68890060,
+    "k_segment_state": 31659830,
+    "k_causal_fwd": 63250398,
+    "k_causal_bwd_dq": 87473517,
+    "k_causal_bwd_dkdv": 89545014,
+    "k_decode_step": 68884939,
 }
 
 
