@@ -152,7 +152,9 @@ template <int KD, int DH>
 int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, rfa::half_t* out,
                    int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, float* savedS, float* savedZ,
                    hipStream_t st) {
-    constexpr int NW = causal_waves(KD, DH);
+    // the two-stage pipelined forward needs both chunk buffers in LDS: K <= 128
+    constexpr bool PIPE = rfa::FwdPipeCfg<KD, DH>::kLds <= 160 * 1024;
+    constexpr int NW = PIPE ? 4 : causal_waves(KD, DH);
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
     // with a saved-state buffer the z totals are written there directly (z has one layout)
@@ -163,10 +165,17 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(64 * NW), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, savedS, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
-    auto kern = rfa::k_causal_fwd<KD, DH, NW, true>;
-    if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
-    RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q, k, v, out,
-                       wsS, wsZ, T, N, p.nseg, p.seg_len);
+    if constexpr (PIPE) {
+        auto kern = rfa::k_causal_fwd_pipe<KD, DH>;
+        if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
+        RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(512), rfa::FwdPipeCfg<KD, DH>::kLds, st, q, k, v, out,
+                           wsS, wsZ, T, N, p.nseg, p.seg_len);
+    } else {
+        auto kern = rfa::k_causal_fwd<KD, DH, NW, true>;
+        if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
+        RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q, k, v, out,
+                           wsS, wsZ, T, N, p.nseg, p.seg_len);
+    }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }

@@ -114,7 +114,7 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
     ChunkRegs<DH, NT> rv;
     chunk_g2r<KD, NT>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
     chunk_g2r<DH, NT>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
-    if (mrow) chunk_mask_rows<KD, NT>(rk, mrow + t_begin, t_end - t_begin, tid);
+    if (mrow) chunk_mask_rows<KD, NT>(rk, mrow + t_begin, tid);
     for (int t0 = t_begin; t0 < t_end; t0 += C) {
         chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
         chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
         if (t0 + C < t_end) {
             chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, t_end - t0 - C, tid);
             chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, t_end - t0 - C, tid);
-            if (mrow) chunk_mask_rows<KD, NT>(rk, mrow + t0 + C, t_end - t0 - C, tid);
+            if (mrow) chunk_mask_rows<KD, NT>(rk, mrow + t0 + C, tid);
         }
         h8 bv[NCT][2];
 #pragma unroll
@@ -408,6 +408,255 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
         RFA_TICK(9);
         __syncthreads();
         RFA_TICK(10);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// forward scan, two-stage pipeline (causal only).  8 waves: waves 0-3 ("tile group")
+// bring chunk u into LDS and form what depends on q, k alone -- the masked A^T tiles,
+// z and the denominators -- while waves 4-7 ("state group") finish chunk u-1: output
+// tiles, division, store and the update of S.  Each SIMD holds one wave of either
+// group, so the two stages overlap instead of adding up; the chunk arrays are double
+// buffered and the groups meet at two workgroup barriers per chunk.  State-group wave
+// w owns value columns [w*DS, (w+1)*DS) of S exactly like k_causal_fwd with 4 waves
+// (same fragment-order segment totals).
+// ---------------------------------------------------------------------------
+template <int KD, int DH>
+struct FwdPipeCfg {
+    using Base = CausalCfg<KD, DH, 4>;
+    static constexpr int C = Base::C, LDQ = Base::LDQ, LDV = Base::LDV, LDA = Base::LDA;
+    static constexpr int kBufHalves = 2 * C * LDQ + C * LDV + C * LDA;
+    static constexpr size_t kBufBytes = (size_t)kBufHalves * 2 + C * 4;     // + dens[C]
+    static constexpr size_t kLds = 2 * kBufBytes + KD * 4;                   // + zs[KD]
+    static_assert(kBufBytes % 16 == 0, "buffer alignment");
+};
+
+__device__ __forceinline__ void wg_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+template <int KD, int DH>
+__global__ __launch_bounds__(512) void k_causal_fwd_pipe(
+    const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ, int T,
+    int N, int nseg, int seg_len) {
+    using Cfg = FwdPipeCfg<KD, DH>;
+    constexpr int NT = 256;      // threads per group
+    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = DH / 4;
+    constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / 4;
+    static_assert(DH % 64 == 0 && NKT % 4 == 0, "shape does not split over the waves");
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    float* zs = reinterpret_cast<float*>(smem_raw + 2 * Cfg::kBufBytes);
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const bool tile_group = wave < 4;
+    const int w = wave & 3;                    // wave inside its group
+    const int tid = threadIdx.x & (NT - 1);    // thread inside its group
+    const int row = lane & 15, G = lane >> 4;
+    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    const int t_begin = seg * seg_len;
+    const int t_end = min(T, t_begin + seg_len);
+    const int n_chunks = t_end > t_begin ? (t_end - t_begin + C - 1) / C : 0;
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+
+    RFA_TICK_INIT();
+    // Both branches run n_chunks + 1 iterations with exactly two barriers each.
+    if (tile_group) {
+        const half_t* qb = q + (int64_t)n * KD;
+        const half_t* kb = k + (int64_t)n * KD;
+        const half_t* vb = v + (int64_t)n * DH;
+        ChunkRegs<KD, NT> rq, rk;
+        ChunkRegs<DH, NT> rv;
+        if (n_chunks > 0) {
+            chunk_g2r<KD, NT>(rq, qb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
+            chunk_g2r<KD, NT>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
+            chunk_g2r<DH, NT>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
+        }
+        f4 zacc[NKTW];      // z for feature tiles kt = w*NKTW + a, element k = 16kt + 4G + e
+#pragma unroll
+        for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
+        for (int s = 0; s < seg; ++s) {
+#pragma unroll
+            for (int a = 0; a < NKTW; ++a)
+                zacc[a] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * nseg + s) * KD + 16 * (w * NKTW + a) + 4 * G);
+        }
+        const h8 ones = h8_ones();
+        RFA_TICK_AT(0, 0);
+        for (int it = 0; it <= n_chunks; ++it) {
+            unsigned char* base = smem_raw + (it & 1) * Cfg::kBufBytes;
+            half_t* Qs = reinterpret_cast<half_t*>(base);
+            half_t* Ks = Qs + C * LDQ;
+            half_t* Vs = Ks + C * LDQ;
+            half_t* As = Vs + C * LDV;
+            float* dens = reinterpret_cast<float*>(As + C * LDA);
+            const bool live = it < n_chunks;
+            if (live) {
+                chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
+                chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
+                chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
+                if (row == 0) {
+#pragma unroll
+                    for (int a = 0; a < NKTW; ++a) *reinterpret_cast<f4*>(zs + 16 * (w * NKTW + a) + 4 * G) = zacc[a];
+                }
+            }
+            RFA_TICK_AT(1, 0);
+            wg_barrier();
+            RFA_TICK_AT(2, 0);
+            if (live) {
+                const int t0 = t_begin + it * C;
+                if (it + 1 < n_chunks) {
+                    const int rows = t_end - t0 - C;
+                    chunk_g2r<KD, NT>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+                    chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+                    chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+                }
+                RFA_TICK_AT(3, 0);
+                // rows i in [16w, 16w+16) of A as A^T tiles (m=j, n=i), all four j tiles
+                f4 at[4];
+#pragma unroll
+                for (int a = 0; a < 4; ++a) at[a] = f4_zero();
+#pragma unroll
+                for (int ks = 0; ks < KD / 32; ++ks) {
+                    h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) at[a] = mfma32(row8(Ks, LDQ, 16 * a + row, ks * 32, G), bq, at[a]);
+                }
+                float part = 0.f;
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {   // keep j <= i
+                        const bool keep = (a < w) || (a == w && 4 * G + e <= row);
+                        at[a][e] = keep ? at[a][e] : 0.f;
+                    }
+                    part += at[a][0] + at[a][1] + at[a][2] + at[a][3];
+                }
+                // + q_i . z : this lane covers features [G*KD/4, (G+1)*KD/4)
+                f4 qz4 = f4_zero();
+#pragma unroll
+                for (int kk = 0; kk < KD / 4; kk += 8) {
+                    const int k0 = G * (KD / 4) + kk;
+                    h8 qv = *reinterpret_cast<const h8*>(Qs + (16 * w + row) * LDQ + k0);
+                    f4 z0 = *reinterpret_cast<const f4*>(zs + k0);
+                    f4 z1 = *reinterpret_cast<const f4*>(zs + k0 + 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        qz4[e] += (float)qv[e] * z0[e];
+                        qz4[e] += (float)qv[4 + e] * z1[e];
+                    }
+                }
+                part += (qz4[0] + qz4[1]) + (qz4[2] + qz4[3]);
+                part = sum_over_groups(part);
+                if (G == 0) dens[16 * w + row] = part;
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+                    *reinterpret_cast<h4*>(As + (16 * w + row) * LDA + 16 * a + 4 * G) = to_h4(at[a]);
+                // z += K^T 1 for the next chunk
+#pragma unroll
+                for (int a = 0; a < NKTW; ++a)
+#pragma unroll
+                    for (int js = 0; js < 2; ++js)
+                        zacc[a] = mfma32(col8(Ks, LDQ, js * 32, 16 * (w * NKTW + a), lane), ones, zacc[a]);
+            }
+            RFA_TICK_AT(4, 0);
+            wg_barrier();
+            RFA_TICK_AT(5, 0);
+        }
+    } else {
+        half_t* ob = out + (int64_t)n * DH;
+        f4 S[NKT][NCT];
+#pragma unroll
+        for (int a = 0; a < NKT; ++a)
+#pragma unroll
+            for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
+        for (int s = 0; s < seg; ++s) {
+            const f4* sf = reinterpret_cast<const f4*>(wsS + ((int64_t)(n * nseg + s) * KD) * DH) + (int64_t)w * NKT * NCT * 64;
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct) S[kt][ct] += sf[(kt * NCT + ct) * 64 + lane];
+        }
+        RFA_TICK_AT(8, 256);
+        for (int it = 0; it <= n_chunks; ++it) {
+            unsigned char* base = smem_raw + ((it + 1) & 1) * Cfg::kBufBytes;   // chunk it - 1
+            const half_t* Qs = reinterpret_cast<const half_t*>(base);
+            const half_t* Ks = Qs + C * LDQ;
+            const half_t* Vs = Ks + C * LDQ;
+            const half_t* As = Vs + C * LDV;
+            const float* dens = reinterpret_cast<const float*>(As + C * LDA);
+            const bool live = it >= 1;
+            const int t0 = t_begin + (it - 1) * C;
+            h8 av[NCT][2];   // V column fragments: element V[j = 32js+8G+e][c = w*DS+16ct+i]
+            f4 acc[4][NCT];  // out^T tiles (m=c, n=i)
+            if (live) {
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                    for (int js = 0; js < 2; ++js) av[ct][js] = col8(Vs, LDV, js * 32, w * DS + 16 * ct, lane);
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = f4_zero();
+#pragma unroll
+                    for (int js = 0; js < 2; ++js) {
+                        if (js == 0 || i4 >= 2) {
+                            h8 ba = row8(As, LDA, 16 * i4 + row, js * 32, G);
+#pragma unroll
+                            for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(av[ct][js], ba, acc[i4][ct]);
+                        }
+                    }
+                }
+            }
+            RFA_TICK_AT(9, 256);
+            wg_barrier();
+            RFA_TICK_AT(10, 256);
+            if (live) {
+#pragma unroll
+                for (int ks = 0; ks < KD / 32; ++ks) {
+                    h8 hi[NCT], lo[NCT];
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct) acc_to_operand(S[2 * ks][ct], S[2 * ks + 1][ct], hi[ct], lo[ct]);
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) {
+                        h8 bq = row_split8(Qs, LDQ, 16 * i4 + row, ks * 32, G);
+#pragma unroll
+                        for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(hi[ct], bq, acc[i4][ct]);
+#pragma unroll
+                        for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(lo[ct], bq, acc[i4][ct]);
+                    }
+                }
+                RFA_TICK_AT(11, 256);
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    const int i = 16 * i4 + row;
+                    const float inv = 1.0f / fmaxf(dens[i], 1.0f);
+                    if (t0 + i < t_end) {
+#pragma unroll
+                        for (int ct = 0; ct < NCT; ++ct) {
+                            f4 o = acc[i4][ct];
+                            o[0] *= inv; o[1] *= inv; o[2] *= inv; o[3] *= inv;
+                            *reinterpret_cast<h4*>(ob + (int64_t)(t0 + i) * v_stride + w * DS + 16 * ct + 4 * G) = to_h4(o);
+                        }
+                    }
+                }
+                RFA_TICK_AT(12, 256);
+                // S (m=k, n=c) += K^T V
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                    for (int js = 0; js < 2; ++js) {
+                        h8 ak = col8(Ks, LDQ, js * 32, 16 * kt, lane);
+#pragma unroll
+                        for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, av[ct][js], S[kt][ct]);
+                    }
+            }
+            RFA_TICK_AT(13, 256);
+            wg_barrier();
+            RFA_TICK_AT(14, 256);
+        }
     }
 }
 
@@ -845,12 +1094,13 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
 #pragma unroll
             for (int it = 0; it < ChunkRegs<DH, NT>::kPieces; ++it) {
                 // raw den only: dividing here would wait for the loads issued just above
-                const int r_ = (tid + NT * it) / PPRV;
-                inv_den[it] = (r_ < rows) ? den_ws[(int64_t)(t0 + r_) * N + n] : 0.f;
+                // (rows past the end read the last valid one; chunk_r2s_scaled zeroes them)
+                const int r_ = min((tid + NT * it) / PPRV, rg.rows - 1);
+                inv_den[it] = den_ws[(int64_t)(t0 + r_) * N + n];
             }
-            gz_next = (tid < C && tid < rows) ? gz_ws[(int64_t)(t0 + tid) * N + n] : 0.f;
+            gz_next = gz_ws[(int64_t)(t0 + min(tid, rg.rows - 1)) * N + n];
         } else if (mrow) {
-            chunk_mask_rows<KD, NT>(rk, mrow + t0, rows, tid);
+            chunk_mask_rows<KD, NT>(rk, mrow + t0, tid);
         }
     };
 
@@ -866,7 +1116,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
             for (int it = 0; it < ChunkRegs<DH, NT>::kPieces; ++it)
                 inv_den[it] = inv_den[it] > 0.f ? 1.0f / inv_den[it] : 0.f;   // den >= 1 on valid rows
             chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
-            if (tid < C) gzs[tid] = gz_next;
+            if (tid < C) gzs[tid] = tid < rg.rows ? gz_next : 0.f;
         }
         if (row == 0) {
 #pragma unroll

@@ -31,9 +31,10 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 #ifdef RFA_PHASE_TIMING
 __device__ unsigned long long g_phase_ticks[32];
 #define RFA_TICK_INIT() long long tick_last_ = clock64()
-#define RFA_TICK(i)                                                                        \
+#define RFA_TICK(i) RFA_TICK_AT(i, 0)
+#define RFA_TICK_AT(i, thr)                                                                \
     do {                                                                                   \
-        if (blockIdx.x == RFA_PHASE_TIMING && threadIdx.x == 0) {                          \
+        if (blockIdx.x == RFA_PHASE_TIMING && threadIdx.x == (thr)) {                      \
             const long long now_ = clock64();                                              \
             atomicAdd(&g_phase_ticks[i], (unsigned long long)(now_ - tick_last_));         \
             tick_last_ = now_;                                                             \
@@ -42,6 +43,7 @@ __device__ unsigned long long g_phase_ticks[32];
 #else
 #define RFA_TICK_INIT() do { } while (0)
 #define RFA_TICK(i) do { } while (0)
+#define RFA_TICK_AT(i, thr) do { } while (0)
 #endif
 
 // Row padding (in halves) of an LDS array with F halves per row.  With 64 banks of 4
@@ -164,35 +166,44 @@ __device__ __forceinline__ float sum_over_groups(float x) {
 // sequence, F halves per step; in HBM consecutive steps are `row_stride` halves
 // apart ([T, N, F] time-major layout).
 // ---------------------------------------------------------------------------
+// Loads never depend on control flow: a row past the end of the chunk is read from the
+// last valid row (clamped address) and replaced by zeros when the registers are written
+// to LDS, i.e. after the data has arrived.  A load under a lane- or row-dependent branch
+// makes the compiler wait for all outstanding loads at the join, which serialises the
+// prefetch of a chunk into several memory round trips.
 template <int F, int NT = kThreads>
 struct ChunkRegs {
     static constexpr int kPieces = kChunk * F / 8 / NT;   // 16-byte pieces per thread
     static_assert(kPieces >= 1, "feature width too small for this many threads");
     uint4 v[kPieces];
+    unsigned char drop[kPieces];   // non-zero: the piece's row is masked out (chunk_mask_rows)
+    int rows;                      // rows of the chunk that exist
 };
 
+// rows_valid >= 1
 template <int F, int NT = kThreads>
 __device__ __forceinline__ void chunk_g2r(ChunkRegs<F, NT>& r, const half_t* __restrict__ base,
                                           int64_t row_stride, int rows_valid, int tid) {
     constexpr int PPR = F / 8;
-    if (rows_valid >= kChunk) {   // full chunk (uniform): no per-lane predication
-#pragma unroll
-        for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
-            const int p = tid + NT * it;
-            const int row = p / PPR, c8 = p % PPR;
-            r.v[it] = *reinterpret_cast<const uint4*>(base + (int64_t)row * row_stride + c8 * 8);
-        }
-        return;
-    }
+    r.rows = min(rows_valid, kChunk);
 #pragma unroll
     for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
         const int p = tid + NT * it;
-        const int row = p / PPR, c8 = p % PPR;
-        if (row < rows_valid) {
-            r.v[it] = *reinterpret_cast<const uint4*>(base + (int64_t)row * row_stride + c8 * 8);
-        } else {
-            r.v[it] = make_uint4(0u, 0u, 0u, 0u);
-        }
+        const int row = min(p / PPR, r.rows - 1), c8 = p % PPR;
+        r.v[it] = *reinterpret_cast<const uint4*>(base + (int64_t)row * row_stride + c8 * 8);
+        r.drop[it] = 0;
+    }
+}
+
+// mark the rows whose mask byte is non-zero (mask already offset to the chunk's first
+// step); they are written to LDS as zeros.  Call after chunk_g2r.
+template <int F, int NT = kThreads>
+__device__ __forceinline__ void chunk_mask_rows(ChunkRegs<F, NT>& r, const uint8_t* __restrict__ mask, int tid) {
+    constexpr int PPR = F / 8;
+#pragma unroll
+    for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
+        const int row = min((tid + NT * it) / PPR, r.rows - 1);
+        r.drop[it] = mask[row];
     }
 }
 
@@ -203,19 +214,10 @@ __device__ __forceinline__ void chunk_r2s(const ChunkRegs<F, NT>& r, half_t* Xs,
     for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
         const int p = tid + NT * it;
         const int row = p / PPR, c8 = p % PPR;
-        *reinterpret_cast<uint4*>(Xs + row * ld + c8 * 8) = r.v[it];
-    }
-}
-
-// zero the rows whose mask byte is non-zero (mask already offset to the chunk's first step)
-template <int F, int NT = kThreads>
-__device__ __forceinline__ void chunk_mask_rows(ChunkRegs<F, NT>& r, const uint8_t* __restrict__ mask,
-                                                int rows_valid, int tid) {
-    constexpr int PPR = F / 8;
-#pragma unroll
-    for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
-        const int row = (tid + NT * it) / PPR;
-        if (row < rows_valid && mask[row]) r.v[it] = make_uint4(0u, 0u, 0u, 0u);
+        const bool keep = row < r.rows && !r.drop[it];
+        uint4 x = r.v[it];
+        x.x = keep ? x.x : 0u; x.y = keep ? x.y : 0u; x.z = keep ? x.z : 0u; x.w = keep ? x.w : 0u;
+        *reinterpret_cast<uint4*>(Xs + row * ld + c8 * 8) = x;
     }
 }
 
@@ -228,11 +230,12 @@ __device__ __forceinline__ void chunk_r2s_scaled(const ChunkRegs<F, NT>& r, cons
     for (int it = 0; it < ChunkRegs<F, NT>::kPieces; ++it) {
         const int p = tid + NT * it;
         const int row = p / PPR, c8 = p % PPR;
+        const float sc = row < r.rows ? scale[it] : 0.f;
         union { uint4 u; h8 h; } x;
         x.u = r.v[it];
         h8 y;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)x.h[e] * scale[it]);
+        for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)x.h[e] * sc);
         *reinterpret_cast<h8*>(Xs + row * ld + c8 * 8) = y;
     }
 }
