@@ -212,7 +212,15 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqLds, st, q, k, v, g,
                            dq, inS, inZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
     }
-    {
+    if constexpr (NW == 4 && KD <= 128) {
+        // 8 waves with the state phase split by role (dK waves / dV waves): two waves per SIMD
+        // (K = 256 would spill at 256 registers per wave)
+        using CfgK = rfa::CausalCfg<KD, DH, 8>;
+        auto kern = rfa::k_causal_bwd_dkdv<KD, DH, 8, true, true>;
+        if (int rc = set_lds(kern, CfgK::kBwdDkLds)) return rc;
+        RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(512), CfgK::kBwdDkLds, st, q, k, v, g,
+                           dk, dv, wsR, wsr, den, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
+    } else {
         auto kern = rfa::k_causal_bwd_dkdv<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDkLds, st, q, k, v, g,

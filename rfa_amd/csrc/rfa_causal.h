@@ -1006,7 +1006,12 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
 // dV = K dS; q, g, den_ws, gz_ws are not read.  pad_mask ([B, T] bytes, may be
 // NULL; H heads per batch entry) marks padded keys: their phi_k rows are read as
 // zero and their dK rows are written as zero (the gradient of masked_fill).
-template <int KD, int DH, int NW, bool CAUSAL>
+//
+// SPLIT (8 waves only): the state phase is divided by role instead of by slice.  Waves
+// 0-3 carry RT and r and produce dK, waves 4-7 carry RR and produce dV, each for a
+// quarter of the feature rows / value columns; the tile phase is shared by all 8 waves
+// as usual.  Two waves per SIMD then work on independent halves of the state phase.
+template <int KD, int DH, int NW, bool CAUSAL, bool SPLIT = false>
 __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, half_t* __restrict__ dk, half_t* __restrict__ dv,
@@ -1015,10 +1020,12 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     int nseg, int seg_len) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
-    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS, DS = Cfg::DS;
+    static_assert(!SPLIT || NW == 8, "the role split needs 8 waves");
+    constexpr int NOWN = SPLIT ? 4 : NW;             // waves sharing one role
+    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = KD / NOWN, DS = DH / NOWN;
     constexpr int NKT = KS / 16, NCT = DH / 16;      // RT tiles
     constexpr int NKT2 = KD / 16, NCT2 = DS / 16;    // RR tiles
-    static_assert(KD % (16 * NW) == 0 && DH % (16 * NW) == 0, "shape does not split over the waves");
+    static_assert(KD % (16 * NOWN) == 0 && DH % (16 * NOWN) == 0, "shape does not split over the waves");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
     half_t* Ks = Qs + C * LDQ;
@@ -1033,6 +1040,8 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
     const int rb = w & 3, half = w >> 2;   // tile-phase role: 16-row block and which of its tiles
+    const int ws = SPLIT ? (w & 3) : w;    // state-phase slice
+    const bool do_dk = !SPLIT || w < 4, do_dv = !SPLIT || w >= 4;
     constexpr int JPW = Cfg::JPW, NH = Cfg::NH;
     const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
     const int t_begin = seg * seg_len;
@@ -1062,21 +1071,25 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     const int state_stride = CAUSAL ? nseg : 1;
     for (int s = s_first; s < s_last; ++s) {
         const float* ri = wsR + ((int64_t)(n * state_stride + s) * KD) * DH;
+        if (do_dk) {
 #pragma unroll
-        for (int ct = 0; ct < NCT; ++ct)
+            for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt)
+                    RT[ct][kt] += *reinterpret_cast<const f4*>(ri + (ws * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
 #pragma unroll
             for (int kt = 0; kt < NKT; ++kt)
-                RT[ct][kt] += *reinterpret_cast<const f4*>(ri + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
+                racc[kt] += *reinterpret_cast<const f4*>(wsr + (int64_t)(n * state_stride + s) * KD + ws * KS + 16 * kt + 4 * G);
+        }
+        if (do_dv) {
 #pragma unroll
-        for (int kt = 0; kt < NKT2; ++kt)
+            for (int kt = 0; kt < NKT2; ++kt)
 #pragma unroll
-            for (int ct = 0; ct < NCT2; ++ct)
+                for (int ct = 0; ct < NCT2; ++ct)
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    RR[kt][ct][e] += ri[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row];
-#pragma unroll
-        for (int kt = 0; kt < NKT; ++kt)
-            racc[kt] += *reinterpret_cast<const f4*>(wsr + (int64_t)(n * state_stride + s) * KD + w * KS + 16 * kt + 4 * G);
+                    for (int e = 0; e < 4; ++e)
+                        RR[kt][ct][e] += ri[(16 * kt + 4 * G + e) * DH + ws * DS + 16 * ct + row];
+        }
     }
 
     ChunkRegs<KD, NT> rq, rk;
@@ -1118,9 +1131,9 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
             chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
             if (tid < C) gzs[tid] = tid < rg.rows ? gz_next : 0.f;
         }
-        if (row == 0) {
+        if (row == 0 && do_dk) {
 #pragma unroll
-            for (int kt = 0; kt < NKT; ++kt) *reinterpret_cast<f4*>(rs + w * KS + 16 * kt + 4 * G) = racc[kt];
+            for (int kt = 0; kt < NKT; ++kt) *reinterpret_cast<f4*>(rs + ws * KS + 16 * kt + 4 * G) = racc[kt];
         }
         __syncthreads();
         if (ci > 0) prefetch(t0 - C);
@@ -1167,21 +1180,26 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
             h8 qf[NKT][2];    // Q column fragments for this wave's feature slice
             h8 gf2[NCT2][2];  // (G/den) column fragments for this wave's value slice
             if (CAUSAL) {
+                if (do_dk) {
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt)
+                    for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-                    for (int is = 0; is < 2; ++is) qf[kt][is] = col8(Qs, LDQ, is * 32, w * KS + 16 * kt, lane);
+                        for (int is = 0; is < 2; ++is) qf[kt][is] = col8(Qs, LDQ, is * 32, ws * KS + 16 * kt, lane);
+                }
+                if (do_dv) {
 #pragma unroll
-                for (int ct = 0; ct < NCT2; ++ct)
+                    for (int ct = 0; ct < NCT2; ++ct)
 #pragma unroll
-                    for (int is = 0; is < 2; ++is) gf2[ct][is] = col8(Gs, LDV, is * 32, w * DS + 16 * ct, lane);
+                        for (int is = 0; is < 2; ++is) gf2[ct][is] = col8(Gs, LDV, is * 32, ws * DS + 16 * ct, lane);
+                }
             }
 
+            if (do_dk) {
             // dK^T tiles (m=k, n=j)
             f4 dkacc[NKT][4];
 #pragma unroll
             for (int kt = 0; kt < NKT; ++kt) {
-                f4 rv4 = *reinterpret_cast<const f4*>(rs + w * KS + 16 * kt + 4 * G);
+                f4 rv4 = *reinterpret_cast<const f4*>(rs + ws * KS + 16 * kt + 4 * G);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
                     f4 acc = rv4;
@@ -1213,11 +1231,13 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
                     const bool padded = mrow && mrow[t0 + jj];
 #pragma unroll
                     for (int kt = 0; kt < NKT; ++kt)
-                        *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + w * KS + 16 * kt + 4 * G) =
+                        *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + ws * KS + 16 * kt + 4 * G) =
                             padded ? h4_zero() : to_h4(dkacc[kt][jt]);
                 }
             }
+            }
 
+            if (do_dv) {
             // dV^T tiles (m=c, n=j)
             f4 dvacc[NCT2][4];
 #pragma unroll
@@ -1251,31 +1271,36 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
                 if (t0 + jj < t_end) {
 #pragma unroll
                     for (int ct = 0; ct < NCT2; ++ct)
-                        *reinterpret_cast<h4*>(dvb + (int64_t)(t0 + jj) * v_stride + w * DS + 16 * ct + 4 * G) = to_h4(dvacc[ct][jt]);
+                        *reinterpret_cast<h4*>(dvb + (int64_t)(t0 + jj) * v_stride + ws * DS + 16 * ct + 4 * G) = to_h4(dvacc[ct][jt]);
                 }
+            }
             }
 
             // carried sums
 #pragma unroll
             for (int is = 0; is < (CAUSAL ? 2 : 0); ++is) {
-                h8 ghi, glo;   // r (m=k) += Q^T gz
-                f8_to_operand(*reinterpret_cast<const f4*>(gzs + is * 32 + 8 * G),
-                              *reinterpret_cast<const f4*>(gzs + is * 32 + 8 * G + 4), ghi, glo);
+                if (do_dk) {
+                    h8 ghi, glo;   // r (m=k) += Q^T gz
+                    f8_to_operand(*reinterpret_cast<const f4*>(gzs + is * 32 + 8 * G),
+                                  *reinterpret_cast<const f4*>(gzs + is * 32 + 8 * G + 4), ghi, glo);
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt][is], ghi, racc[kt]);
+                    for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt][is], ghi, racc[kt]);
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt][is], glo, racc[kt]);
+                    for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt][is], glo, racc[kt]);
 #pragma unroll
-                for (int ct = 0; ct < NCT; ++ct) {
-                    h8 gf = col8(Gs, LDV, is * 32, 16 * ct, lane);
+                    for (int ct = 0; ct < NCT; ++ct) {
+                        h8 gf = col8(Gs, LDV, is * 32, 16 * ct, lane);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) RT[ct][kt] = mfma32(gf, qf[kt][is], RT[ct][kt]);
+                        for (int kt = 0; kt < NKT; ++kt) RT[ct][kt] = mfma32(gf, qf[kt][is], RT[ct][kt]);
+                    }
                 }
+                if (do_dv) {
 #pragma unroll
-                for (int kt = 0; kt < NKT2; ++kt) {
-                    h8 qa = col8(Qs, LDQ, is * 32, 16 * kt, lane);
+                    for (int kt = 0; kt < NKT2; ++kt) {
+                        h8 qa = col8(Qs, LDQ, is * 32, 16 * kt, lane);
 #pragma unroll
-                    for (int ct = 0; ct < NCT2; ++ct) RR[kt][ct] = mfma32(qa, gf2[ct][is], RR[kt][ct]);
+                        for (int ct = 0; ct < NCT2; ++ct) RR[kt][ct] = mfma32(qa, gf2[ct][is], RR[kt][ct]);
+                    }
                 }
             }
         }
