@@ -92,7 +92,7 @@ def main():
         # what RFA.apply(...).backward(grad) runs: the forward hands its segment totals to the backward
         _lib.check(lib.rfa_causal_forward_save(p(pq), p(pk), p(vv), p(out), p(saved), sbytes, T, N, K, d,
                                                p(ws), fbytes, stream))
-        _lib.check(lib.rfa_causal_backward_saved(p(pq), p(pk), p(vv), p(gg), p(saved), sbytes, p(dq), p(dk), p(dv),
+        _lib.check(lib.rfa_causal_backward_saved(p(pq), p(pk), p(vv), p(gg), p(out), p(saved), sbytes, p(dq), p(dk), p(dv),
                                                  T, N, K, d, p(ws), bbytes, stream))
 
     for _ in range(args.warmup):
@@ -124,7 +124,7 @@ def main():
     per_tok = {
         "k_segment_state": (K + d) * 2,
         "k_causal_fwd": (2 * K + d) * 2 + d * 2,
-        "k_causal_bwd_dq": (2 * K + 2 * d) * 2 + K * 2 + 8,
+        "k_causal_bwd_dq": (2 * K + 3 * d) * 2 + K * 2 + 8,       # q, k, v, g, out in; dq out; den in, gz out
         "k_causal_bwd_dkdv": (2 * K + 2 * d) * 2 + 8 + (K + d) * 2,
     }
     nseg = lib.rfa_causal_num_segments(T, N)

@@ -76,19 +76,21 @@ int rfa_causal_backward(const void* q, const void* k, const void* v, const void*
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* Training-step variants (no counterpart in the reference, whose autograd Function
- * saves only q, k, v: rfa.py:124).  rfa_causal_forward_save additionally writes the
- * per-segment state totals it computed into `saved` (rfa_causal_saved_state_bytes
- * bytes, fp32); rfa_causal_backward_saved reads them back instead of recomputing
- * them from k and v.  Results are identical to the plain pair; `saved` must come from
- * a forward call with the same q/k/v shapes. */
+ * saves only q, k, v: rfa.py:124).  rfa_causal_forward_save additionally writes what
+ * the backward pass can reuse into `saved` (rfa_causal_saved_state_bytes bytes: the
+ * per-segment state totals and the raw denominators, fp32); rfa_causal_backward_saved
+ * reads them, and the forward output `out` (fp16 [T, N, d], as written by that forward
+ * call), instead of recomputing the forward pass: with num = out * den the term
+ * g . num of rfa.py:91 is (g . out) * den.  `saved` and `out` must come from a forward
+ * call on the same q, k, v. */
 size_t rfa_causal_saved_state_bytes(int64_t T, int64_t N, int K, int d);
 int rfa_causal_forward_save(const void* q, const void* k, const void* v, void* out, void* saved,
                             size_t saved_bytes, int64_t T, int64_t N, int K, int d, void* workspace,
                             size_t workspace_bytes, void* stream);
 int rfa_causal_backward_saved(const void* q, const void* k, const void* v, const void* grad_attn,
-                              const void* saved, size_t saved_bytes, void* dq, void* dk, void* dv,
-                              int64_t T, int64_t N, int K, int d, void* workspace, size_t workspace_bytes,
-                              void* stream);
+                              const void* out, const void* saved, size_t saved_bytes, void* dq, void* dk,
+                              void* dv, int64_t T, int64_t N, int K, int d, void* workspace,
+                              size_t workspace_bytes, void* stream);
 
 /* Number of time segments the causal kernels cut a sequence into for the given
  * shape (>= 1).  Environment variable RFA_HIP_NSEG overrides the heuristic. */

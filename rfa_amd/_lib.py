@@ -41,7 +41,7 @@ SIGNATURES = {
     "rfa_causal_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "rfa_causal_saved_state_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
     "rfa_causal_forward_save": (c_int, [c_void_p] * 5 + [c_size_t, c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
-    "rfa_causal_backward_saved": (c_int, [c_void_p] * 5 + [c_size_t] + [c_void_p] * 3 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "rfa_causal_backward_saved": (c_int, [c_void_p] * 6 + [c_size_t] + [c_void_p] * 3 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "rfa_feature_map_supported": (c_int, [c_int, c_int]),
     "rfa_feature_map_forward": (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int, c_int, c_float, c_void_p]),
     "rfa_feature_map_backward_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int]),

@@ -151,7 +151,7 @@ int set_lds(Kern kern, size_t bytes) {
 template <int KD, int DH>
 int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, rfa::half_t* out,
                    int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, float* savedS, float* savedZ,
-                   hipStream_t st) {
+                   float* savedDen, hipStream_t st) {
     // the two-stage pipelined forward needs both chunk buffers in LDS: K <= 128
     constexpr bool PIPE = rfa::FwdPipeCfg<KD, DH>::kLds <= 160 * 1024;
     constexpr int NW = PIPE ? 4 : causal_waves(KD, DH);
@@ -169,12 +169,12 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
         auto kern = rfa::k_causal_fwd_pipe<KD, DH>;
         if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(512), rfa::FwdPipeCfg<KD, DH>::kLds, st, q, k, v, out,
-                           wsS, wsZ, T, N, p.nseg, p.seg_len);
+                           wsS, wsZ, savedDen, T, N, p.nseg, p.seg_len);
     } else {
         auto kern = rfa::k_causal_fwd<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q, k, v, out,
-                           wsS, wsZ, T, N, p.nseg, p.seg_len);
+                           wsS, wsZ, savedDen, T, N, p.nseg, p.seg_len);
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -182,9 +182,9 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
 
 template <int KD, int DH>
 int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v,
-                    const rfa::half_t* g, rfa::half_t* dq, rfa::half_t* dk, rfa::half_t* dv, int T, int N,
-                    const ScanPlan& p, char* ws, const Workspace& wl, const float* savedS, const float* savedZ,
-                    hipStream_t st) {
+                    const rfa::half_t* g, const rfa::half_t* out, rfa::half_t* dq, rfa::half_t* dk,
+                    rfa::half_t* dv, int T, int N, const ScanPlan& p, char* ws, const Workspace& wl,
+                    const float* savedS, const float* savedZ, const float* savedDen, hipStream_t st) {
     constexpr int NW = causal_waves(KD, DH);
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
@@ -204,7 +204,17 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(64 * NW), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
-    {
+    const float* den_in = den;
+    if (savedDen) {
+        // the forward's output and raw denominators are at hand: the sweep that needs no A = Q K^T
+        constexpr int NWQ = dq_waves(KD, DH);
+        using CfgQ = rfa::CausalCfg<KD, DH, NWQ>;
+        auto kern = rfa::k_causal_bwd_dq_saved<KD, DH, NWQ>;
+        if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
+        RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g, out,
+                   savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len);
+        den_in = savedDen;
+    } else {
         constexpr int NWQ = dq_waves(KD, DH);
         using CfgQ = rfa::CausalCfg<KD, DH, NWQ>;
         auto kern = rfa::k_causal_bwd_dq<KD, DH, NWQ, true>;
@@ -219,12 +229,12 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         auto kern = rfa::k_causal_bwd_dkdv<KD, DH, 8, true, true>;
         if (int rc = set_lds(kern, CfgK::kBwdDkLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(512), CfgK::kBwdDkLds, st, q, k, v, g,
-                           dk, dv, wsR, wsr, den, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
+                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
     } else {
         auto kern = rfa::k_causal_bwd_dkdv<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDkLds, st, q, k, v, g,
-                           dk, dv, wsR, wsr, den, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
+                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -268,8 +278,8 @@ int launch_cross_readout(const rfa::half_t* q, const float* s, const float* z, r
     auto kern = rfa::k_causal_fwd<KD, DH, NW, false>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
     RFA_LAUNCH(CROSS_READOUT, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q,
-                       (const rfa::half_t*)nullptr, (const rfa::half_t*)nullptr, out, s, z, T, N, p.nseg,
-                       p.seg_len);
+                       (const rfa::half_t*)nullptr, (const rfa::half_t*)nullptr, out, s, z, (float*)nullptr, T, N,
+                       p.nseg, p.seg_len);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -470,17 +480,19 @@ size_t rfa_causal_backward_workspace_bytes(int64_t T, int64_t N, int K, int d) {
     if (K == 128 && d == 128) { return CALL(128, 128); }              \
     if (K == 256 && d == 128) { return CALL(256, 128); }
 
-// bytes of the segment totals (row-major S then z) for the saved-state buffer
-static size_t saved_state_bytes(int64_t T, int64_t N, int K, int d, size_t* z_offset) {
+// bytes of the saved buffer: segment totals (row-major S, then z), then the raw denominators
+static size_t saved_state_bytes(int64_t T, int64_t N, int K, int d, size_t* z_offset, size_t* den_offset) {
     const ScanPlan p = make_plan(T, N);
     const size_t s_bytes = align_up((size_t)N * p.nseg * K * d * 4);
+    const size_t z_bytes = align_up((size_t)N * p.nseg * K * 4);
     if (z_offset) *z_offset = s_bytes;
-    return s_bytes + align_up((size_t)N * p.nseg * K * 4);
+    if (den_offset) *den_offset = s_bytes + z_bytes;
+    return s_bytes + z_bytes + align_up((size_t)T * N * 4);
 }
 
 size_t rfa_causal_saved_state_bytes(int64_t T, int64_t N, int K, int d) {
     if (T <= 0 || N <= 0 || !rfa_shape_supported(K, d)) return 0;
-    return saved_state_bytes(T, N, K, d, nullptr);
+    return saved_state_bytes(T, N, K, d, nullptr, nullptr);
 }
 
 static int causal_forward_impl(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
@@ -505,14 +517,16 @@ static int causal_forward_impl(const void* q, const void* k, const void* v, void
     if (T == 0 || N == 0) return RFA_OK;
     float* savedS = nullptr;
     float* savedZ = nullptr;
+    float* savedDen = nullptr;
     if (want_saved) {
-        size_t zoff = 0;
-        const size_t need = saved_state_bytes(T, N, K, d, &zoff);
+        size_t zoff = 0, doff = 0;
+        const size_t need = saved_state_bytes(T, N, K, d, &zoff, &doff);
         if (!saved || saved_bytes < need || !aligned16(saved))
             return fail(RFA_ERR_WORKSPACE, "rfa_causal_forward_save: saved-state buffer of %zu bytes required, got %zu",
                         need, saved ? saved_bytes : (size_t)0);
         savedS = static_cast<float*>(saved);
         savedZ = reinterpret_cast<float*>(static_cast<char*>(saved) + zoff);
+        savedDen = reinterpret_cast<float*>(static_cast<char*>(saved) + doff);
     }
     if (!q || !k || !v || !out) return fail(RFA_ERR_NULL_POINTER, "rfa_causal_forward: NULL tensor pointer");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
@@ -528,47 +542,54 @@ static int causal_forward_impl(const void* q, const void* k, const void* v, void
     auto* vh = static_cast<const rfa::half_t*>(v);
     auto* oh = static_cast<rfa::half_t*>(out);
     char* ws = static_cast<char*>(workspace);
-#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedS, savedZ, st)
+#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedS, savedZ, savedDen, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_FWD)
 #undef RFA_CALL_FWD
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
 }
 
-static int causal_backward_impl(const void* q, const void* k, const void* v, const void* grad_attn, void* dq,
-                                void* dk, void* dv, int64_t T, int64_t N, int K, int d, const void* saved,
-                                size_t saved_bytes, bool have_saved, void* workspace, size_t workspace_bytes,
-                                void* stream);
+static int causal_backward_impl(const void* q, const void* k, const void* v, const void* grad_attn,
+                                const void* out, void* dq, void* dk, void* dv, int64_t T, int64_t N, int K, int d,
+                                const void* saved, size_t saved_bytes, bool have_saved, void* workspace,
+                                size_t workspace_bytes, void* stream);
 
 int rfa_causal_backward(const void* q, const void* k, const void* v, const void* grad_attn, void* dq,
                         void* dk, void* dv, int64_t T, int64_t N, int K, int d, void* workspace,
                         size_t workspace_bytes, void* stream) {
-    return causal_backward_impl(q, k, v, grad_attn, dq, dk, dv, T, N, K, d, nullptr, 0, false, workspace,
+    return causal_backward_impl(q, k, v, grad_attn, nullptr, dq, dk, dv, T, N, K, d, nullptr, 0, false, workspace,
                                 workspace_bytes, stream);
 }
 
 int rfa_causal_backward_saved(const void* q, const void* k, const void* v, const void* grad_attn,
-                              const void* saved, size_t saved_bytes, void* dq, void* dk, void* dv, int64_t T,
-                              int64_t N, int K, int d, void* workspace, size_t workspace_bytes, void* stream) {
-    return causal_backward_impl(q, k, v, grad_attn, dq, dk, dv, T, N, K, d, saved, saved_bytes, true, workspace,
+                              const void* out, const void* saved, size_t saved_bytes, void* dq, void* dk,
+                              void* dv, int64_t T, int64_t N, int K, int d, void* workspace,
+                              size_t workspace_bytes, void* stream) {
+    if (T > 0 && N > 0) {
+        if (!out) return fail(RFA_ERR_NULL_POINTER, "rfa_causal_backward_saved: NULL forward output");
+        if (!aligned16(out)) return fail(RFA_ERR_ALIGNMENT, "rfa_causal_backward_saved: out must be 16-byte aligned");
+    }
+    return causal_backward_impl(q, k, v, grad_attn, out, dq, dk, dv, T, N, K, d, saved, saved_bytes, true, workspace,
                                 workspace_bytes, stream);
 }
 
-static int causal_backward_impl(const void* q, const void* k, const void* v, const void* grad_attn, void* dq,
-                                void* dk, void* dv, int64_t T, int64_t N, int K, int d, const void* saved,
-                                size_t saved_bytes, bool have_saved, void* workspace, size_t workspace_bytes,
-                                void* stream) {
+static int causal_backward_impl(const void* q, const void* k, const void* v, const void* grad_attn,
+                                const void* out, void* dq, void* dk, void* dv, int64_t T, int64_t N, int K, int d,
+                                const void* saved, size_t saved_bytes, bool have_saved, void* workspace,
+                                size_t workspace_bytes, void* stream) {
     if (int rc = check_causal_dims(T, N, K, d)) return rc;
     if (T == 0 || N == 0) return RFA_OK;
     const float* savedS = nullptr;
     const float* savedZ = nullptr;
+    const float* savedDen = nullptr;
     if (have_saved) {
-        size_t zoff = 0;
-        const size_t need = saved_state_bytes(T, N, K, d, &zoff);
+        size_t zoff = 0, doff = 0;
+        const size_t need = saved_state_bytes(T, N, K, d, &zoff, &doff);
         if (!saved || saved_bytes < need || !aligned16(saved))
             return fail(RFA_ERR_WORKSPACE, "rfa_causal_backward_saved: saved-state buffer of %zu bytes required, got %zu",
                         need, saved ? saved_bytes : (size_t)0);
         savedS = static_cast<const float*>(saved);
         savedZ = reinterpret_cast<const float*>(static_cast<const char*>(saved) + zoff);
+        savedDen = reinterpret_cast<const float*>(static_cast<const char*>(saved) + doff);
     }
     if (!q || !k || !v || !grad_attn || !dq || !dk || !dv)
         return fail(RFA_ERR_NULL_POINTER, "rfa_causal_backward: NULL tensor pointer");
@@ -585,11 +606,12 @@ static int causal_backward_impl(const void* q, const void* k, const void* v, con
     auto* kh = static_cast<const rfa::half_t*>(k);
     auto* vh = static_cast<const rfa::half_t*>(v);
     auto* gh = static_cast<const rfa::half_t*>(grad_attn);
+    auto* outh = static_cast<const rfa::half_t*>(out);
     auto* dqh = static_cast<rfa::half_t*>(dq);
     auto* dkh = static_cast<rfa::half_t*>(dk);
     auto* dvh = static_cast<rfa::half_t*>(dv);
     char* ws = static_cast<char*>(workspace);
-#define RFA_CALL_BWD(KD, DH) launch_backward<KD, DH>(qh, kh, vh, gh, dqh, dkh, dvh, (int)T, (int)N, p, ws, wl, savedS, savedZ, st)
+#define RFA_CALL_BWD(KD, DH) launch_backward<KD, DH>(qh, kh, vh, gh, outh, dqh, dkh, dvh, (int)T, (int)N, p, ws, wl, savedS, savedZ, savedDen, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_BWD)
 #undef RFA_CALL_BWD
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");

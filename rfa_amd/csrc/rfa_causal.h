@@ -54,6 +54,8 @@ struct CausalCfg {
     static constexpr size_t kFwdLds = (size_t)(2 * C * LDQ + C * LDV + C * LDA) * 2 + (KD + NH * C) * 4;
     static constexpr size_t kBwdDqLds =
         (size_t)(2 * C * LDQ + 2 * C * LDV + C * LDA) * 2 + (size_t)(KD + (2 * NH + NW + 2) * C) * 4;
+    static constexpr size_t kBwdDqSavedLds =
+        (size_t)(2 * C * LDQ + 2 * C * LDV + C * LDA) * 2 + (size_t)(KD + C) * 4;
     static constexpr size_t kBwdDkLds =
         (size_t)(2 * C * LDQ + 2 * C * LDV + 2 * C * LDA) * 2 + (size_t)(KD + C) * 4;
 };
@@ -174,6 +176,9 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
 // held as accumulator tiles S[kt][ct] with element (k = 16kt+4G+e, c = w*DS+16ct+i).
 // ---------------------------------------------------------------------------
 //
+// den_out (causal only, may be NULL) receives the raw denominators rowsum(A) + q.z, fp32
+// [T][N], for a backward pass that reuses them.
+//
 // CAUSAL = false is the cross-attention readout (reference: cross_attention.py:266-269):
 // the state is the fixed total S, z of the source (wsS/wsZ hold one state per
 // sequence), there is no intra-chunk term and no update, and the denominator is
@@ -181,8 +186,8 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
 template <int KD, int DH, int NW, bool CAUSAL>
 __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
-    half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ, int T,
-    int N, int nseg, int seg_len) {
+    half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
+    float* __restrict__ den_out, int T, int N, int nseg, int seg_len) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = Cfg::DS;
@@ -379,6 +384,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
                 for (int h = 1; h < NH; ++h) dr += dparts[h * C + i];
                 const float inv = 1.0f / fmaxf(CAUSAL ? dr : fabsf(dr), 1.0f);
                 if (t0 + i < t_end) {
+                    if (CAUSAL && den_out && w == 0 && G == 0) den_out[(int64_t)(t0 + i) * N + n] = dr;
 #pragma unroll
                     for (int ct = 0; ct < NCT; ++ct) {
                         f4 o = acc[it][ct];
@@ -440,8 +446,8 @@ __device__ __forceinline__ void wg_barrier() {
 template <int KD, int DH>
 __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
-    half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ, int T,
-    int N, int nseg, int seg_len) {
+    half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
+    float* __restrict__ den_out, int T, int N, int nseg, int seg_len) {
     using Cfg = FwdPipeCfg<KD, DH>;
     constexpr int NT = 256;      // threads per group
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = DH / 4;
@@ -550,7 +556,10 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
                 }
                 part += (qz4[0] + qz4[1]) + (qz4[2] + qz4[3]);
                 part = sum_over_groups(part);
-                if (G == 0) dens[16 * w + row] = part;
+                if (G == 0) {
+                    dens[16 * w + row] = part;
+                    if (den_out && t0 + 16 * w + row < t_end) den_out[(int64_t)(t0 + 16 * w + row) * N + n] = part;
+                }
 #pragma unroll
                 for (int a = 0; a < 4; ++a)
                     *reinterpret_cast<h4*>(As + (16 * w + row) * LDA + 16 * a + 4 * G) = to_h4(at[a]);
@@ -996,6 +1005,258 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
 }
 
 // ---------------------------------------------------------------------------
+// backward, forward-in-time sweep for a backward pass that has the forward's output and
+// raw denominators (rfa_causal_forward_save).  With num = out * den the reference's
+// g . num (rfa.py:91) is (g . out) * den, so
+//     gz_i = den_raw_i > 1 ? -(g_i . out_i) / den_i : 0
+// is known when a chunk is loaded, and the sweep needs neither A = Q K^T nor the row sums
+// of A*X and Q*Y:  per chunk, with G^ = G / den written to LDS at load time,
+//     X^T = V G^T (tiles for 16 rows per wave),  P = tril(X + gz 1^T)
+//     dQ^T = K^T P^T + S G^T + z gz^T ;  dR += G^T Q, dr += Q^T gz, S += V^T K, z += K^T 1
+// Same state ownership, totals and (gz) stash as k_causal_bwd_dq<.., CAUSAL = true>.
+// ---------------------------------------------------------------------------
+template <int KD, int DH, int NW>
+__global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
+    const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    const half_t* __restrict__ g, const half_t* __restrict__ o, const float* __restrict__ den_raw,
+    half_t* __restrict__ dq, const float* __restrict__ wsS, const float* __restrict__ wsZ,
+    float* __restrict__ wsR, float* __restrict__ wsr, float* __restrict__ gz_ws, int T, int N, int nseg,
+    int seg_len) {
+    using Cfg = CausalCfg<KD, DH, NW>;
+    constexpr int NT = Cfg::NT;
+    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS;
+    constexpr int NKT = KS / 16, NCT = DH / 16;
+    constexpr int PPR = DH / 8, VP = ChunkRegs<DH, NT>::kPieces;
+    static_assert(KD % (16 * NW) == 0, "feature rows do not split over the waves");
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
+    half_t* Ks = Qs + C * LDQ;
+    half_t* Vs = Ks + C * LDQ;
+    half_t* Gs = Vs + C * LDV;        // G / den
+    half_t* Ps = Gs + C * LDV;
+    float* zs = reinterpret_cast<float*>(Ps + C * LDA);
+    float* gzs = zs + KD;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, G = lane >> 4;
+    const int rb = w & 3, half = w >> 2;
+    constexpr int JPW = Cfg::JPW;
+    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    const int t_begin = seg * seg_len;
+    const int t_end = min(T, t_begin + seg_len);
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+    const half_t* qb = q + (int64_t)n * KD;
+    const half_t* kb = k + (int64_t)n * KD;
+    const half_t* vb = v + (int64_t)n * DH;
+    const half_t* gb = g + (int64_t)n * DH;
+    const half_t* ob = o + (int64_t)n * DH;
+    half_t* dqb = dq + (int64_t)n * KD;
+
+    f4 ST[NCT][NKT], RT[NCT][NKT];
+#pragma unroll
+    for (int a = 0; a < NCT; ++a)
+#pragma unroll
+        for (int b = 0; b < NKT; ++b) { ST[a][b] = f4_zero(); RT[a][b] = f4_zero(); }
+    f4 zacc[NKT], racc[NKT];
+#pragma unroll
+    for (int b = 0; b < NKT; ++b) { zacc[b] = f4_zero(); racc[b] = f4_zero(); }
+    const h8 ones = h8_ones();
+    for (int s = 0; s < seg; ++s) {
+        const float* si = wsS + ((int64_t)(n * nseg + s) * KD) * DH;
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+                ST[ct][kt] += *reinterpret_cast<const f4*>(si + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+            zacc[kt] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * nseg + s) * KD + w * KS + 16 * kt + 4 * G);
+    }
+
+    RFA_TICK_INIT();
+    ChunkRegs<KD, NT> rq, rk;
+    ChunkRegs<DH, NT> rv, rg, ro;
+    float dn[VP];
+    auto prefetch = [&](int t0) {
+        const int rows = t_end - t0;
+        chunk_g2r<KD, NT>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<DH, NT>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+        chunk_g2r<DH, NT>(ro, ob + (int64_t)t0 * v_stride, v_stride, rows, tid);
+        chunk_g2r<KD, NT>(rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<DH, NT>(rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+#pragma unroll
+        for (int it = 0; it < VP; ++it) {
+            const int r_ = min((tid + NT * it) / PPR, rg.rows - 1);
+            dn[it] = den_raw[(int64_t)(t0 + r_) * N + n];
+        }
+    };
+    prefetch(t_begin);
+    RFA_TICK(0);
+
+    for (int t0 = t_begin; t0 < t_end; t0 += C) {
+        chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
+        chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
+        chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
+        // G^ = G / den into LDS; gz from g . out (the PPR lanes holding one row are adjacent)
+#pragma unroll
+        for (int it = 0; it < VP; ++it) {
+            const int pc = tid + NT * it;
+            const int r_ = pc / PPR, c8 = pc % PPR;
+            union { uint4 u; h8 h; } xg, xo;
+            xg.u = rg.v[it];
+            xo.u = ro.v[it];
+            float dot = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dot += (float)xg.h[e] * (float)xo.h[e];
+#pragma unroll
+            for (int m = 1; m < PPR; m <<= 1) dot += __shfl_xor(dot, m, 64);
+            const bool valid = r_ < rg.rows;
+            const float inv = valid ? 1.0f / fmaxf(dn[it], 1.0f) : 0.f;
+            const float gzv = (valid && dn[it] > 1.0f) ? -dot * inv : 0.f;
+            h8 y;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)xg.h[e] * inv);
+            *reinterpret_cast<h8*>(Gs + r_ * LDV + c8 * 8) = y;
+            if (c8 == 0) {
+                gzs[r_] = gzv;
+                if (valid) gz_ws[(int64_t)(t0 + r_) * N + n] = gzv;
+            }
+        }
+        if (row == 0) {
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) *reinterpret_cast<f4*>(zs + w * KS + 16 * kt + 4 * G) = zacc[kt];
+        }
+        RFA_TICK(1);
+        __syncthreads();
+        RFA_TICK(2);
+        if (t0 + C < t_end) prefetch(t0 + C);
+        RFA_TICK(3);
+
+        // ---- phase A: P rows of this wave's row block (tiles jt = half*JPW + a); Y^T for the wave's feature slice
+        f4 yt[NKT][4];      // (S G^T) tiles (m=k, n=i), k in this wave's slice, all i
+        {
+            const int i = 16 * rb + row;
+            const float gzi = gzs[i];
+            f4 xt[JPW];     // X^T tiles (m=j, n=i)
+#pragma unroll
+            for (int a = 0; a < JPW; ++a) xt[a] = f4_zero();
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 bg = row8(Gs, LDV, i, cs * 32, G);
+#pragma unroll
+                for (int a = 0; a < JPW; ++a)
+                    xt[a] = mfma32(row8(Vs, LDV, 16 * (half * JPW + a) + row, cs * 32, G), bg, xt[a]);
+            }
+#pragma unroll
+            for (int a = 0; a < JPW; ++a) {
+                const int jt = half * JPW + a;
+                h4 pv;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = 16 * jt + 4 * G + e;
+                    pv[e] = (j <= i) ? (half_t)(xt[a][e] + gzi) : (half_t)0.f;
+                }
+                *reinterpret_cast<h4*>(Ps + i * LDA + 16 * jt + 4 * G) = pv;
+            }
+            RFA_TICK(4);
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int it = 0; it < 4; ++it) yt[kt][it] = f4_zero();
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 hi[NKT], lo[NKT];
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) acc_to_operand(ST[2 * cs][kt], ST[2 * cs + 1][kt], hi[kt], lo[kt]);
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    h8 bg = row_split8(Gs, LDV, 16 * it + row, cs * 32, G);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(hi[kt], bg, yt[kt][it]);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(lo[kt], bg, yt[kt][it]);
+                }
+            }
+        }
+        RFA_TICK(5);
+        __syncthreads();
+        RFA_TICK(6);
+
+        // ---- phase D: dQ^T tiles (m=k, n=i), then the carried sums
+        {
+            h8 kf[NKT][2];   // K column fragments: K[j = 32js+8G+e][k = w*KS+16kt+i]
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int js = 0; js < 2; ++js) kf[kt][js] = col8(Ks, LDQ, js * 32, w * KS + 16 * kt, lane);
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int i = 16 * it + row;
+                const float gzi = gzs[i];
+                const h8 bp0 = row8(Ps, LDA, i, 0, G);
+                const h8 bp1 = row8(Ps, LDA, i, 32, G);
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) {
+                    f4 zv = *reinterpret_cast<const f4*>(zs + w * KS + 16 * kt + 4 * G);
+                    f4 acc;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e] = yt[kt][it][e] + gzi * zv[e];
+                    acc = mfma32(kf[kt][0], bp0, acc);
+                    if (it >= 2) acc = mfma32(kf[kt][1], bp1, acc);
+                    if (t0 + i < t_end)
+                        *reinterpret_cast<h4*>(dqb + (int64_t)(t0 + i) * k_stride + w * KS + 16 * kt + 4 * G) = to_h4(acc);
+                }
+            }
+            RFA_TICK(7);
+#pragma unroll
+            for (int js = 0; js < 2; ++js) {
+                h8 qf[NKT];   // Q column fragments
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) qf[kt] = col8(Qs, LDQ, js * 32, w * KS + 16 * kt, lane);
+                h8 ghi, glo;
+                f8_to_operand(*reinterpret_cast<const f4*>(gzs + js * 32 + 8 * G),
+                              *reinterpret_cast<const f4*>(gzs + js * 32 + 8 * G + 4), ghi, glo);
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) {
+                    racc[kt] = mfma32(qf[kt], ghi, racc[kt]);
+                    zacc[kt] = mfma32(kf[kt][js], ones, zacc[kt]);
+                }
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt], glo, racc[kt]);
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct) {
+                    h8 gf = col8(Gs, LDV, js * 32, 16 * ct, lane);
+                    h8 vf = col8(Vs, LDV, js * 32, 16 * ct, lane);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) RT[ct][kt] = mfma32(gf, qf[kt], RT[ct][kt]);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) ST[ct][kt] = mfma32(vf, kf[kt][js], ST[ct][kt]);
+                }
+            }
+        }
+        RFA_TICK(8);
+        __syncthreads();
+        RFA_TICK(9);
+    }
+
+    if (seg > 0) {   // totals of segment 0 are never consumed
+        float* ro_ = wsR + ((int64_t)(n * nseg + seg) * KD) * DH;
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+                *reinterpret_cast<f4*>(ro_ + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G) = RT[ct][kt];
+        if (row == 0) {
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+                *reinterpret_cast<f4*>(wsr + (int64_t)(n * nseg + seg) * KD + w * KS + 16 * kt + 4 * G) = racc[kt];
+        }
+    }
+    RFA_TICK(10);
+}
+
+// ---------------------------------------------------------------------------
 // backward, reverse-in-time sweep: dK, dV.  R is carried twice, once per
 // contraction: RT[ct][kt] (c = 16ct+4G+e, k = w*KS+16kt+i) contracts over c for
 // dK; RR[kt][ct] (k = 16kt+4G+e, c = w*DS+16ct+i) contracts over k for dV.
@@ -1127,7 +1388,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
             chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
 #pragma unroll
             for (int it = 0; it < ChunkRegs<DH, NT>::kPieces; ++it)
-                inv_den[it] = inv_den[it] > 0.f ? 1.0f / inv_den[it] : 0.f;   // den >= 1 on valid rows
+                inv_den[it] = 1.0f / fmaxf(inv_den[it], 1.0f);   // den_ws may hold raw or clamped denominators
             chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
             if (tid < C) gzs[tid] = tid < rg.rows ? gz_next : 0.f;
         }

@@ -77,20 +77,21 @@ class RFA(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q: Tensor, k: Tensor, v: Tensor) -> Tensor:
-        """attn [tgt_len, bsz*heads, head_dim]; saves (q, k, v) like rfa.py:124 (plus the segment totals)."""
+        """attn [tgt_len, bsz*heads, head_dim]; saves (q, k, v) like rfa.py:124 (plus the forward products backward reuses)."""
         ctx.in_dtypes = (q.dtype, k.dtype, v.dtype)
         q, k, v = _as_kernel_input(q), _as_kernel_input(k), _as_kernel_input(v)
         if any(ctx.needs_input_grad):
-            # also keep the per-segment state totals so that backward need not rebuild them
-            attn, seg_totals = rfa_hip.forward_save(q, k, v)
-            ctx.save_for_backward(q, k, v, seg_totals)
+            # also keep the forward's segment totals, denominators and output so that backward
+            # need not rebuild them
+            attn, fwd_saved = rfa_hip.forward_save(q, k, v)
+            ctx.save_for_backward(q, k, v, attn, fwd_saved)
         else:
             attn = rfa_hip.forward(q, k, v)
         return attn.to(ctx.in_dtypes[2])
 
     @staticmethod
     def backward(ctx, grad_attn: Tensor):
-        q, k, v, seg_totals = ctx.saved_tensors
-        gq, gk, gv = rfa_hip.backward_saved(q, k, v, _as_kernel_input(grad_attn), seg_totals)
+        q, k, v, attn, fwd_saved = ctx.saved_tensors
+        gq, gk, gv = rfa_hip.backward_saved(q, k, v, _as_kernel_input(grad_attn), attn, fwd_saved)
         dq, dk, dv = ctx.in_dtypes
         return gq.to(dq), gk.to(dk), gv.to(dv)

@@ -78,7 +78,7 @@ def forward(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
 
 
 def forward_save(q: Tensor, k: Tensor, v: Tensor):
-    """(attn, saved): forward that also returns the per-segment state totals for backward_saved."""
+    """(attn, saved): forward that also returns the buffer backward_saved reuses (segment totals, denominators)."""
     _check_qkv(q, k, v)
     lib = _lib.load()
     T, N, K = q.shape
@@ -95,12 +95,14 @@ def forward_save(q: Tensor, k: Tensor, v: Tensor):
     return out, saved
 
 
-def backward_saved(q: Tensor, k: Tensor, v: Tensor, grad_attn: Tensor, saved: Tensor) -> List[Tensor]:
-    """backward() that reuses the segment totals returned by forward_save for the same q, k, v."""
+def backward_saved(q: Tensor, k: Tensor, v: Tensor, grad_attn: Tensor, out: Tensor, saved: Tensor) -> List[Tensor]:
+    """backward() that reuses what forward_save returned for the same q, k, v: its output and saved buffer."""
     _check_qkv(q, k, v)
     _check_half_cuda("grad_attn", grad_attn, 3)
+    _check_half_cuda("out", out, 3)
     _require(grad_attn.shape == v.shape, ValueError,
              f"grad_attn {tuple(grad_attn.shape)} must match v {tuple(v.shape)}")
+    _require(out.shape == v.shape, ValueError, f"out {tuple(out.shape)} must match v {tuple(v.shape)}")
     _require(saved.is_cuda and saved.dtype == torch.uint8 and saved.is_contiguous(), TypeError,
              "saved must be the byte buffer returned by forward_save")
     lib = _lib.load()
@@ -111,7 +113,7 @@ def backward_saved(q: Tensor, k: Tensor, v: Tensor, grad_attn: Tensor, saved: Te
         nbytes = lib.rfa_causal_backward_workspace_bytes(T, N, K, d)
         ws = _workspace(nbytes, q.device)
         _lib.check(lib.rfa_causal_backward_saved(q.data_ptr(), k.data_ptr(), v.data_ptr(), grad_attn.data_ptr(),
-                                                 saved.data_ptr(), saved.numel(), dq.data_ptr(), dk.data_ptr(),
+                                                 out.data_ptr(), saved.data_ptr(), saved.numel(), dq.data_ptr(), dk.data_ptr(),
                                                  dv.data_ptr(), T, N, K, d, ws.data_ptr(), nbytes,
                                                  _stream_ptr(q.device)))
     return [dq, dk, dv]
