@@ -141,6 +141,12 @@ constexpr int causal_waves(int KD, int DH) { return (DH >= 128 && KD >= 128) ? 8
 // K >= 128
 constexpr int dq_waves(int KD, int DH) { return KD >= 128 ? 8 : 4; }
 
+// waves that own the forward state (value-column slices): 4 in the two-stage pipelined forward
+constexpr int fwd_state_waves(int KD, int DH) {
+    return ((size_t)2 * ((size_t)(2 * 64 * (KD + rfa::lds_pad(KD)) + 64 * (DH + rfa::lds_pad(DH)) + 64 * (64 + 8)) * 2 + 64 * 4) + KD * 4
+            <= 160 * 1024) ? 4 : causal_waves(KD, DH);
+}
+
 template <typename Kern>
 int set_lds(Kern kern, size_t bytes) {
     RFA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -155,15 +161,17 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
     // the two-stage pipelined forward needs both chunk buffers in LDS: K <= 128
     constexpr bool PIPE = rfa::FwdPipeCfg<KD, DH>::kLds <= 160 * 1024;
     constexpr int NW = PIPE ? 4 : causal_waves(KD, DH);
+    static_assert(NW == fwd_state_waves(KD, DH), "fragment layout of the segment totals");
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
-    float* wsS = reinterpret_cast<float*>(ws + wl.S);
-    // with a saved-state buffer the z totals are written there directly (z has one layout)
+    // with a saved buffer the segment totals are written there directly (S in the forward's
+    // fragment order, which the saved-pair backward reads as is)
+    float* wsS = savedS ? savedS : reinterpret_cast<float*>(ws + wl.S);
     float* wsZ = savedZ ? savedZ : reinterpret_cast<float*>(ws + wl.Z);
     if (p.nseg > 1) {
         auto kern = rfa::k_segment_state<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(64 * NW), Cfg::kSegStateLds, st,
-                           k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, savedS, T, N, p.nseg, p.nseg - 1, p.seg_len);
+                           k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     if constexpr (PIPE) {
         auto kern = rfa::k_causal_fwd_pipe<KD, DH>;
@@ -209,7 +217,7 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         // the forward's output and raw denominators are at hand: the sweep that needs no A = Q K^T
         constexpr int NWQ = dq_waves(KD, DH);
         using CfgQ = rfa::CausalCfg<KD, DH, NWQ>;
-        auto kern = rfa::k_causal_bwd_dq_saved<KD, DH, NWQ>;
+        auto kern = rfa::k_causal_bwd_dq_saved<KD, DH, NWQ, fwd_state_waves(KD, DH)>;
         if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g, out,
                    savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len);

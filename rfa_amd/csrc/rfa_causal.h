@@ -50,7 +50,10 @@ struct CausalCfg {
     static constexpr int LDA = C + 8;
     static constexpr int DS = DH / NW;    // value columns owned by one wave
     static constexpr int KS = KD / NW;    // feature rows owned by one wave
-    static constexpr size_t kSegStateLds = (size_t)(C * LDQ + C * LDV) * 2;
+    // chunks k_segment_state keeps in flight / in LDS at once (as many as fit in 128 KB, at most 4)
+    static constexpr int kSegStateGroup =
+        (size_t)(C * LDQ + C * LDV) * 2 * 4 <= 128 * 1024 ? 4 : ((size_t)(C * LDQ + C * LDV) * 2 * 2 <= 128 * 1024 ? 2 : 1);
+    static constexpr size_t kSegStateLds = (size_t)(C * LDQ + C * LDV) * 2 * kSegStateGroup;
     static constexpr size_t kFwdLds = (size_t)(2 * C * LDQ + C * LDV + C * LDA) * 2 + (KD + NH * C) * 4;
     static constexpr size_t kBwdDqLds =
         (size_t)(2 * C * LDQ + 2 * C * LDV + C * LDA) * 2 + (size_t)(KD + (2 * NH + NW + 2) * C) * 4;
@@ -88,8 +91,7 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
     constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / NW;
     static_assert(DH % (16 * NW) == 0 && NKT % NW == 0, "shape does not split over the waves");
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    half_t* Ks = reinterpret_cast<half_t*>(smem_raw);
-    half_t* Vs = Ks + C * LDQ;
+    half_t* Ks = reinterpret_cast<half_t*>(smem_raw);   // kGroup buffers of [K chunk | V chunk]
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -112,39 +114,50 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
     for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
     const h8 ones = h8_ones();
 
-    ChunkRegs<KD, NT> rk;
-    ChunkRegs<DH, NT> rv;
-    chunk_g2r<KD, NT>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
-    chunk_g2r<DH, NT>(rv, vb + (int64_t)t_begin * v_stride, v_stride, t_end - t_begin, tid);
-    if (mrow) chunk_mask_rows<KD, NT>(rk, mrow + t_begin, tid);
-    for (int t0 = t_begin; t0 < t_end; t0 += C) {
-        chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
-        chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
-        __syncthreads();
-        if (t0 + C < t_end) {
-            chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, t_end - t0 - C, tid);
-            chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, t_end - t0 - C, tid);
-            if (mrow) chunk_mask_rows<KD, NT>(rk, mrow + t0 + C, tid);
+    // The chunks are requested kGroup at a time, each into its own LDS buffer: one memory round
+    // trip per group instead of one per chunk (the products of a chunk take far less time than
+    // its load), one barrier per chunk and one more where the buffers are reused.
+    constexpr int kGroup = Cfg::kSegStateGroup;
+    ChunkRegs<KD, NT> rk[kGroup];
+    ChunkRegs<DH, NT> rv[kGroup];
+    for (int tg = t_begin; tg < t_end; tg += kGroup * C) {
+#pragma unroll
+        for (int c = 0; c < kGroup; ++c) {
+            // branch-free: a chunk past the end re-reads the last valid row and is never used
+            const int t0 = min(tg + c * C, t_end - 1);
+            chunk_g2r<KD, NT>(rk[c], kb + (int64_t)t0 * k_stride, k_stride, t_end - t0, tid);
+            chunk_g2r<DH, NT>(rv[c], vb + (int64_t)t0 * v_stride, v_stride, t_end - t0, tid);
+            if (mrow) chunk_mask_rows<KD, NT>(rk[c], mrow + t0, tid);
         }
-        h8 bv[NCT][2];
+        if (tg > t_begin) __syncthreads();   // every wave is done with the previous group's buffers
 #pragma unroll
-        for (int ct = 0; ct < NCT; ++ct)
+        for (int c = 0; c < kGroup; ++c) {
+            const int t0 = tg + c * C;
+            if (t0 >= t_end) break;
+            half_t* Kc = Ks + c * (C * LDQ + C * LDV);
+            half_t* Vc = Kc + C * LDQ;
+            chunk_r2s<KD, NT>(rk[c], Kc, LDQ, tid);
+            chunk_r2s<DH, NT>(rv[c], Vc, LDV, tid);
+            __syncthreads();
+            h8 bv[NCT][2];
 #pragma unroll
-            for (int js = 0; js < 2; ++js) bv[ct][js] = col8(Vs, LDV, js * 32, w * DS + 16 * ct, lane);
+            for (int ct = 0; ct < NCT; ++ct)
 #pragma unroll
-        for (int kt = 0; kt < NKT; ++kt)
+                for (int js = 0; js < 2; ++js) bv[ct][js] = col8(Vc, LDV, js * 32, w * DS + 16 * ct, lane);
 #pragma unroll
-            for (int js = 0; js < 2; ++js) {
-                h8 ak = col8(Ks, LDQ, js * 32, 16 * kt, lane);
+            for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-                for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, bv[ct][js], S[kt][ct]);
-            }
+                for (int js = 0; js < 2; ++js) {
+                    h8 ak = col8(Kc, LDQ, js * 32, 16 * kt, lane);
 #pragma unroll
-        for (int a = 0; a < NKTW; ++a)
+                    for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, bv[ct][js], S[kt][ct]);
+                }
 #pragma unroll
-            for (int js = 0; js < 2; ++js)
-                zacc[a] = mfma32(col8(Ks, LDQ, js * 32, 16 * (w * NKTW + a), lane), ones, zacc[a]);
-        __syncthreads();
+            for (int a = 0; a < NKTW; ++a)
+#pragma unroll
+                for (int js = 0; js < 2; ++js)
+                    zacc[a] = mfma32(col8(Kc, LDQ, js * 32, 16 * (w * NKTW + a), lane), ones, zacc[a]);
+        }
     }
     float* so = wsS + ((int64_t)(n * nseg + seg) * KD) * DH;
     if (FRAG) {
@@ -1015,7 +1028,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
 //     dQ^T = K^T P^T + S G^T + z gz^T ;  dR += G^T Q, dr += Q^T gz, S += V^T K, z += K^T 1
 // Same state ownership, totals and (gz) stash as k_causal_bwd_dq<.., CAUSAL = true>.
 // ---------------------------------------------------------------------------
-template <int KD, int DH, int NW>
+template <int KD, int DH, int NW, int NWF>
 __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, const half_t* __restrict__ o, const float* __restrict__ den_raw,
@@ -1062,13 +1075,24 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
 #pragma unroll
     for (int b = 0; b < NKT; ++b) { zacc[b] = f4_zero(); racc[b] = f4_zero(); }
     const h8 ones = h8_ones();
+    // The segment totals are read in the accumulator-fragment order the forward pass left them
+    // in (k_segment_state<FRAG = true> for NWF waves: [wave][kt][ct][lane][4], element
+    // (k = 16kt + 4G + e, c = wave*DSF + 16ct + i)); this wave needs (c = 16ct + 4G + e,
+    // k = w*KS + 16kt + row), i.e. four scalar loads per tile, once per workgroup.
+    constexpr int DSF = DH / NWF, NCTF = DSF / 16, NKTF = KD / 16;
     for (int s = 0; s < seg; ++s) {
         const float* si = wsS + ((int64_t)(n * nseg + s) * KD) * DH;
 #pragma unroll
-        for (int ct = 0; ct < NCT; ++ct)
+        for (int ct = 0; ct < NCT; ++ct) {
+            const int wf = (16 * ct) / DSF, ctf = ((16 * ct) % DSF) / 16;
 #pragma unroll
-            for (int kt = 0; kt < NKT; ++kt)
-                ST[ct][kt] += *reinterpret_cast<const f4*>(si + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
+            for (int kt = 0; kt < NKT; ++kt) {
+                const int ktf = (w * KS + 16 * kt) / 16;
+                const float* tile = si + (int64_t)((wf * NKTF + ktf) * NCTF + ctf) * 256 + ((row >> 2) * 16 + 4 * G) * 4 + (row & 3);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ST[ct][kt][e] += tile[4 * e];
+            }
+        }
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
             zacc[kt] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * nseg + s) * KD + w * KS + 16 * kt + 4 * G);
