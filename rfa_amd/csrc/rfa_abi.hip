@@ -215,12 +215,24 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
     const float* den_in = den;
     if (savedDen) {
         // the forward's output and raw denominators are at hand: the sweep that needs no A = Q K^T
-        constexpr int NWQ = dq_waves(KD, DH);
-        using CfgQ = rfa::CausalCfg<KD, DH, NWQ>;
-        auto kern = rfa::k_causal_bwd_dq_saved<KD, DH, NWQ, fwd_state_waves(KD, DH)>;
-        if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
-        RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g, out,
-                   savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len);
+        if constexpr (KD >= 256 && DH >= 128) {
+            // both carried states of one workgroup would not fit the register file: the feature
+            // rows split over two workgroups (half of S^T and of R^T each)
+            constexpr int KL = KD / 2;
+            constexpr int NWQ = dq_waves(KL, DH);
+            using CfgQ = rfa::CausalCfg<KL, DH, NWQ>;
+            auto kern = rfa::k_causal_bwd_dq_saved<KL, DH, NWQ, fwd_state_waves(KD, DH), KD>;
+            if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
+            RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(2 * N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g,
+                       out, savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len);
+        } else {
+            constexpr int NWQ = dq_waves(KD, DH);
+            using CfgQ = rfa::CausalCfg<KD, DH, NWQ>;
+            auto kern = rfa::k_causal_bwd_dq_saved<KD, DH, NWQ, fwd_state_waves(KD, DH)>;
+            if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
+            RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g, out,
+                       savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len);
+        }
         den_in = savedDen;
     } else {
         constexpr int NWQ = dq_waves(KD, DH);
@@ -230,6 +242,17 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqLds, st, q, k, v, g,
                            dq, inS, inZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
     }
+    if constexpr (KD >= 256) {
+        // two copies of R in one workgroup would not fit the register file: dK and dV in separate
+        // workgroups (one copy each); measured 2.5x (d = 64) and 1.7x (d = 128) faster at K = 256,
+        // slower than the shared tile phase below at K <= 128
+        constexpr int NWR = (KD >= 128 && DH >= 128) ? 8 : 4;
+        using CfgR = rfa::DkDvRoleCfg<KD, DH, NWR>;
+        auto kern = rfa::k_causal_bwd_dkdv_roles<KD, DH, NWR>;
+        if (int rc = set_lds(kern, CfgR::kLds)) return rc;
+        RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(2 * N * p.nseg), dim3(64 * NWR), CfgR::kLds, st, q, k, v, g, dk, dv,
+                   (const float*)wsR, (const float*)wsr, den_in, (const float*)gz, T, N, p.nseg, p.seg_len);
+    } else
     if constexpr (NW == 4 && KD <= 128) {
         // 8 waves with the state phase split by role (dK waves / dV waves): two waves per SIMD
         // (K = 256 would spill at 256 registers per wave)

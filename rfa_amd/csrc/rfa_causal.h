@@ -1028,7 +1028,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
 //     dQ^T = K^T P^T + S G^T + z gz^T ;  dR += G^T Q, dr += Q^T gz, S += V^T K, z += K^T 1
 // Same state ownership, totals and (gz) stash as k_causal_bwd_dq<.., CAUSAL = true>.
 // ---------------------------------------------------------------------------
-template <int KD, int DH, int NW, int NWF>
+template <int KD, int DH, int NW, int NWF, int KDG = KD>
 __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, const half_t* __restrict__ o, const float* __restrict__ den_raw,
@@ -1055,16 +1055,22 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     const int row = lane & 15, G = lane >> 4;
     const int rb = w & 3, half = w >> 2;
     constexpr int JPW = Cfg::JPW;
-    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    // KDG > KD: the feature rows are split over KDG / KD workgroups per (sequence, segment);
+    // this one owns features [koff, koff + KD) of the KDG-wide rows
+    static_assert(KDG % KD == 0, "feature split");
+    const int nsq = N * nseg;
+    const int koff = (int)(blockIdx.x / nsq) * KD;
+    const int bid = blockIdx.x % nsq;
+    const int n = bid / nseg, seg = bid % nseg;
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
-    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
-    const half_t* qb = q + (int64_t)n * KD;
-    const half_t* kb = k + (int64_t)n * KD;
+    const int64_t k_stride = (int64_t)N * KDG, v_stride = (int64_t)N * DH;
+    const half_t* qb = q + (int64_t)n * KDG + koff;
+    const half_t* kb = k + (int64_t)n * KDG + koff;
     const half_t* vb = v + (int64_t)n * DH;
     const half_t* gb = g + (int64_t)n * DH;
     const half_t* ob = o + (int64_t)n * DH;
-    half_t* dqb = dq + (int64_t)n * KD;
+    half_t* dqb = dq + (int64_t)n * KDG + koff;
 
     f4 ST[NCT][NKT], RT[NCT][NKT];
 #pragma unroll
@@ -1079,15 +1085,15 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     // in (k_segment_state<FRAG = true> for NWF waves: [wave][kt][ct][lane][4], element
     // (k = 16kt + 4G + e, c = wave*DSF + 16ct + i)); this wave needs (c = 16ct + 4G + e,
     // k = w*KS + 16kt + row), i.e. four scalar loads per tile, once per workgroup.
-    constexpr int DSF = DH / NWF, NCTF = DSF / 16, NKTF = KD / 16;
+    constexpr int DSF = DH / NWF, NCTF = DSF / 16, NKTF = KDG / 16;
     for (int s = 0; s < seg; ++s) {
-        const float* si = wsS + ((int64_t)(n * nseg + s) * KD) * DH;
+        const float* si = wsS + ((int64_t)(n * nseg + s) * KDG) * DH;
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct) {
             const int wf = (16 * ct) / DSF, ctf = ((16 * ct) % DSF) / 16;
 #pragma unroll
             for (int kt = 0; kt < NKT; ++kt) {
-                const int ktf = (w * KS + 16 * kt) / 16;
+                const int ktf = (koff + w * KS + 16 * kt) / 16;
                 const float* tile = si + (int64_t)((wf * NKTF + ktf) * NCTF + ctf) * 256 + ((row >> 2) * 16 + 4 * G) * 4 + (row & 3);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) ST[ct][kt][e] += tile[4 * e];
@@ -1095,7 +1101,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
         }
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
-            zacc[kt] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * nseg + s) * KD + w * KS + 16 * kt + 4 * G);
+            zacc[kt] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * nseg + s) * KDG + koff + w * KS + 16 * kt + 4 * G);
     }
 
     RFA_TICK_INIT();
@@ -1144,7 +1150,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
             *reinterpret_cast<h8*>(Gs + r_ * LDV + c8 * 8) = y;
             if (c8 == 0) {
                 gzs[r_] = gzv;
-                if (valid) gz_ws[(int64_t)(t0 + r_) * N + n] = gzv;
+                if (valid && koff == 0) gz_ws[(int64_t)(t0 + r_) * N + n] = gzv;
             }
         }
         if (row == 0) {
@@ -1265,16 +1271,16 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     }
 
     if (seg > 0) {   // totals of segment 0 are never consumed
-        float* ro_ = wsR + ((int64_t)(n * nseg + seg) * KD) * DH;
+        float* ro_ = wsR + ((int64_t)(n * nseg + seg) * KDG) * DH;
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct)
 #pragma unroll
             for (int kt = 0; kt < NKT; ++kt)
-                *reinterpret_cast<f4*>(ro_ + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G) = RT[ct][kt];
+                *reinterpret_cast<f4*>(ro_ + (koff + w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G) = RT[ct][kt];
         if (row == 0) {
 #pragma unroll
             for (int kt = 0; kt < NKT; ++kt)
-                *reinterpret_cast<f4*>(wsr + (int64_t)(n * nseg + seg) * KD + w * KS + 16 * kt + 4 * G) = racc[kt];
+                *reinterpret_cast<f4*>(wsr + (int64_t)(n * nseg + seg) * KDG + koff + w * KS + 16 * kt + 4 * G) = racc[kt];
         }
     }
     RFA_TICK(10);
@@ -1591,6 +1597,367 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
         }
         __syncthreads();
     }
+}
+
+
+// ---------------------------------------------------------------------------
+// backward, reverse-in-time sweep with dK and dV in separate workgroups (causal only).
+// The two gradients share the masked tiles' inputs but nothing else:
+//     dK = P^T Q + V R^T + 1 r^T   reads q, v, g   carries R^T (d x K) and r
+//     dV = A^T (G/den) + K R       reads q, k, g   carries R   (K x d)
+// so a workgroup of either role holds one copy of R instead of two and loads three of the
+// four operands; the two roles of a (sequence, segment) run side by side on one CU where
+// LDS and registers allow, each hiding the other's LDS and memory latency.
+// grid = 2 * N * nseg: blocks [0, N*nseg) compute dK, blocks [N*nseg, 2*N*nseg) compute dV.
+// ---------------------------------------------------------------------------
+template <int KD, int DH, int NW>
+struct DkDvRoleCfg {
+    using Base = CausalCfg<KD, DH, NW>;
+    static constexpr int C = Base::C, LDQ = Base::LDQ, LDV = Base::LDV, LDA = Base::LDA;
+    static constexpr size_t kDkLds = (size_t)(C * LDQ + 2 * C * LDV + C * LDA) * 2 + (size_t)(KD + C) * 4;
+    static constexpr size_t kDvLds = (size_t)(2 * C * LDQ + C * LDV + C * LDA) * 2;
+    static constexpr size_t kLds = kDkLds > kDvLds ? kDkLds : kDvLds;
+};
+
+template <int KD, int DH, int NW>
+__device__ __forceinline__ void dkdv_role_dk(
+    unsigned char* smem_raw, int bid, const half_t* __restrict__ q, const half_t* __restrict__ v,
+    const half_t* __restrict__ g, half_t* __restrict__ dk, const float* __restrict__ wsR,
+    const float* __restrict__ wsr, const float* __restrict__ den_ws, const float* __restrict__ gz_ws, int T,
+    int N, int nseg, int seg_len) {
+    using Cfg = CausalCfg<KD, DH, NW>;
+    constexpr int NT = Cfg::NT;
+    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = KD / NW;
+    constexpr int NKT = KS / 16, NCT = DH / 16, JPW = Cfg::JPW;
+    constexpr int PPRV = DH / 8, VP = ChunkRegs<DH, NT>::kPieces;
+    static_assert(KD % (16 * NW) == 0, "feature rows do not split over the waves");
+    half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
+    half_t* Vs = Qs + C * LDQ;
+    half_t* Gs = Vs + C * LDV;       // G / den
+    half_t* PTs = Gs + C * LDV;      // PT[j][i] = P[i][j]
+    float* rs = reinterpret_cast<float*>(PTs + C * LDA);
+    float* gzs = rs + KD;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, G = lane >> 4;
+    const int rb = w & 3, half = w >> 2;
+    const int n = bid / nseg, seg = bid % nseg;
+    const int t_begin = seg * seg_len;
+    const int t_end = min(T, t_begin + seg_len);
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+    const half_t* qb = q + (int64_t)n * KD;
+    const half_t* vb = v + (int64_t)n * DH;
+    const half_t* gb = g + (int64_t)n * DH;
+    half_t* dkb = dk + (int64_t)n * KD;
+
+    f4 RT[NCT][NKT];   // element (c = 16ct+4G+e, k = w*KS+16kt+i)
+#pragma unroll
+    for (int a = 0; a < NCT; ++a)
+#pragma unroll
+        for (int b = 0; b < NKT; ++b) RT[a][b] = f4_zero();
+    f4 racc[NKT];
+#pragma unroll
+    for (int b = 0; b < NKT; ++b) racc[b] = f4_zero();
+    for (int s = seg + 1; s < nseg; ++s) {
+        const float* ri = wsR + ((int64_t)(n * nseg + s) * KD) * DH;
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+                RT[ct][kt] += *reinterpret_cast<const f4*>(ri + (w * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+            racc[kt] += *reinterpret_cast<const f4*>(wsr + (int64_t)(n * nseg + s) * KD + w * KS + 16 * kt + 4 * G);
+    }
+
+    ChunkRegs<KD, NT> rq;
+    ChunkRegs<DH, NT> rv, rg;
+    float inv_den[VP];
+    float gz_next = 0.f;
+    auto prefetch = [&](int t0) {
+        const int rows = t_end - t0;
+        chunk_g2r<KD, NT>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<DH, NT>(rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+        chunk_g2r<DH, NT>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+#pragma unroll
+        for (int it = 0; it < VP; ++it) {
+            const int r_ = min((tid + NT * it) / PPRV, rg.rows - 1);
+            inv_den[it] = den_ws[(int64_t)(t0 + r_) * N + n];
+        }
+        gz_next = gz_ws[(int64_t)(t0 + min(tid & (C - 1), rg.rows - 1)) * N + n];
+    };
+    const int n_chunks = (t_end - t_begin + C - 1) / C;
+    prefetch(t_begin + (n_chunks - 1) * C);
+    for (int ci = n_chunks - 1; ci >= 0; --ci) {
+        const int t0 = t_begin + ci * C;
+        chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
+        chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
+#pragma unroll
+        for (int it = 0; it < VP; ++it) inv_den[it] = 1.0f / fmaxf(inv_den[it], 1.0f);
+        chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
+        if (tid < C) gzs[tid] = tid < rg.rows ? gz_next : 0.f;
+        if (row == 0) {
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) *reinterpret_cast<f4*>(rs + w * KS + 16 * kt + 4 * G) = racc[kt];
+        }
+        __syncthreads();
+        if (ci > 0) prefetch(t0 - C);
+
+        // ---- P tiles (m=i, n=j) for column block rb, rows 16*(half*JPW + a)
+        {
+            f4 p_[JPW];
+#pragma unroll
+            for (int a = 0; a < JPW; ++a) p_[a] = f4_zero();
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 bv = row8(Vs, LDV, 16 * rb + row, cs * 32, G);
+#pragma unroll
+                for (int a = 0; a < JPW; ++a)
+                    p_[a] = mfma32(row8(Gs, LDV, 16 * (half * JPW + a) + row, cs * 32, G), bv, p_[a]);
+            }
+            const int j = 16 * rb + row;
+#pragma unroll
+            for (int a = 0; a < JPW; ++a) {
+                const int it = half * JPW + a;
+                h4 pv;
+                f4 gzv = *reinterpret_cast<const f4*>(gzs + 16 * it + 4 * G);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int i = 16 * it + 4 * G + e;
+                    pv[e] = (i >= j) ? (half_t)(p_[a][e] + gzv[e]) : (half_t)0.f;
+                }
+                *reinterpret_cast<h4*>(PTs + j * LDA + 16 * it + 4 * G) = pv;
+            }
+        }
+        __syncthreads();
+
+        // ---- dK^T tiles (m=k, n=j) and the carried sums
+        {
+            h8 qf[NKT][2];
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int is = 0; is < 2; ++is) qf[kt][is] = col8(Qs, LDQ, is * 32, w * KS + 16 * kt, lane);
+            f4 dkacc[NKT][4];
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) {
+                f4 rv4 = *reinterpret_cast<const f4*>(rs + w * KS + 16 * kt + 4 * G);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    f4 acc = rv4;
+                    if (jt < 2) acc = mfma32(qf[kt][0], row8(PTs, LDA, 16 * jt + row, 0, G), acc);
+                    acc = mfma32(qf[kt][1], row8(PTs, LDA, 16 * jt + row, 32, G), acc);
+                    dkacc[kt][jt] = acc;
+                }
+            }
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 hi[NKT], lo[NKT];
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) acc_to_operand(RT[2 * cs][kt], RT[2 * cs + 1][kt], hi[kt], lo[kt]);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    h8 bvv = row_split8(Vs, LDV, 16 * jt + row, cs * 32, G);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(hi[kt], bvv, dkacc[kt][jt]);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(lo[kt], bvv, dkacc[kt][jt]);
+                }
+            }
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                const int jj = 16 * jt + row;
+                if (t0 + jj < t_end) {
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt)
+                        *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + w * KS + 16 * kt + 4 * G) = to_h4(dkacc[kt][jt]);
+                }
+            }
+#pragma unroll
+            for (int is = 0; is < 2; ++is) {
+                h8 ghi, glo;   // r (m=k) += Q^T gz
+                f8_to_operand(*reinterpret_cast<const f4*>(gzs + is * 32 + 8 * G),
+                              *reinterpret_cast<const f4*>(gzs + is * 32 + 8 * G + 4), ghi, glo);
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt][is], ghi, racc[kt]);
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) racc[kt] = mfma32(qf[kt][is], glo, racc[kt]);
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct) {
+                    h8 gf = col8(Gs, LDV, is * 32, 16 * ct, lane);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt) RT[ct][kt] = mfma32(gf, qf[kt][is], RT[ct][kt]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <int KD, int DH, int NW>
+__device__ __forceinline__ void dkdv_role_dv(
+    unsigned char* smem_raw, int bid, const half_t* __restrict__ q, const half_t* __restrict__ k,
+    const half_t* __restrict__ g, half_t* __restrict__ dv, const float* __restrict__ wsR,
+    const float* __restrict__ den_ws, int T, int N, int nseg, int seg_len) {
+    using Cfg = CausalCfg<KD, DH, NW>;
+    constexpr int NT = Cfg::NT;
+    constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = DH / NW;
+    constexpr int NKT2 = KD / 16, NCT2 = DS / 16, JPW = Cfg::JPW;
+    constexpr int PPRV = DH / 8, VP = ChunkRegs<DH, NT>::kPieces;
+    static_assert(DH % (16 * NW) == 0, "value columns do not split over the waves");
+    half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
+    half_t* Ks = Qs + C * LDQ;
+    half_t* Gs = Ks + C * LDQ;       // G / den
+    half_t* ATs = Gs + C * LDV;      // AT[j][i] = A[i][j]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, G = lane >> 4;
+    const int rb = w & 3, half = w >> 2;
+    const int n = bid / nseg, seg = bid % nseg;
+    const int t_begin = seg * seg_len;
+    const int t_end = min(T, t_begin + seg_len);
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+    const half_t* qb = q + (int64_t)n * KD;
+    const half_t* kb = k + (int64_t)n * KD;
+    const half_t* gb = g + (int64_t)n * DH;
+    half_t* dvb = dv + (int64_t)n * DH;
+
+    f4 RR[NKT2][NCT2];   // element (k = 16kt+4G+e, c = w*DS+16ct+i)
+#pragma unroll
+    for (int a = 0; a < NKT2; ++a)
+#pragma unroll
+        for (int b = 0; b < NCT2; ++b) RR[a][b] = f4_zero();
+    for (int s = seg + 1; s < nseg; ++s) {
+        const float* ri = wsR + ((int64_t)(n * nseg + s) * KD) * DH;
+#pragma unroll
+        for (int kt = 0; kt < NKT2; ++kt)
+#pragma unroll
+            for (int ct = 0; ct < NCT2; ++ct)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    RR[kt][ct][e] += ri[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row];
+    }
+
+    ChunkRegs<KD, NT> rq, rk;
+    ChunkRegs<DH, NT> rg;
+    float inv_den[VP];
+    auto prefetch = [&](int t0) {
+        const int rows = t_end - t0;
+        chunk_g2r<KD, NT>(rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<KD, NT>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<DH, NT>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+#pragma unroll
+        for (int it = 0; it < VP; ++it) {
+            const int r_ = min((tid + NT * it) / PPRV, rg.rows - 1);
+            inv_den[it] = den_ws[(int64_t)(t0 + r_) * N + n];
+        }
+    };
+    const int n_chunks = (t_end - t_begin + C - 1) / C;
+    prefetch(t_begin + (n_chunks - 1) * C);
+    for (int ci = n_chunks - 1; ci >= 0; --ci) {
+        const int t0 = t_begin + ci * C;
+        chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
+        chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
+#pragma unroll
+        for (int it = 0; it < VP; ++it) inv_den[it] = 1.0f / fmaxf(inv_den[it], 1.0f);
+        chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
+        __syncthreads();
+        if (ci > 0) prefetch(t0 - C);
+
+        // ---- A tiles (m=i, n=j) for column block rb, rows 16*(half*JPW + a)
+        {
+            f4 a_[JPW];
+#pragma unroll
+            for (int a = 0; a < JPW; ++a) a_[a] = f4_zero();
+#pragma unroll
+            for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 bk = row8(Ks, LDQ, 16 * rb + row, ks * 32, G);
+#pragma unroll
+                for (int a = 0; a < JPW; ++a)
+                    a_[a] = mfma32(row8(Qs, LDQ, 16 * (half * JPW + a) + row, ks * 32, G), bk, a_[a]);
+            }
+            const int j = 16 * rb + row;
+#pragma unroll
+            for (int a = 0; a < JPW; ++a) {
+                const int it = half * JPW + a;
+                h4 av;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int i = 16 * it + 4 * G + e;
+                    av[e] = (i >= j) ? (half_t)a_[a][e] : (half_t)0.f;
+                }
+                *reinterpret_cast<h4*>(ATs + j * LDA + 16 * it + 4 * G) = av;
+            }
+        }
+        __syncthreads();
+
+        // ---- dV^T tiles (m=c, n=j) and the carried sum
+        {
+            h8 gf2[NCT2][2];
+#pragma unroll
+            for (int ct = 0; ct < NCT2; ++ct)
+#pragma unroll
+                for (int is = 0; is < 2; ++is) gf2[ct][is] = col8(Gs, LDV, is * 32, w * DS + 16 * ct, lane);
+            f4 dvacc[NCT2][4];
+#pragma unroll
+            for (int ct = 0; ct < NCT2; ++ct)
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    f4 acc = f4_zero();
+                    if (jt < 2) acc = mfma32(gf2[ct][0], row8(ATs, LDA, 16 * jt + row, 0, G), acc);
+                    acc = mfma32(gf2[ct][1], row8(ATs, LDA, 16 * jt + row, 32, G), acc);
+                    dvacc[ct][jt] = acc;
+                }
+#pragma unroll
+            for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 hi[NCT2], lo[NCT2];
+#pragma unroll
+                for (int ct = 0; ct < NCT2; ++ct) acc_to_operand(RR[2 * ks][ct], RR[2 * ks + 1][ct], hi[ct], lo[ct]);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    h8 bkk = row_split8(Ks, LDQ, 16 * jt + row, ks * 32, G);
+#pragma unroll
+                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(hi[ct], bkk, dvacc[ct][jt]);
+#pragma unroll
+                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(lo[ct], bkk, dvacc[ct][jt]);
+                }
+            }
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                const int jj = 16 * jt + row;
+                if (t0 + jj < t_end) {
+#pragma unroll
+                    for (int ct = 0; ct < NCT2; ++ct)
+                        *reinterpret_cast<h4*>(dvb + (int64_t)(t0 + jj) * v_stride + w * DS + 16 * ct + 4 * G) = to_h4(dvacc[ct][jt]);
+                }
+            }
+#pragma unroll
+            for (int is = 0; is < 2; ++is)
+#pragma unroll
+                for (int kt = 0; kt < NKT2; ++kt) {
+                    h8 qa = col8(Qs, LDQ, is * 32, 16 * kt, lane);
+#pragma unroll
+                    for (int ct = 0; ct < NCT2; ++ct) RR[kt][ct] = mfma32(qa, gf2[ct][is], RR[kt][ct]);
+                }
+        }
+        __syncthreads();
+    }
+}
+
+template <int KD, int DH, int NW>
+__global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv_roles(
+    const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    const half_t* __restrict__ g, half_t* __restrict__ dk, half_t* __restrict__ dv,
+    const float* __restrict__ wsR, const float* __restrict__ wsr, const float* __restrict__ den_ws,
+    const float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int nsq = N * nseg;
+    if ((int)blockIdx.x < nsq)
+        dkdv_role_dk<KD, DH, NW>(smem_raw, blockIdx.x, q, v, g, dk, wsR, wsr, den_ws, gz_ws, T, N, nseg, seg_len);
+    else
+        dkdv_role_dv<KD, DH, NW>(smem_raw, blockIdx.x - nsq, q, k, g, dv, wsR, den_ws, T, N, nseg, seg_len);
 }
 
 }  // namespace rfa
