@@ -70,6 +70,16 @@ int rfa_causal_forward(const void* q, const void* k, const void* v, void* out, i
                        int64_t N, int K, int d, void* workspace, size_t workspace_bytes,
                        void* stream);
 
+/* Prefill for incremental decoding: rfa_causal_forward over a prompt of T steps that also
+ * returns the state after the last step, s fp32 [N, K, d] and z fp32 [N, K] (every element
+ * written; zero for T = 0), from which rfa_incremental / rfa_incremental_fused continue.
+ * In the reference the same hand-off is T calls of incremental_rfa from a zero state
+ * (causal_attention.py:17-54, saved_state keys "prev_s" / "prev_z" at :249-265).
+ * Workspace: rfa_causal_forward_workspace_bytes. */
+int rfa_causal_prefill(const void* q, const void* k, const void* v, void* out, float* s, float* z,
+                       int64_t T, int64_t N, int K, int d, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
 size_t rfa_causal_backward_workspace_bytes(int64_t T, int64_t N, int K, int d);
 int rfa_causal_backward(const void* q, const void* k, const void* v, const void* grad_attn,
                         void* dq, void* dk, void* dv, int64_t T, int64_t N, int K, int d,

@@ -37,6 +37,7 @@ SIGNATURES = {
     "rfa_causal_num_segments": (c_int, [c_int64, c_int64]),
     "rfa_causal_forward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
     "rfa_causal_forward": (c_int, [c_void_p] * 4 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "rfa_causal_prefill": (c_int, [c_void_p] * 6 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "rfa_causal_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
     "rfa_causal_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "rfa_causal_saved_state_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),

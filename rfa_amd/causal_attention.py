@@ -107,6 +107,18 @@ def cuda_causal_rfa(*, phi_q: Tensor, phi_k: Tensor, v: Tensor,
 hip_causal_rfa = cuda_causal_rfa
 
 
+def reorder_incremental_state(saved_state: Dict[str, Optional[Tensor]], new_order: Tensor) -> Dict[str, Optional[Tensor]]:
+    """Beam-search reordering of a decode state: batch entry i of the result is entry
+    ``new_order[i]`` of the input ("prev_s" [bsz, heads, 2*proj_dim, head_dim], "prev_z"
+    [bsz, heads, 2*proj_dim]; reference state layout causal_attention.py:249-265).  The dict
+    is updated in place and returned; an empty state is left alone."""
+    for key in ("prev_s", "prev_z"):
+        t = saved_state.get(key)
+        if t is not None:
+            saved_state[key] = t.index_select(0, new_order.to(device=t.device, dtype=torch.long))
+    return saved_state
+
+
 class CausalAttention(nn.Module):
     """Causal random feature self-attention (reference causal_attention.py:154-280)."""
 
@@ -141,8 +153,11 @@ class CausalAttention(nn.Module):
                 saved_state: Optional[Dict[str, Optional[Tensor]]] = None) -> Tensor:
         """x: [tgt_len, bsz, embed_dim]; random_matrices: [heads, proj_dim, head_dim] -> [tgt_len, bsz, embed_dim].
 
-        With ``saved_state`` (a dict, tgt_len must be 1) one decode step is taken and the
-        state under "prev_s" / "prev_z" is advanced (reference causal_attention.py:249-265).
+        With ``saved_state`` (a dict) the call is part of incremental decoding and the state under
+        "prev_s" / "prev_z" is advanced (reference causal_attention.py:249-265, where tgt_len
+        must be 1).  Here tgt_len > 1 is accepted as well: on an empty state the whole prompt
+        goes through the chunked-scan kernels once and the state after its last step is kept
+        (prefill); on a non-empty state the steps are taken one after the other.
         """
         tgt_len, bsz, embed_dim = x.size()
         assert embed_dim == self.embed_dim
@@ -153,20 +168,35 @@ class CausalAttention(nn.Module):
                                   sigma=self.sigma if self.reparam_proj else None,
                                   reparam_proj=self.reparam_proj)
         if saved_state is not None:
-            assert tgt_len == 1
             feat = 2 * self.proj_dim
             s, z = saved_state.get("prev_s"), saved_state.get("prev_z")
-            if s is None:
-                s = torch.zeros((bsz, self.num_heads, feat, self.head_dim), device=x.device, dtype=torch.float32)
-                z = torch.zeros((bsz, self.num_heads, feat), device=x.device, dtype=torch.float32)
+            if s is None and tgt_len > 1:
+                # prefill: one pass of the training kernels over the prompt, final state kept
+                with torch.no_grad():
+                    phi_q = random_project(x=q, random_matrices=w)
+                    phi_k = random_project(x=k, random_matrices=w)
+                    pad = _drop_scalar_mask(key_padding_mask)
+                    if pad is not None:
+                        phi_k = phi_k.masked_fill(pad.to(torch.bool).transpose(0, 1)[:, :, None, None], 0.0)
+                    n = bsz * self.num_heads
+                    attn, s, z = rfa_hip.prefill(
+                        phi_q.to(torch.float16).contiguous().view(tgt_len, n, feat),
+                        phi_k.to(torch.float16).contiguous().view(tgt_len, n, feat),
+                        v.detach().to(torch.float16).contiguous().view(tgt_len, n, self.head_dim))
+                s = s.view(bsz, self.num_heads, feat, self.head_dim)
+                z = z.view(bsz, self.num_heads, feat)
             else:
-                assert z is not None
-                s = s.to(torch.float32).contiguous()
-                z = z.to(torch.float32).contiguous()
-            # feature map + state update + readout in one kernel; state advanced in place
-            attn = rfa_hip.incremental_fused(
-                q.detach().to(torch.float16).contiguous(), k.detach().to(torch.float16).contiguous(),
-                v.detach().to(torch.float16).contiguous(), w.detach().to(torch.float16).contiguous(), SCALE, s, z)
+                if s is None:
+                    s = torch.zeros((bsz, self.num_heads, feat, self.head_dim), device=x.device, dtype=torch.float32)
+                    z = torch.zeros((bsz, self.num_heads, feat), device=x.device, dtype=torch.float32)
+                else:
+                    assert z is not None
+                    s = s.to(torch.float32).contiguous()
+                    z = z.to(torch.float32).contiguous()
+                # feature map + state update + readout in one kernel per step; state advanced in place
+                attn = rfa_hip.incremental_fused(
+                    q.detach().to(torch.float16).contiguous(), k.detach().to(torch.float16).contiguous(),
+                    v.detach().to(torch.float16).contiguous(), w.detach().to(torch.float16).contiguous(), SCALE, s, z)
             attn = attn.to(x.dtype).view(tgt_len, bsz, embed_dim)
             saved_state["prev_s"], saved_state["prev_z"] = s, z
         else:

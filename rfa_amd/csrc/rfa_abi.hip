@@ -157,7 +157,7 @@ int set_lds(Kern kern, size_t bytes) {
 template <int KD, int DH>
 int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, rfa::half_t* out,
                    int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, float* savedS, float* savedZ,
-                   float* savedDen, hipStream_t st) {
+                   float* savedDen, float* final_s, float* final_z, hipStream_t st) {
     // the two-stage pipelined forward needs both chunk buffers in LDS: K <= 128
     constexpr bool PIPE = rfa::FwdPipeCfg<KD, DH>::kLds <= 160 * 1024;
     constexpr int NW = PIPE ? 4 : causal_waves(KD, DH);
@@ -177,12 +177,12 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
         auto kern = rfa::k_causal_fwd_pipe<KD, DH>;
         if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(512), rfa::FwdPipeCfg<KD, DH>::kLds, st, q, k, v, out,
-                           wsS, wsZ, savedDen, T, N, p.nseg, p.seg_len);
+                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len);
     } else {
         auto kern = rfa::k_causal_fwd<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q, k, v, out,
-                           wsS, wsZ, savedDen, T, N, p.nseg, p.seg_len);
+                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len);
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -309,8 +309,8 @@ int launch_cross_readout(const rfa::half_t* q, const float* s, const float* z, r
     auto kern = rfa::k_causal_fwd<KD, DH, NW, false>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
     RFA_LAUNCH(CROSS_READOUT, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q,
-                       (const rfa::half_t*)nullptr, (const rfa::half_t*)nullptr, out, s, z, (float*)nullptr, T, N,
-                       p.nseg, p.seg_len);
+                       (const rfa::half_t*)nullptr, (const rfa::half_t*)nullptr, out, s, z, (float*)nullptr,
+                       (float*)nullptr, (float*)nullptr, T, N, p.nseg, p.seg_len);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -527,23 +527,40 @@ size_t rfa_causal_saved_state_bytes(int64_t T, int64_t N, int K, int d) {
 }
 
 static int causal_forward_impl(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
-                               int K, int d, void* saved, size_t saved_bytes, bool want_saved, void* workspace,
-                               size_t workspace_bytes, void* stream);
+                               int K, int d, void* saved, size_t saved_bytes, bool want_saved, float* final_s,
+                               float* final_z, void* workspace, size_t workspace_bytes, void* stream);
 
 int rfa_causal_forward(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
                        int K, int d, void* workspace, size_t workspace_bytes, void* stream) {
-    return causal_forward_impl(q, k, v, out, T, N, K, d, nullptr, 0, false, workspace, workspace_bytes, stream);
+    return causal_forward_impl(q, k, v, out, T, N, K, d, nullptr, 0, false, nullptr, nullptr, workspace,
+                               workspace_bytes, stream);
+}
+
+int rfa_causal_prefill(const void* q, const void* k, const void* v, void* out, float* s, float* z, int64_t T,
+                       int64_t N, int K, int d, void* workspace, size_t workspace_bytes, void* stream) {
+    if (int rc = check_causal_dims(T, N, K, d)) return rc;
+    if (N == 0) return RFA_OK;
+    if (!s || !z) return fail(RFA_ERR_NULL_POINTER, "rfa_causal_prefill: NULL state pointer");
+    if (!aligned16(s) || !aligned16(z)) return fail(RFA_ERR_ALIGNMENT, "rfa_causal_prefill: state must be 16-byte aligned");
+    if (T == 0) {   // empty prompt: the state is zero
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        zero_f32(s, (int64_t)N * K * d, st);
+        zero_f32(z, (int64_t)N * K, st);
+        return RFA_OK;
+    }
+    return causal_forward_impl(q, k, v, out, T, N, K, d, nullptr, 0, false, s, z, workspace, workspace_bytes, stream);
 }
 
 int rfa_causal_forward_save(const void* q, const void* k, const void* v, void* out, void* saved,
                             size_t saved_bytes, int64_t T, int64_t N, int K, int d, void* workspace,
                             size_t workspace_bytes, void* stream) {
-    return causal_forward_impl(q, k, v, out, T, N, K, d, saved, saved_bytes, true, workspace, workspace_bytes, stream);
+    return causal_forward_impl(q, k, v, out, T, N, K, d, saved, saved_bytes, true, nullptr, nullptr, workspace,
+                               workspace_bytes, stream);
 }
 
 static int causal_forward_impl(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
-                               int K, int d, void* saved, size_t saved_bytes, bool want_saved, void* workspace,
-                               size_t workspace_bytes, void* stream) {
+                               int K, int d, void* saved, size_t saved_bytes, bool want_saved, float* final_s,
+                               float* final_z, void* workspace, size_t workspace_bytes, void* stream) {
     if (int rc = check_causal_dims(T, N, K, d)) return rc;
     if (T == 0 || N == 0) return RFA_OK;
     float* savedS = nullptr;
@@ -573,7 +590,7 @@ static int causal_forward_impl(const void* q, const void* k, const void* v, void
     auto* vh = static_cast<const rfa::half_t*>(v);
     auto* oh = static_cast<rfa::half_t*>(out);
     char* ws = static_cast<char*>(workspace);
-#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedS, savedZ, savedDen, st)
+#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedS, savedZ, savedDen, final_s, final_z, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_FWD)
 #undef RFA_CALL_FWD
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");

@@ -190,7 +190,8 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
 // ---------------------------------------------------------------------------
 //
 // den_out (causal only, may be NULL) receives the raw denominators rowsum(A) + q.z, fp32
-// [T][N], for a backward pass that reuses them.
+// [T][N], for a backward pass that reuses them.  final_s / final_z (causal only, may be NULL)
+// receive the state after step T - 1, fp32 [N][KD][DH] / [N][KD].
 //
 // CAUSAL = false is the cross-attention readout (reference: cross_attention.py:266-269):
 // the state is the fixed total S, z of the source (wsS/wsZ hold one state per
@@ -200,7 +201,8 @@ template <int KD, int DH, int NW, bool CAUSAL>
 __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
-    float* __restrict__ den_out, int T, int N, int nseg, int seg_len) {
+    float* __restrict__ den_out, float* __restrict__ final_s, float* __restrict__ final_z, int T, int N,
+    int nseg, int seg_len) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = Cfg::DS;
@@ -428,6 +430,21 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
         __syncthreads();
         RFA_TICK(10);
     }
+    // the state after the last step of the sequence, for a decode loop that continues from it
+    if (CAUSAL && final_s && seg == nseg - 1) {
+        float* so = final_s + (int64_t)n * KD * DH;
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) so[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row] = S[kt][ct][e];
+        if (row == 0) {
+#pragma unroll
+            for (int a = 0; a < NKTW; ++a)
+                *reinterpret_cast<f4*>(final_z + (int64_t)n * KD + 16 * (w * NKTW + a) + 4 * G) = zacc[a];
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -460,7 +477,8 @@ template <int KD, int DH>
 __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
-    float* __restrict__ den_out, int T, int N, int nseg, int seg_len) {
+    float* __restrict__ den_out, float* __restrict__ final_s, float* __restrict__ final_z, int T, int N,
+    int nseg, int seg_len) {
     using Cfg = FwdPipeCfg<KD, DH>;
     constexpr int NT = 256;      // threads per group
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = DH / 4;
@@ -587,6 +605,11 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
             wg_barrier();
             RFA_TICK_AT(5, 0);
         }
+        if (final_z && seg == nseg - 1 && row == 0) {
+#pragma unroll
+            for (int a = 0; a < NKTW; ++a)
+                *reinterpret_cast<f4*>(final_z + (int64_t)n * KD + 16 * (w * NKTW + a) + 4 * G) = zacc[a];
+        }
     } else {
         half_t* ob = out + (int64_t)n * DH;
         f4 S[NKT][NCT];
@@ -678,6 +701,15 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
             RFA_TICK_AT(13, 256);
             wg_barrier();
             RFA_TICK_AT(14, 256);
+        }
+        if (final_s && seg == nseg - 1) {
+            float* so = final_s + (int64_t)n * KD * DH;
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) so[(16 * kt + 4 * G + e) * DH + w * DS + 16 * ct + row] = S[kt][ct][e];
         }
     }
 }

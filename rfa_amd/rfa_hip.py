@@ -77,6 +77,26 @@ def forward(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
     return out
 
 
+def prefill(q: Tensor, k: Tensor, v: Tensor):
+    """(attn, s, z): causal forward over a prompt plus the state after its last step.
+
+    s: fp32 [N, K, d], z: fp32 [N, K] -- what ``incremental`` / ``incremental_fused`` continue from.
+    """
+    _check_qkv(q, k, v)
+    lib = _lib.load()
+    T, N, K = q.shape
+    d = v.shape[2]
+    out = torch.empty_like(v)
+    s = torch.empty((N, K, d), dtype=torch.float32, device=q.device)
+    z = torch.empty((N, K), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        nbytes = lib.rfa_causal_forward_workspace_bytes(T, N, K, d)
+        ws = _workspace(nbytes, q.device)
+        _lib.check(lib.rfa_causal_prefill(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), s.data_ptr(),
+                                          z.data_ptr(), T, N, K, d, ws.data_ptr(), nbytes, _stream_ptr(q.device)))
+    return out, s, z
+
+
 def forward_save(q: Tensor, k: Tensor, v: Tensor):
     """(attn, saved): forward that also returns the buffer backward_saved reuses (segment totals, denominators)."""
     _check_qkv(q, k, v)

@@ -161,3 +161,55 @@ def test_incremental_rfa_out_of_place_and_inplace():
                                          v.float().cpu().reshape(T, B * H, d))
     got = torch.cat([a1, a2], 0).float().cpu().reshape(T, B * H, d)
     assert (got - want).abs().max().item() <= 2e-3
+
+
+@pytest.mark.parametrize("T,B,H,d,D", [(1, 1, 1, 64, 64), (70, 2, 2, 64, 64), (1024, 1, 4, 64, 64), (200, 1, 2, 128, 32),
+                                        (130, 1, 1, 128, 128)])
+def test_prefill_state_equals_loop_state_and_decode_continues(T, B, H, d, D):
+    """rfa_causal_prefill: the output is the causal forward, the returned state is what T
+    single steps from a zero state leave behind (reference causal_attention.py:42-50), and a
+    decode step taken from it reproduces row T of the forward over T + 1 steps."""
+    from rfa_amd import rfa_hip
+    q, k, v, _ = O.make_qkv(T + 1, B, H, d, seed=900 + T)
+    W = O.make_w(d, D, H)
+    N, K = B * H, 2 * D
+    pq = O.random_project(q.float(), W).half().reshape(T + 1, N, K)
+    pk = O.random_project(k.float(), W).half().reshape(T + 1, N, K)
+    vv = v.reshape(T + 1, N, d)
+    cq, ck, cv = pq.cuda(), pk.cuda(), vv.cuda()
+    print(f"prefill T={T} N={N} K={K} d={d}", flush=True)
+    out, s, z = rfa_hip.prefill(cq[:T].contiguous(), ck[:T].contiguous(), cv[:T].contiguous())
+    assert torch.equal(out, rfa_hip.forward(cq[:T].contiguous(), ck[:T].contiguous(), cv[:T].contiguous()))
+    _, s_ref, z_ref = O.causal_forward_loop(pq[:T].float(), pk[:T].float(), vv[:T].float())
+    assert _rel(s.cpu(), s_ref) < 1e-5 and _rel(z.cpu(), z_ref) < 1e-5
+    step = rfa_hip.incremental(cq[T:].contiguous(), ck[T:].contiguous(), cv[T:].contiguous(), s, z)
+    full = O.causal_forward_chunked(pq.float(), pk.float(), vv.float()) if T > 256 else \
+        O.causal_forward_cumsum(pq.float(), pk.float(), vv.float())
+    assert (step.float().cpu() - full[T:]).abs().max().item() <= 2e-3
+
+
+def test_module_prefill_then_decode_and_beam_reorder():
+    """CausalAttention with saved_state: a prompt of several steps on an empty state (prefill),
+    then single steps, equals the full causal forward; reorder_incremental_state permutes the
+    batch entries of the state."""
+    from rfa_amd.causal_attention import CausalAttention, reorder_incremental_state
+    torch.manual_seed(11)
+    T, B, E, H, d, D = 96, 3, 128, 2, 64, 64
+    m = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half()
+    W = O.make_w(d, D, H).half().cuda()
+    x = (torch.randn(T + 2, B, E) * 0.5).half().cuda()
+    with torch.no_grad():
+        full = m(x, W)
+        state = {}
+        a = m(x[:T], W, saved_state=state)                    # prefill
+        b1 = m(x[T:T + 1], W, saved_state=state)               # decode steps
+        b2 = m(x[T + 1:], W, saved_state=state)
+    got = torch.cat([a, b1, b2], 0)
+    assert (got.float() - full.float()).abs().max().item() <= 4e-3
+    assert state["prev_s"].shape == (B, H, 2 * D, d) and state["prev_z"].dtype == torch.float32
+    order = torch.tensor([2, 0, 0])
+    before = {k_: t.clone() for k_, t in state.items()}
+    reorder_incremental_state(state, order.cuda())
+    for k_ in ("prev_s", "prev_z"):
+        assert torch.equal(state[k_], before[k_][order.cuda()])
+    assert reorder_incremental_state({}, order) == {}
