@@ -292,10 +292,17 @@ int launch_cross_state(const rfa::half_t* k, const rfa::half_t* v, const uint8_t
     constexpr int NW = causal_waves(KD, DH);
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
-    auto kern = rfa::k_segment_state<KD, DH, NW, false>;
-    if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
-    RFA_LAUNCH(SEG_STATE, kern, dim3(N), dim3(64 * NW), Cfg::kSegStateLds, st, k, v, mask, H, s, z,
-               (float*)nullptr, T, N, 1, 1, seg_len);
+    if (mask) {
+        auto kern = rfa::k_segment_state<KD, DH, NW, false, true>;
+        if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
+        RFA_LAUNCH(SEG_STATE, kern, dim3(N), dim3(64 * NW), Cfg::kSegStateLds, st, k, v, mask, H, s, z,
+                   (float*)nullptr, T, N, 1, 1, seg_len);
+    } else {
+        auto kern = rfa::k_segment_state<KD, DH, NW, false, false>;
+        if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
+        RFA_LAUNCH(SEG_STATE, kern, dim3(N), dim3(64 * NW), Cfg::kSegStateLds, st, k, v, mask, H, s, z,
+                   (float*)nullptr, T, N, 1, 1, seg_len);
+    }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }

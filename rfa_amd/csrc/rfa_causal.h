@@ -68,7 +68,7 @@ struct CausalCfg {
 // grid = N * nseg_out: the causal passes compute nseg_out = nseg - 1 totals per
 // sequence (the last segment's total is never consumed); cross attention computes
 // the single total of the whole source (nseg = nseg_out = 1) straight into its
-// state tensors.  pad_mask ([B, T] bytes, 1 = padded key, may be NULL) zeroes
+// state tensors.  pad_mask ([B, T] bytes, 1 = padded key; read only when MASKED) zeroes
 // phi_k rows (reference: cross_attention.py:97-100).
 // ---------------------------------------------------------------------------
 //
@@ -80,7 +80,7 @@ struct CausalCfg {
 // wave w owns the feature tiles kt in [w*NKTW, (w+1)*NKTW).
 // row_copy (FRAG only, may be NULL) receives a second, row-major copy of the totals: the
 // forward pass of a training step hands it to the backward pass, which then skips this pass.
-template <int KD, int DH, int NW, bool FRAG>
+template <int KD, int DH, int NW, bool FRAG, bool MASKED = false>
 __global__ __launch_bounds__(64 * NW) void k_segment_state(
     const half_t* __restrict__ k, const half_t* __restrict__ v, const uint8_t* __restrict__ pad_mask,
     int H, float* __restrict__ wsS, float* __restrict__ wsZ, float* __restrict__ row_copy, int T, int N,
@@ -97,7 +97,9 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
     const int n = blockIdx.x / nseg_out, seg = blockIdx.x % nseg_out;
-    const uint8_t* mrow = pad_mask ? pad_mask + (int64_t)(n / H) * T : nullptr;
+    // MASKED is a compile-time switch: a run-time test around the mask loads would be a branch
+    // between the chunk loads, and the compiler drains all outstanding loads at its join
+    const uint8_t* mrow = MASKED ? pad_mask + (int64_t)(n / H) * T : nullptr;
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
@@ -114,22 +116,26 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
     for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
     const h8 ones = h8_ones();
 
-    // The chunks are requested kGroup at a time, each into its own LDS buffer: one memory round
-    // trip per group instead of one per chunk (the products of a chunk take far less time than
-    // its load), one barrier per chunk and one more where the buffers are reused.
+    // Rolling prefetch kGroup chunks deep: chunk u lives in registers rk[u % kGroup] until it is
+    // written to LDS buffer u % kGroup, and the load of chunk u + kGroup is issued right after
+    // that write.  Between the products on buffer b for chunk u and its next write (chunk
+    // u + kGroup) lie the barriers of the chunks in between, so one barrier per chunk suffices.
+    // All loads are branch-free: a chunk past the end re-reads the last valid row and is never
+    // used (a branch between loads makes the compiler drain the outstanding ones at its join).
     constexpr int kGroup = Cfg::kSegStateGroup;
+    RFA_TICK_INIT();
     ChunkRegs<KD, NT> rk[kGroup];
     ChunkRegs<DH, NT> rv[kGroup];
-    for (int tg = t_begin; tg < t_end; tg += kGroup * C) {
+    auto load_chunk = [&](int c, int t0_want) {
+        const int t0 = min(t0_want, t_end - 1);
+        chunk_g2r<KD, NT>(rk[c], kb + (int64_t)t0 * k_stride, k_stride, t_end - t0, tid);
+        chunk_g2r<DH, NT>(rv[c], vb + (int64_t)t0 * v_stride, v_stride, t_end - t0, tid);
+        if (MASKED) chunk_mask_rows<KD, NT>(rk[c], mrow + t0, tid);
+    };
 #pragma unroll
-        for (int c = 0; c < kGroup; ++c) {
-            // branch-free: a chunk past the end re-reads the last valid row and is never used
-            const int t0 = min(tg + c * C, t_end - 1);
-            chunk_g2r<KD, NT>(rk[c], kb + (int64_t)t0 * k_stride, k_stride, t_end - t0, tid);
-            chunk_g2r<DH, NT>(rv[c], vb + (int64_t)t0 * v_stride, v_stride, t_end - t0, tid);
-            if (mrow) chunk_mask_rows<KD, NT>(rk[c], mrow + t0, tid);
-        }
-        if (tg > t_begin) __syncthreads();   // every wave is done with the previous group's buffers
+    for (int c = 0; c < kGroup; ++c) load_chunk(c, t_begin + c * C);
+    RFA_TICK(20);
+    for (int tg = t_begin; tg < t_end; tg += kGroup * C) {
 #pragma unroll
         for (int c = 0; c < kGroup; ++c) {
             const int t0 = tg + c * C;
@@ -138,7 +144,11 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
             half_t* Vc = Kc + C * LDQ;
             chunk_r2s<KD, NT>(rk[c], Kc, LDQ, tid);
             chunk_r2s<DH, NT>(rv[c], Vc, LDV, tid);
+            RFA_TICK(21);
             __syncthreads();
+            RFA_TICK(22);
+            load_chunk(c, t0 + kGroup * C);
+            RFA_TICK(24);
             h8 bv[NCT][2];
 #pragma unroll
             for (int ct = 0; ct < NCT; ++ct)
@@ -157,6 +167,7 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
 #pragma unroll
                 for (int js = 0; js < 2; ++js)
                     zacc[a] = mfma32(col8(Kc, LDQ, js * 32, 16 * (w * NKTW + a), lane), ones, zacc[a]);
+            RFA_TICK(23);
         }
     }
     float* so = wsS + ((int64_t)(n * nseg + seg) * KD) * DH;
@@ -182,6 +193,7 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
         for (int a = 0; a < NKTW; ++a)
             *reinterpret_cast<f4*>(wsZ + (int64_t)(n * nseg + seg) * KD + 16 * (w * NKTW + a) + 4 * G) = zacc[a];
     }
+    RFA_TICK(25);
 }
 
 // ---------------------------------------------------------------------------
