@@ -28,11 +28,11 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the bench configuration, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
 # passes summarised in profiles/bench_cfg2_hbm_traffic.md (counters scaled on the 512 MiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "k_segment_state": 31659830,
-    "k_causal_fwd": 63250398,
-    "k_causal_bwd_dq": 87473517,
-    "k_causal_bwd_dkdv": 89545014,
-    "k_decode_step": 68884939,
+    "k_segment_state": 25427685,
+    "k_causal_fwd": 63782891,
+    "k_causal_bwd_dq": 95829740,
+    "k_causal_bwd_dkdv": 89476682,
+    "k_decode_step": 68884948,
 }
 
 
@@ -165,11 +165,12 @@ def main():
     result = {
         "metric": "causal fwd+bwd tok/s @L=1024 fp16", "value": round(value, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16 in, fp32 accumulate",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16",
         "data": "synthetic",
         "config": {"workload": "configs[1]: RFA causal self-attention fwd+bwd, seq 1024, batch 8, 8 heads, "
                                "head_dim 64, proj_dim 64 (phi width 128), feature-level boundary RFA.apply",
-                   "T": T, "B": B, "H": H, "head_dim": d, "proj_dim": D, "segments": nseg},
+                   "T": T, "B": B, "H": H, "head_dim": d, "proj_dim": D, "segments": nseg,
+                   "arithmetic": "fp16 operands and outputs, fp32 accumulation and state"},
         "parity": parity, "roofline": roofline, "cpu_baseline": cpu_baseline,
     }
 
