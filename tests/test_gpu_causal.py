@@ -55,6 +55,9 @@ SHAPES = [
     (192, 1, 2, 64, 32),     # K = 64
     (160, 1, 2, 128, 64),    # d = 128
     (130, 1, 1, 64, 128),    # K = 256
+    (70, 65, 8, 64, 64),     # many sequences (N = 520), two chunks each
+    (3000, 1, 2, 64, 64),    # long ragged sequence: 16 segments, last one short
+    (1100, 1, 2, 128, 128),  # K = 256, d = 128: split dQ sweep, dK / dV in separate workgroups
 ]
 
 
