@@ -249,6 +249,47 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream):
                    "tgt_tokens_per_s": round(B * Tt / (ms * 1e-3), 1), "us_per_step": round(1e3 * ms, 2),
                    "algorithmic_tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
 
+    # ---- long-context causal fwd+bwd (config 5): seq 16384, batch 2, 16 heads, head_dim 128, proj_dim 128
+    T5, B5, H5, d5, D5 = 16384, 2, 16, 128, 128
+    N5, K5 = B5 * H5, 2 * D5
+    W5 = O.make_w(d5, D5, H5).half().to(dev)
+    g5 = torch.Generator(device="cpu").manual_seed(1234 + 5)
+    mk = lambda last: torch.randn(T5, B5, H5, last, generator=g5)
+    pq5 = rfa_hip.feature_map_forward(unit(mk(d5)).half().to(dev), W5, O.SCALE).view(T5, N5, K5)
+    pk5 = rfa_hip.feature_map_forward(unit(mk(d5)).half().to(dev), W5, O.SCALE).view(T5, N5, K5)
+    v5 = mk(d5).half().to(dev).view(T5, N5, d5)
+    go5 = mk(d5).half().to(dev).view(T5, N5, d5)
+
+    o5 = torch.empty_like(v5)
+    dq5, dk5, dv5 = torch.empty_like(pq5), torch.empty_like(pk5), torch.empty_like(v5)
+    fb5 = lib.rfa_causal_forward_workspace_bytes(T5, N5, K5, d5)
+    bb5 = lib.rfa_causal_backward_workspace_bytes(T5, N5, K5, d5)
+    sb5 = lib.rfa_causal_saved_state_bytes(T5, N5, K5, d5)
+    ws5 = torch.empty(max(fb5, bb5, 1), dtype=torch.uint8, device=dev)
+    sv5 = torch.empty(max(sb5, 1), dtype=torch.uint8, device=dev)
+
+    def long_step():
+        _lib.check(lib.rfa_causal_forward_save(p(pq5), p(pk5), p(v5), p(o5), p(sv5), sb5, T5, N5, K5, d5,
+                                               p(ws5), fb5, stream))
+        _lib.check(lib.rfa_causal_backward_saved(p(pq5), p(pk5), p(v5), p(go5), p(o5), p(sv5), sb5, p(dq5), p(dk5),
+                                                 p(dv5), T5, N5, K5, d5, p(ws5), bb5, stream))
+    for _ in range(2):
+        long_step()
+    ms = _event_time_ms(torch, long_step, 5)
+    ns = 2                                                  # parity on two sequences (chunked-exact oracle)
+    sl = lambda t: t[:, :ns].float().cpu()
+    ref5 = O.causal_forward_chunked(sl(pq5), sl(pk5), sl(v5))
+    rq5, rk5, rv5 = O.causal_backward_chunked(sl(pq5), sl(pk5), sl(v5), sl(go5))
+    rel = lambda a, b: ((a - b).norm() / b.norm()).item()
+    bytes5 = (2 * K5 * 2 + 2 * d5 * 2 + 2 * K5 * 2 + 2 * d5 * 2 + 2 * K5 * 2 + d5 * 2) * N5 * T5   # 4352 B per (head, token)
+    ex["long_context"] = {"workload": "configs[4]: seq 16384, batch 2, 16 heads, head_dim 128, proj_dim 128 (phi width 256), "
+                                      "causal fwd+bwd (saved pair)",
+                          "tokens_per_s": round(B5 * T5 / (ms * 1e-3), 1), "ms_per_step": round(ms, 4),
+                          "algorithmic_bytes": bytes5, "frac_of_hbm": round(bytes5 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                          "parity": {"out_max_abs": (sl(o5) - ref5).abs().max().item(), "dq_rel": rel(sl(dq5), rq5),
+                                     "dk_rel": rel(sl(dk5), rk5), "dv_rel": rel(sl(dv5), rv5)}}
+    del pq5, pk5, v5, go5, o5, dq5, dk5, dv5, ws5, sv5
+
     # ---- feature map (config 2 shape): phi forward + backward for q
     T, B, H = 1024, 8, 8
     x = torch.randn(T, B, H, d, generator=g).half().to(dev)

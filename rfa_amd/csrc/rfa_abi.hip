@@ -142,10 +142,8 @@ constexpr int causal_waves(int KD, int DH) { return (DH >= 128 && KD >= 128) ? 8
 constexpr int dq_waves(int KD, int DH) { return KD >= 128 ? 8 : 4; }
 
 // waves that own the forward state (value-column slices): 4 in the two-stage pipelined forward
-constexpr int fwd_state_waves(int KD, int DH) {
-    return ((size_t)2 * ((size_t)(2 * 64 * (KD + rfa::lds_pad(KD)) + 64 * (DH + rfa::lds_pad(DH)) + 64 * (64 + 8)) * 2 + 64 * 4) + KD * 4
-            <= 160 * 1024) ? 4 : causal_waves(KD, DH);
-}
+template <int KD, int DH>
+constexpr int fwd_state_waves_v = (rfa::FwdPipeCfg<KD, DH>::kLds <= 160 * 1024) ? 4 : causal_waves(KD, DH);
 
 template <typename Kern>
 int set_lds(Kern kern, size_t bytes) {
@@ -161,7 +159,7 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
     // the two-stage pipelined forward needs both chunk buffers in LDS: K <= 128
     constexpr bool PIPE = rfa::FwdPipeCfg<KD, DH>::kLds <= 160 * 1024;
     constexpr int NW = PIPE ? 4 : causal_waves(KD, DH);
-    static_assert(NW == fwd_state_waves(KD, DH), "fragment layout of the segment totals");
+    static_assert(NW == fwd_state_waves_v<KD, DH>, "fragment layout of the segment totals");
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     // with a saved buffer the segment totals are written there directly (S in the forward's
     // fragment order, which the saved-pair backward reads as is)
@@ -221,14 +219,14 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
             constexpr int KL = KD / 2;
             constexpr int NWQ = dq_waves(KL, DH);
             using CfgQ = rfa::CausalCfg<KL, DH, NWQ>;
-            auto kern = rfa::k_causal_bwd_dq_saved<KL, DH, NWQ, fwd_state_waves(KD, DH), KD>;
+            auto kern = rfa::k_causal_bwd_dq_saved<KL, DH, NWQ, fwd_state_waves_v<KD, DH>, KD>;
             if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
             RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(2 * N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g,
                        out, savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len);
         } else {
             constexpr int NWQ = dq_waves(KD, DH);
             using CfgQ = rfa::CausalCfg<KD, DH, NWQ>;
-            auto kern = rfa::k_causal_bwd_dq_saved<KD, DH, NWQ, fwd_state_waves(KD, DH)>;
+            auto kern = rfa::k_causal_bwd_dq_saved<KD, DH, NWQ, fwd_state_waves_v<KD, DH>>;
             if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
             RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g, out,
                        savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len);
