@@ -158,6 +158,31 @@ int rfa_cross_state_backward(const void* phi_k, const void* v, const uint8_t* ke
                              int64_t B, int H, int K, int d, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Quadratic form with explicit masks: masked_rfa(phi_q, phi_k, v, key_padding_mask,
+ * attn_mask) (random_feature_attention/causal_attention.py:57-109), the path
+ * CausalAttention takes with cuda_causal_rfa = False, and its gradient (autograd of
+ * the same lines).  Weights a[t][s] = phi_q[t] . phi_k[s], zero where key s is padded
+ * or attn_mask[t][s] is set, divided by max(|row sum|, 1e-3) (utils.py:123-130),
+ * applied to v.
+ *   phi_q, phi_k : fp16 [T, N, K]  (N = B * H, time-major);  v, out, grad_attn : fp16 [T, N, d]
+ *   key_padding_mask : bytes [B, T], non-zero = padded key, may be NULL
+ *   attn_mask        : bytes [T, Tp], non-zero = masked (the reference's `attn_mask < 0`),
+ *                      Tp = T rounded up to a multiple of 64, padding columns non-zero; may be NULL
+ *   attn_mask_t      : its transpose, bytes [T (key), Tp (query)], padded the same way
+ *   rsum             : fp32 [T, N] raw row sums (forward: optional output; backward: input)
+ *   dphi_q, dphi_k, dv : every element written; a padded key gets zero dphi_k and dv.
+ * ------------------------------------------------------------------------- */
+int rfa_masked_forward(const void* phi_q, const void* phi_k, const void* v, const uint8_t* key_padding_mask,
+                       const uint8_t* attn_mask, void* out, float* rsum, int64_t T, int64_t Tp, int64_t B,
+                       int H, int K, int d, void* stream);
+size_t rfa_masked_backward_workspace_bytes(int64_t T, int64_t N, int d);
+int rfa_masked_backward(const void* phi_q, const void* phi_k, const void* v, const void* grad_attn,
+                        const void* out, const float* rsum, const uint8_t* key_padding_mask,
+                        const uint8_t* attn_mask, const uint8_t* attn_mask_t, void* dphi_q, void* dphi_k,
+                        void* dv, int64_t T, int64_t Tp, int64_t B, int H, int K, int d, void* workspace,
+                        size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Incremental decoding.  The fp32 state (s [N, K, d], z [N, K]) is updated IN
  * PLACE; one kernel is launched per step, in order, on `stream`.
  *

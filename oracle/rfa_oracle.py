@@ -13,7 +13,7 @@ gates uses float32).
 Pinning status (see tests/test_oracle_*.py): every function below is pinned by
 checks that do not retype its formula -- mutual agreement of independent
 forms (cumulative-sum, per-step loop, chunked, quadratic brute force),
-closed-form known answers, ``torch.autograd`` / ``gradcheck`` for the
+closed-form known answers (element-by-element loops for the masked quadratic form), ``torch.autograd`` / ``gradcheck`` for the
 backward formulas, library ``matmul`` for the contractions, and the
 softmax-kernel Monte-Carlo identity for the feature map.  The reference ships
 no golden vectors for this path, so none are checked.
@@ -109,6 +109,24 @@ def causal_forward_quadratic(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
     num = torch.einsum("nts,snd->tnd", a, v)
     den = a.sum(-1).transpose(0, 1).clamp_min(EPS)
     return num / den.unsqueeze(-1)
+
+
+def masked_rfa(phi_q: Tensor, phi_k: Tensor, v: Tensor, key_padding_mask: Optional[Tensor] = None,
+               attn_mask: Optional[Tensor] = None) -> Tensor:
+    """Quadratic form with explicit masks (causal_attention.py:57-109, utils.py:123-130).
+
+    phi_q, phi_k: [T, B, H, K]; v: [T, B, H, d]; key_padding_mask: [B, T], non-zero = padded key;
+    attn_mask: [T, T], entries < 0 are masked.  Weights are zeroed where masked, then divided by
+    |row sum|.clamp(1e-3); returns [T, B, H, d].  (The reference casts the normalised weights back
+    to the input dtype before applying them to v; here everything stays in the given dtype.)
+    """
+    w = torch.einsum("tbhk,sbhk->bhts", phi_q, phi_k)
+    if key_padding_mask is not None:
+        w = w.masked_fill(key_padding_mask.to(torch.bool)[:, None, None, :], 0.0)
+    if attn_mask is not None:
+        w = w.masked_fill((attn_mask < 0.0)[None, None], 0.0)
+    w = w / w.sum(-1, keepdim=True).abs().clamp(1e-3)
+    return torch.einsum("bhts,sbhd->tbhd", w, v)
 
 
 def causal_forward_chunked(q: Tensor, k: Tensor, v: Tensor, chunk: int = 64) -> Tensor:

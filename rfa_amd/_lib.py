@@ -51,6 +51,9 @@ SIGNATURES = {
     "rfa_cross_readout": (c_int, [c_void_p] * 4 + [c_int64, c_int64, c_int, c_int, c_void_p]),
     "rfa_cross_readout_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_void_p]),
     "rfa_cross_state_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
+    "rfa_masked_forward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
+    "rfa_masked_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int]),
+    "rfa_masked_backward": (c_int, [c_void_p] * 12 + [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "rfa_incremental": (c_int, [c_void_p] * 6 + [c_int64, c_int64, c_int, c_int, c_void_p]),
     "rfa_profile_enable": (c_int, [c_int]),
     "rfa_profile_collect": (c_int, []),

@@ -3,7 +3,7 @@
 Functional forms (keyword-only, as in the reference):
   incremental_rfa   decode loop                       -> HIP step kernel, fp32 state
   cuda_causal_rfa   training / prefill                -> HIP chunked-scan kernels via RFA.apply
-  masked_rfa        quadratic form with explicit masks -> ATen ops, as in the reference
+  masked_rfa        quadratic form with explicit masks -> HIP quadratic-form kernels
 and the ``CausalAttention`` module with the reference's parameter names
 (q_proj, k_proj, v_proj, out_proj, sigma) and ``saved_state`` keys
 ("prev_s", "prev_z").
@@ -19,7 +19,7 @@ from torch.nn import Parameter
 
 from . import rfa_hip
 from .rfa import RFA
-from .utils import (EPS, SCALE, build_random_matrices, normalize_attn_weights, random_project,
+from .utils import (EPS, SCALE, build_random_matrices, random_project,
                     upgrade_state_dict_named)
 
 
@@ -61,24 +61,52 @@ def incremental_rfa(*, phi_q: Tensor, phi_k: Tensor, v: Tensor, s: Optional[Tens
     return attn.to(v.dtype).view(tgt_len, bsz, num_heads * head_dim), s, z
 
 
+class _MaskedRFA(torch.autograd.Function):
+    """masked_rfa on the quadratic-form kernels (rfa_masked_forward / rfa_masked_backward)."""
+
+    @staticmethod
+    def forward(ctx, phi_q, phi_k, v, heads, key_padding_mask, mask_bytes, mask_t_bytes):
+        ctx.in_dtypes = (phi_q.dtype, phi_k.dtype, v.dtype)
+        q16, k16, v16 = (t.to(torch.float16).contiguous() for t in (phi_q, phi_k, v))
+        attn, rsum = rfa_hip.masked_forward(q16, k16, v16, heads, key_padding_mask, mask_bytes)
+        ctx.heads = heads
+        ctx.masks = (key_padding_mask, mask_bytes, mask_t_bytes)
+        ctx.save_for_backward(q16, k16, v16, attn, rsum)
+        return attn.to(v.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_attn):
+        q16, k16, v16, attn, rsum = ctx.saved_tensors
+        pad, mb, mtb = ctx.masks
+        dq, dk, dv = rfa_hip.masked_backward(q16, k16, v16, grad_attn.to(torch.float16).contiguous(), attn, rsum,
+                                             ctx.heads, pad, mb, mtb)
+        tq, tk, tv = ctx.in_dtypes
+        return dq.to(tq), dk.to(tk), dv.to(tv), None, None, None, None
+
+
 def masked_rfa(*, phi_q: Tensor, phi_k: Tensor, v: Tensor, key_padding_mask: Optional[Tensor] = None,
                attn_mask: Optional[Tensor] = None) -> Tensor:
     """Quadratic-form RFA with explicit masks (reference causal_attention.py:57-109).
 
-    Note its normaliser, |row sum|.clamp(1e-3) in fp32 (utils.py:123-130), is not the
-    clamp-at-1 of the scan path.  Runs as ATen ops on the tensors' device.
+    phi_q, phi_k: [tgt_len, bsz, heads, 2*proj_dim]; v: [tgt_len, bsz, heads, head_dim];
+    key_padding_mask: [bsz, tgt_len], 1 = padded key (a 0-dim tensor stands for None);
+    attn_mask: [tgt_len, tgt_len], entries < 0 are masked (typically the causal mask).
+    Note its normaliser, |row sum|.clamp(1e-3) (utils.py:123-130), is not the clamp-at-1 of
+    the scan path.  Runs on the quadratic-form HIP kernels; tensors must be on a HIP device.
     """
-    tgt_len, bsz, num_heads, _ = phi_q.size()
+    tgt_len, bsz, num_heads, feat = phi_q.size()
     head_dim = v.size(-1)
     key_padding_mask = _drop_scalar_mask(key_padding_mask)
-    weights = torch.einsum("tbhk,sbhk->bhts", phi_q, phi_k)
     if key_padding_mask is not None:
         assert key_padding_mask.size(0) == bsz and key_padding_mask.size(1) == tgt_len
-        weights = weights.masked_fill(key_padding_mask.to(torch.bool)[:, None, None, :], 0.0)
+    mask_bytes = mask_t_bytes = None
     if attn_mask is not None:
-        weights = weights.masked_fill((attn_mask < 0.0)[None, None], 0.0)
-    weights = normalize_attn_weights(weights, dtype=weights.dtype)
-    attn = torch.einsum("bhts,sbhd->tbhd", weights, v)
+        assert attn_mask.size(0) == tgt_len and attn_mask.size(1) == tgt_len
+        mask_bytes, mask_t_bytes = rfa_hip.pack_attn_mask((attn_mask < 0.0).to(phi_q.device))
+    n = bsz * num_heads
+    attn = _MaskedRFA.apply(phi_q.contiguous().view(tgt_len, n, feat), phi_k.contiguous().view(tgt_len, n, feat),
+                            v.contiguous().view(tgt_len, n, head_dim), num_heads, key_padding_mask, mask_bytes,
+                            mask_t_bytes)
     return attn.contiguous().view(tgt_len, bsz, num_heads * head_dim)
 
 

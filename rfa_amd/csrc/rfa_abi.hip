@@ -15,6 +15,7 @@
 #include "rfa_causal.h"
 #include "rfa_decode.h"
 #include "rfa_featuremap.h"
+#include "rfa_masked.h"
 
 namespace {
 
@@ -39,10 +40,12 @@ int fail(int code, const char* fmt, ...) {
 // ---- optional per-kernel timing with HIP events ------------------------------------
 namespace prof {
 enum Id { SEG_STATE, CAUSAL_FWD, CAUSAL_BWD_DQ, CAUSAL_BWD_DKDV, CROSS_READOUT, CROSS_READOUT_BWD,
-          CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, ZERO_FILL, SELFTEST, COUNT };
+          CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, MASKED_FWD, MASKED_PREP, MASKED_DQ, MASKED_DKDV, ZERO_FILL,
+          SELFTEST, COUNT };
 const char* const kNames[COUNT] = {"k_segment_state", "k_causal_fwd", "k_causal_bwd_dq", "k_causal_bwd_dkdv",
                                    "k_cross_readout", "k_cross_readout_bwd", "k_cross_state_bwd", "k_decode_step",
                                    "k_feature_map_fwd", "k_feature_map_bwd", "k_feature_map_dw_reduce",
+                                   "k_masked_fwd", "k_masked_bwd_prep", "k_masked_dq", "k_masked_dkdv",
                                    "k_zero_f32", "k_selftest"};
 struct Rec { int id; hipEvent_t a, b; };
 std::mutex mu;
@@ -347,6 +350,44 @@ int launch_cross_state_bwd(const rfa::half_t* k, const rfa::half_t* v, const uin
     RFA_LAUNCH(CROSS_STATE_BWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDkLds, st,
                        (const rfa::half_t*)nullptr, k, v, (const rfa::half_t*)nullptr, dk, dv, ds, dz,
                        (const float*)nullptr, (const float*)nullptr, mask, H, T, N, p.nseg, p.seg_len);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+
+// ---- quadratic form with explicit masks ---------------------------------------------------
+template <int KD, int DH>
+int launch_masked_fwd(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, const uint8_t* pad,
+                      const uint8_t* amask, rfa::half_t* out, float* rsum, int T, int Tp, int N, int H,
+                      hipStream_t st) {
+    using Cfg = rfa::MaskedCfg<KD, DH>;
+    auto kern = rfa::k_masked_fwd<KD, DH>;
+    if (int rc = set_lds(kern, Cfg::kLds)) return rc;
+    const int nblk = (T + rfa::kChunk - 1) / rfa::kChunk;
+    RFA_LAUNCH(MASKED_FWD, kern, dim3(N * nblk), dim3(256), Cfg::kLds, st, q, k, v, pad, amask, out, rsum, T, Tp, N, H);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+template <int KD, int DH>
+int launch_masked_bwd(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, const rfa::half_t* g,
+                      const rfa::half_t* out, const float* rsum, const uint8_t* pad, const uint8_t* amask,
+                      const uint8_t* amask_t, rfa::half_t* dq, rfa::half_t* dk, rfa::half_t* dv,
+                      rfa::half_t* ghat, float* gz, int T, int Tp, int N, int H, hipStream_t st) {
+    using Cfg = rfa::MaskedCfg<KD, DH>;
+    const int nblk = (T + rfa::kChunk - 1) / rfa::kChunk;
+    const int64_t rows = (int64_t)T * N;
+    const int64_t pieces = rows * (DH / 8);
+    RFA_LAUNCH(MASKED_PREP, rfa::k_masked_bwd_prep<DH>, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, g, out,
+               rsum, ghat, gz, rows);
+    auto kq = rfa::k_masked_dq<KD, DH>;
+    if (int rc = set_lds(kq, Cfg::kLds)) return rc;
+    RFA_LAUNCH(MASKED_DQ, kq, dim3(N * nblk), dim3(256), Cfg::kLds, st, (const rfa::half_t*)ghat, (const float*)gz, k,
+               v, pad, amask, dq, T, Tp, N, H);
+    auto kk = rfa::k_masked_dkdv<KD, DH>;
+    if (int rc = set_lds(kk, Cfg::kLds)) return rc;
+    RFA_LAUNCH(MASKED_DKDV, kk, dim3(N * nblk), dim3(256), Cfg::kLds, st, q, k, v, (const rfa::half_t*)ghat,
+               (const float*)gz, pad, amask_t, dk, dv, T, Tp, N, H);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -762,6 +803,76 @@ int rfa_cross_state_backward(const void* phi_k, const void* v, const uint8_t* ke
     auto* dkh = static_cast<rfa::half_t*>(dphi_k);
     auto* dvh = static_cast<rfa::half_t*>(dv);
 #define RFA_CALL(KD, DH) launch_cross_state_bwd<KD, DH>(kh, vh, key_padding_mask, H, ds, dz, dkh, dvh, (int)S_len, (int)N, st)
+    RFA_DISPATCH_KD(K, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+
+// ---- quadratic form with explicit masks ---------------------------------------------------
+static int check_masked(const char* fn, int64_t T, int64_t Tp, int64_t B, int H, int K, int d, const void* amask) {
+    if (int rc = check_cross_dims(fn, T, B, H, K, d)) return rc;
+    if (amask && (Tp < T || Tp % 64 != 0))
+        return fail(RFA_ERR_BAD_SHAPE, "%s: the attn_mask row stride must be T rounded up to a multiple of 64 (got %lld for T=%lld)",
+                    fn, (long long)Tp, (long long)T);
+    return RFA_OK;
+}
+
+int rfa_masked_forward(const void* phi_q, const void* phi_k, const void* v, const uint8_t* key_padding_mask,
+                       const uint8_t* attn_mask, void* out, float* rsum, int64_t T, int64_t Tp, int64_t B, int H,
+                       int K, int d, void* stream) {
+    if (int rc = check_masked("rfa_masked_forward", T, Tp, B, H, K, d, attn_mask)) return rc;
+    const int64_t N = B * H;
+    if (T == 0 || N == 0) return RFA_OK;
+    if (!phi_q || !phi_k || !v || !out) return fail(RFA_ERR_NULL_POINTER, "rfa_masked_forward: NULL tensor pointer");
+    if (!aligned16(phi_q) || !aligned16(phi_k) || !aligned16(v) || !aligned16(out) || (attn_mask && !aligned16(attn_mask)))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_masked_forward: tensors must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* qh = static_cast<const rfa::half_t*>(phi_q);
+    auto* kh = static_cast<const rfa::half_t*>(phi_k);
+    auto* vh = static_cast<const rfa::half_t*>(v);
+    auto* oh = static_cast<rfa::half_t*>(out);
+#define RFA_CALL(KD, DH) launch_masked_fwd<KD, DH>(qh, kh, vh, key_padding_mask, attn_mask, oh, rsum, (int)T, (int)Tp, (int)N, H, st)
+    RFA_DISPATCH_KD(K, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+size_t rfa_masked_backward_workspace_bytes(int64_t T, int64_t N, int d) {
+    if (T <= 0 || N <= 0 || d <= 0) return 0;
+    return align_up((size_t)T * N * d * 2) + align_up((size_t)T * N * 4);
+}
+
+int rfa_masked_backward(const void* phi_q, const void* phi_k, const void* v, const void* grad_attn, const void* out,
+                        const float* rsum, const uint8_t* key_padding_mask, const uint8_t* attn_mask,
+                        const uint8_t* attn_mask_t, void* dphi_q, void* dphi_k, void* dv, int64_t T, int64_t Tp,
+                        int64_t B, int H, int K, int d, void* workspace, size_t workspace_bytes, void* stream) {
+    if (int rc = check_masked("rfa_masked_backward", T, Tp, B, H, K, d, attn_mask)) return rc;
+    const int64_t N = B * H;
+    if (T == 0 || N == 0) return RFA_OK;
+    if (!phi_q || !phi_k || !v || !grad_attn || !out || !rsum || !dphi_q || !dphi_k || !dv)
+        return fail(RFA_ERR_NULL_POINTER, "rfa_masked_backward: NULL tensor pointer");
+    if ((attn_mask == nullptr) != (attn_mask_t == nullptr))
+        return fail(RFA_ERR_NULL_POINTER, "rfa_masked_backward: attn_mask and its transpose must be given together");
+    if (!aligned16(phi_q) || !aligned16(phi_k) || !aligned16(v) || !aligned16(grad_attn) || !aligned16(out) ||
+        !aligned16(dphi_q) || !aligned16(dphi_k) || !aligned16(dv) || (attn_mask && (!aligned16(attn_mask) || !aligned16(attn_mask_t))))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_masked_backward: tensors must be 16-byte aligned");
+    const size_t need = rfa_masked_backward_workspace_bytes(T, N, d);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+        return fail(RFA_ERR_WORKSPACE, "rfa_masked_backward: workspace of %zu bytes required, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* qh = static_cast<const rfa::half_t*>(phi_q);
+    auto* kh = static_cast<const rfa::half_t*>(phi_k);
+    auto* vh = static_cast<const rfa::half_t*>(v);
+    auto* gh = static_cast<const rfa::half_t*>(grad_attn);
+    auto* oh = static_cast<const rfa::half_t*>(out);
+    auto* dqh = static_cast<rfa::half_t*>(dphi_q);
+    auto* dkh = static_cast<rfa::half_t*>(dphi_k);
+    auto* dvh = static_cast<rfa::half_t*>(dv);
+    auto* ghat = static_cast<rfa::half_t*>(workspace);
+    float* gz = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up((size_t)T * N * d * 2));
+#define RFA_CALL(KD, DH) launch_masked_bwd<KD, DH>(qh, kh, vh, gh, oh, rsum, key_padding_mask, attn_mask, attn_mask_t, dqh, dkh, dvh, ghat, gz, (int)T, (int)Tp, (int)N, H, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");

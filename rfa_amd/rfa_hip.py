@@ -326,3 +326,70 @@ def incremental_fused(q: Tensor, k: Tensor, v: Tensor, w: Tensor, scale: float, 
             q.data_ptr(), k.data_ptr(), v.data_ptr(), w.data_ptr(), float(scale), s.data_ptr(), z.data_ptr(),
             out.data_ptr(), steps, B, H, D, d, _stream_ptr(v.device)))
     return out
+
+
+# ---------------------------------------------------------------------------
+# quadratic form with explicit masks (masked_rfa)
+# ---------------------------------------------------------------------------
+def pack_attn_mask(masked: Tensor):
+    """bool [T, S] (True = masked) -> (bytes [T, Sp], bytes of the transpose [S, Tp]), rows padded
+    to a multiple of 64 with ones, as rfa_masked_forward / rfa_masked_backward read them."""
+    _require(masked.dim() == 2 and masked.shape[0] == masked.shape[1], ValueError,
+             f"attn_mask must be [tgt_len, tgt_len] (got {tuple(masked.shape)})")
+    T = masked.shape[0]
+    Tp = (T + 63) // 64 * 64
+    m = torch.ones((T, Tp), dtype=torch.uint8, device=masked.device)
+    m[:, :T] = masked.to(torch.uint8)
+    mt = torch.ones((T, Tp), dtype=torch.uint8, device=masked.device)
+    mt[:, :T] = masked.t().to(torch.uint8)
+    return m, mt
+
+
+def masked_forward(phi_q: Tensor, phi_k: Tensor, v: Tensor, H: int, key_padding_mask=None, attn_mask_bytes=None):
+    """(attn [T, N, d], rsum fp32 [T, N]).  phi_q, phi_k fp16 [T, N, K], v fp16 [T, N, d], N = B * H;
+    key_padding_mask [B, T] (non-zero = pad) or None; attn_mask_bytes from pack_attn_mask()[0] or None."""
+    _check_qkv(phi_q, phi_k, v)
+    T, N, K = phi_q.shape
+    d = v.shape[2]
+    _require(N % H == 0, ValueError, f"N={N} is not a multiple of heads={H}")
+    B = N // H
+    Tp = (T + 63) // 64 * 64
+    out = torch.empty_like(v)
+    rsum = torch.empty((T, N), dtype=torch.float32, device=v.device)
+    keep, mptr = _mask_arg(key_padding_mask, B, T, v.device)
+    if attn_mask_bytes is not None:
+        _require(attn_mask_bytes.is_cuda and attn_mask_bytes.dtype == torch.uint8 and attn_mask_bytes.is_contiguous()
+                 and tuple(attn_mask_bytes.shape) == (T, Tp), ValueError, "attn_mask_bytes must come from pack_attn_mask")
+    with torch.cuda.device(v.device):
+        _lib.check(_lib.load().rfa_masked_forward(
+            phi_q.data_ptr(), phi_k.data_ptr(), v.data_ptr(), mptr,
+            attn_mask_bytes.data_ptr() if attn_mask_bytes is not None else None, out.data_ptr(), rsum.data_ptr(),
+            T, Tp, B, H, K, d, _stream_ptr(v.device)))
+    return out, rsum
+
+
+def masked_backward(phi_q: Tensor, phi_k: Tensor, v: Tensor, grad_attn: Tensor, out: Tensor, rsum: Tensor, H: int,
+                    key_padding_mask=None, attn_mask_bytes=None, attn_mask_t_bytes=None) -> List[Tensor]:
+    """[dphi_q, dphi_k, dv] of masked_forward."""
+    _check_qkv(phi_q, phi_k, v)
+    _check_half_cuda("grad_attn", grad_attn, 3)
+    _check_half_cuda("out", out, 3)
+    T, N, K = phi_q.shape
+    d = v.shape[2]
+    B = N // H
+    Tp = (T + 63) // 64 * 64
+    _require(grad_attn.shape == v.shape and out.shape == v.shape, ValueError, "grad_attn and out must match v")
+    _check_f32_cuda("rsum", rsum, (T, N))
+    dq, dk, dv = torch.empty_like(phi_q), torch.empty_like(phi_k), torch.empty_like(v)
+    keep, mptr = _mask_arg(key_padding_mask, B, T, v.device)
+    lib = _lib.load()
+    with torch.cuda.device(v.device):
+        nbytes = lib.rfa_masked_backward_workspace_bytes(T, N, d)
+        ws = _workspace(nbytes, v.device)
+        _lib.check(lib.rfa_masked_backward(
+            phi_q.data_ptr(), phi_k.data_ptr(), v.data_ptr(), grad_attn.data_ptr(), out.data_ptr(), rsum.data_ptr(),
+            mptr, attn_mask_bytes.data_ptr() if attn_mask_bytes is not None else None,
+            attn_mask_t_bytes.data_ptr() if attn_mask_t_bytes is not None else None,
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), T, Tp, B, H, K, d, ws.data_ptr(), nbytes,
+            _stream_ptr(v.device)))
+    return [dq, dk, dv]

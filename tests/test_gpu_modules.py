@@ -213,3 +213,79 @@ def test_module_prefill_then_decode_and_beam_reorder():
     for k_ in ("prev_s", "prev_z"):
         assert torch.equal(state[k_], before[k_][order.cuda()])
     assert reorder_incremental_state({}, order) == {}
+
+
+def _masked_case(T, B, H, d, D, seed, with_pad, mask_kind):
+    q, k, v, g = O.make_qkv(T, B, H, d, seed)
+    W = O.make_w(d, D, H)
+    pq = O.random_project(q.float(), W).half()
+    pk = O.random_project(k.float(), W).half()
+    pad = None
+    if with_pad:
+        pad = torch.zeros(B, T, dtype=torch.uint8)
+        pad[0, max(T - 5, 1):] = 1
+        if B > 1:
+            pad[1, :2] = 1
+    if mask_kind == "causal":
+        am = torch.triu(torch.full((T, T), float("-inf")), 1)
+    elif mask_kind == "band":       # an arbitrary pattern: causal band of width 40 plus a few holes
+        i = torch.arange(T)
+        am = torch.zeros(T, T)
+        am[(i[None, :] > i[:, None]) | (i[:, None] - i[None, :] >= 40)] = -1.0
+        am[i % 7 == 3, 0] = -1.0
+    else:
+        am = None
+    return pq, pk, v, g, pad, am
+
+
+@pytest.mark.parametrize("T,B,H,d,D,with_pad,mask_kind", [
+    (6, 2, 1, 64, 32, True, "causal"),
+    (64, 1, 2, 64, 64, False, "causal"),
+    (130, 2, 2, 64, 64, True, "causal"),
+    (200, 1, 2, 64, 64, True, "band"),
+    (96, 2, 1, 128, 64, False, None),
+    (70, 1, 1, 128, 128, True, "causal"),
+])
+def test_masked_rfa_matches_oracle_forward_and_backward(T, B, H, d, D, with_pad, mask_kind):
+    """masked_rfa on the quadratic-form kernels against the oracle (causal_attention.py:57-109) and
+    its autograd gradients, with key padding, the causal mask and an arbitrary mask."""
+    from rfa_amd.causal_attention import masked_rfa
+    pq, pk, v, g, pad, am = _masked_case(T, B, H, d, D, 4000 + T, with_pad, mask_kind)
+    print(f"masked_rfa T={T} B={B} H={H} K={2*D} d={d} pad={with_pad} mask={mask_kind}", flush=True)
+    cq, ck, cv = (t.cuda().requires_grad_(True) for t in (pq, pk, v))
+    out = masked_rfa(phi_q=cq, phi_k=ck, v=cv, key_padding_mask=None if pad is None else pad.cuda(),
+                     attn_mask=None if am is None else am.cuda())
+    out.backward(g.reshape(T, B, H * d).cuda())
+    fq, fk, fv = (t.float().requires_grad_(True) for t in (pq, pk, v))
+    ref = O.masked_rfa(fq, fk, fv, pad, am)
+    ref.backward(g.float())
+    assert tuple(out.shape) == (T, B, H * d)
+    # outputs are O(|v|) here (weights sum to 1 in magnitude): the forward gate of the path
+    assert (out.float().cpu().view(T, B, H, d) - ref.detach()).abs().max().item() <= 4e-3
+    for name, got, want in (("dphi_q", cq.grad, fq.grad), ("dphi_k", ck.grad, fk.grad), ("dv", cv.grad, fv.grad)):
+        assert torch.isfinite(got).all(), name
+        assert _rel(got.float().cpu(), want) <= 1e-2, (name, _rel(got.float().cpu(), want))
+    if pad is not None:      # padded keys receive no gradient
+        padded = pad.bool().t()[:, :, None, None].expand_as(ck.grad).cuda()
+        assert ck.grad[padded].abs().max().item() == 0.0
+
+
+def test_causal_attention_module_quadratic_fallback_matches_scan_module():
+    """CausalAttention(cuda_causal_rfa=False) runs masked_rfa; with row sums far below 1 the
+    scan path clamps at 1 while the quadratic form normalises, so compare against the oracle
+    chain rather than the other module."""
+    from rfa_amd.causal_attention import CausalAttention
+    torch.manual_seed(3)
+    T, B, E, H, d, D = 80, 2, 128, 2, 64, 64
+    m = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D, cuda_causal_rfa=False).cuda().half()
+    W = O.make_w(d, D, H).half().cuda()
+    x = (torch.randn(T, B, E) * 0.5).half().cuda()
+    am = torch.triu(torch.full((T, T), float("-inf")), 1).cuda()
+    with torch.no_grad():
+        y = m(x, W, attn_mask=am)
+        f = lambda lin, t: torch.nn.functional.linear(t.float(), lin.weight.float(), lin.bias.float())
+        q, k, v = (f(p_, x).view(T, B, H, d).cpu() for p_ in (m.q_proj, m.k_proj, m.v_proj))
+        w = O.build_random_matrices(W.float().cpu(), m.tau, m.sigma.float().cpu(), True)
+        attn = O.masked_rfa(O.random_project(q, w), O.random_project(k, w), v, None, am.cpu())
+        want = f(m.out_proj, attn.reshape(T, B, E).cuda())
+    assert (y.float() - want).abs().max().item() <= 2e-2

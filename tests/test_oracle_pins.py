@@ -290,3 +290,50 @@ def test_gradcheck_small():
     q, k = (q + 0.7).requires_grad_(True), (k.abs() + 0.5).requires_grad_(True)
     v = v.requires_grad_(True)
     assert torch.autograd.gradcheck(O.causal_forward_chunked, (q, k, v, 2), eps=1e-6, atol=1e-5)
+
+
+def test_masked_rfa_oracle_against_explicit_loops():
+    """The masked quadratic form, element by element: weights over the unmasked, unpadded keys,
+    divided by |their sum| clamped at 1e-3 (sign kept in the numerator), including a row whose
+    weights sum to a negative number and a row whose sum is below the clamp."""
+    g = torch.Generator().manual_seed(1)
+    T, B, H, K, d = 6, 2, 2, 8, 4
+    pq = torch.rand(T, B, H, K, generator=g, dtype=torch.float64) - 0.3
+    pk = torch.rand(T, B, H, K, generator=g, dtype=torch.float64) - 0.3
+    pq[2, 0, 0] = -pq[2, 0, 0].abs()          # a negative row sum
+    pk[:, 0, 0] = pk[:, 0, 0].abs()
+    pq[3, 1, 1] *= 1e-5                        # a row sum below the clamp
+    v = torch.randn(T, B, H, d, generator=g, dtype=torch.float64)
+    causal = torch.triu(torch.full((T, T), float("-inf"), dtype=torch.float64), 1)
+    pad = torch.zeros(B, T, dtype=torch.uint8)
+    pad[1, 4:] = 1
+    out = O.masked_rfa(pq, pk, v, pad, causal)
+    seen_negative = seen_clamped = False
+    for b in range(B):
+        for h in range(H):
+            for t in range(T):
+                keys = [s_ for s_ in range(t + 1) if not pad[b, s_]]
+                wts = torch.stack([(pq[t, b, h] * pk[s_, b, h]).sum() for s_ in keys])
+                rs = wts.sum()
+                seen_negative |= bool(rs < -1e-3)
+                seen_clamped |= bool(rs.abs() < 1e-3)
+                want = (wts[:, None] * torch.stack([v[s_, b, h] for s_ in keys])).sum(0) / max(abs(rs.item()), 1e-3)
+                assert torch.allclose(out[t, b, h], want, atol=1e-12)
+    assert seen_negative and seen_clamped
+    # a 0-dim / absent mask changes nothing; without any mask every key counts
+    full = O.masked_rfa(pq, pk, v)
+    w = torch.einsum("tbhk,sbhk->bhts", pq, pk)
+    assert torch.allclose(full, torch.einsum("bhts,sbhd->tbhd", w / w.sum(-1, keepdim=True).abs().clamp(1e-3), v))
+
+
+def test_masked_rfa_oracle_equals_scan_when_denominators_agree():
+    """With the causal mask and row sums >= 1 the two normalisers coincide:
+    masked quadratic form == causal scan (rfa.py:57-63)."""
+    T, N, K, d = 12, 3, 8, 4
+    g = torch.Generator().manual_seed(5)
+    q = torch.rand(T, N, K, generator=g, dtype=torch.float64) + 0.5
+    k = torch.rand(T, N, K, generator=g, dtype=torch.float64) + 0.5     # q.k > 1 for every pair
+    v = torch.randn(T, N, d, generator=g, dtype=torch.float64)
+    causal = torch.triu(torch.full((T, T), float("-inf"), dtype=torch.float64), 1)
+    a = O.masked_rfa(q.view(T, N, 1, K), k.view(T, N, 1, K), v.view(T, N, 1, d), None, causal).view(T, N, d)
+    assert torch.allclose(a, O.causal_forward_cumsum(q, k, v), atol=1e-12)
