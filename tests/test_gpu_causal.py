@@ -126,3 +126,28 @@ def test_saved_pair_clamped_and_unclamped_rows():
         want = _oracle_bwd(pq, pk2, v, g)
         for name, a, b in zip(("dq", "dk", "dv"), got, want):
             assert _rel(a, b) <= GRAD_RTOL, (scale, name, _rel(a, b))
+
+
+@pytest.mark.parametrize("nseg", [1, 2, 3, 8, 16])
+def test_every_segment_count_gives_the_same_answer(nseg, monkeypatch):
+    """RFA_HIP_NSEG overrides the number of time segments per sequence; the plain pair, the
+    saved pair and the prefill state must meet the oracle for any of them (ragged last segment,
+    single-chunk segments, one segment for the whole sequence)."""
+    from rfa_amd import rfa_hip
+    monkeypatch.setenv("RFA_HIP_NSEG", str(nseg))
+    T, B, H, d, D = 700, 1, 3, 64, 64
+    cpu = _features(T, B, H, d, D, seed=5000)
+    pq, pk, v, g = (t.cuda() for t in cpu)
+    print(f"causal nseg={nseg} T={T}", flush=True)
+    ref = _oracle_fwd(*cpu[:3])
+    want = _oracle_bwd(*cpu)
+    out, saved = rfa_hip.forward_save(pq, pk, v)
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_ATOL
+    assert torch.equal(out, rfa_hip.forward(pq, pk, v))
+    for pair in (rfa_hip.backward_saved(pq, pk, v, g, out, saved), rfa_hip.backward(pq, pk, v, g)):
+        for name, a, b in zip(("dq", "dk", "dv"), pair, want):
+            assert _rel(a.float().cpu(), b) <= GRAD_RTOL, (nseg, name)
+    o2, s, z = rfa_hip.prefill(pq, pk, v)
+    assert torch.equal(o2, out)
+    _, s_ref, z_ref = O.causal_forward_loop(cpu[0].float(), cpu[1].float(), cpu[2].float())
+    assert _rel(s.cpu(), s_ref) < 1e-5 and _rel(z.cpu(), z_ref) < 1e-5
