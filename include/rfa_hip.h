@@ -128,6 +128,43 @@ int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi,
                              size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Linear projections to heads with the feature map in the epilogue.
+ *
+ * rfa_project_feature_map replaces, in one launch, the chain the attention modules run on
+ * their input: q_proj / k_proj / v_proj (torch.nn.Linear), the view to heads and
+ * random_project on the q and k projections
+ *   (random_feature_attention/causal_attention.py:228-247; cross_attention.py:66-76 for the
+ *    k / v projections of the encoder output, :279-283 for the q projection; utils.py:100-120).
+ *   x        : fp16 [R, E]      R = seq_len * bsz rows, E a multiple of 64
+ *   weights  : np pointers (1 <= np <= 3) to fp16 [H*d, E], torch.nn.Linear.weight layout
+ *   biases   : np pointers to fp16 [H*d] (8-byte aligned); the array or any entry may be NULL
+ *   y        : np pointers to fp16 [R, H, d]   y_p = x W_p^T + b_p, always written (the
+ *              backward of the feature map needs it)
+ *   phi      : np pointers to fp16 [R, H, 2D], or NULL entries (or a NULL array): projection p
+ *              gets phi(y_p) only where phi[p] is non-NULL
+ *   w_feat   : fp16 [H, D, d] as for rfa_feature_map_forward; may be NULL if no phi is asked for
+ * The pointer arrays themselves live in host memory and are read during the call only.
+ * With every phi NULL this is a plain batched Linear (e.g. out_proj,
+ * causal_attention.py:278) and D only has to be a supported value.
+ * ------------------------------------------------------------------------- */
+int rfa_project_feature_map(const void* x, const void* const* weights, const void* const* biases,
+                            void* const* y, void* const* phi, int np, const void* w_feat, int64_t R,
+                            int E, int H, int D, int d, float scale, void* stream);
+
+/* rfa_linear_weight_grad: weight and bias gradients of those Linear layers, what autograd
+ * computes for torch.nn.Linear in the backward of the lines cited above,
+ *     dW_p [E_out, E_in] = dy_p^T x,    db_p [E_out] = column sums of dy_p,
+ * for np (1..3) layers that share the input x, as a row-split MFMA contraction plus a reduction.
+ *   x  : fp16 [R, E_in]      dy : np pointers to fp16 [R, E_out]
+ *   dw : np pointers to fp16 [E_out, E_in]      db : np pointers to fp16 [E_out] or NULL entries
+ *        (or a NULL array)
+ *   E_out, E_in multiples of 128; workspace of rfa_linear_weight_grad_workspace_bytes bytes. */
+size_t rfa_linear_weight_grad_workspace_bytes(int64_t R, int E_out, int E_in, int np);
+int rfa_linear_weight_grad(const void* x, const void* const* dy, void* const* dw, void* const* db, int np,
+                           int64_t R, int E_out, int E_in, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
+/* ---------------------------------------------------------------------------
  * Cross attention (encoder -> decoder).  The state is fp32.
  *
  * rfa_cross_state replaces the two reductions of

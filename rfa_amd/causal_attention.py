@@ -18,6 +18,7 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import rfa_hip
+from .projection import fused_projection_supported, project_heads
 from .rfa import RFA
 from .utils import (EPS, SCALE, build_random_matrices, random_project,
                     upgrade_state_dict_named)
@@ -164,6 +165,8 @@ class CausalAttention(nn.Module):
             self.sigma = Parameter(Tensor(num_heads, 1, head_dim))
         self.reset_parameters()
         self.upgrade_state_dict_named = upgrade_state_dict_named
+        # q/k/v projections + view to heads + phi(q), phi(k) as one launch when the tensors allow it
+        self.fuse_projections = True
 
     def reset_parameters(self):
         for proj in (self.q_proj, self.k_proj, self.v_proj, self.out_proj):
@@ -189,12 +192,22 @@ class CausalAttention(nn.Module):
         """
         tgt_len, bsz, embed_dim = x.size()
         assert embed_dim == self.embed_dim
-        q = self._heads(self.q_proj(x), tgt_len, bsz)
-        k = self._heads(self.k_proj(x), tgt_len, bsz)
-        v = self._heads(self.v_proj(x), tgt_len, bsz)
         w = build_random_matrices(random_matrices=random_matrices, tau=self.tau,
                                   sigma=self.sigma if self.reparam_proj else None,
                                   reparam_proj=self.reparam_proj)
+        qkv = (self.q_proj, self.k_proj, self.v_proj)
+        if self.fuse_projections and saved_state is None and fused_projection_supported(x, qkv, self.num_heads, w):
+            # the three projections, the view to heads and phi of q and k in one launch
+            phi_q, phi_k, v = project_heads(x, qkv, (True, True, False), self.num_heads, w, SCALE)
+            if self.cuda_causal_rfa:
+                attn = cuda_causal_rfa(phi_q=phi_q, phi_k=phi_k, v=v, key_padding_mask=key_padding_mask)
+            else:
+                attn = masked_rfa(phi_q=phi_q, phi_k=phi_k, v=v, attn_mask=attn_mask,
+                                  key_padding_mask=key_padding_mask)
+            return self.out_proj(attn)
+        q = self._heads(self.q_proj(x), tgt_len, bsz)
+        k = self._heads(self.k_proj(x), tgt_len, bsz)
+        v = self._heads(self.v_proj(x), tgt_len, bsz)
         if saved_state is not None:
             feat = 2 * self.proj_dim
             s, z = saved_state.get("prev_s"), saved_state.get("prev_z")

@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "rfa_causal.h"
+#include "rfa_project.h"
 #include "rfa_decode.h"
 #include "rfa_featuremap.h"
 #include "rfa_masked.h"
@@ -40,12 +41,13 @@ int fail(int code, const char* fmt, ...) {
 // ---- optional per-kernel timing with HIP events ------------------------------------
 namespace prof {
 enum Id { SEG_STATE, CAUSAL_FWD, CAUSAL_BWD_DQ, CAUSAL_BWD_DKDV, CROSS_READOUT, CROSS_READOUT_BWD,
-          CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, MASKED_FWD, MASKED_PREP, MASKED_DQ, MASKED_DKDV, ZERO_FILL,
+          CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, MASKED_FWD, MASKED_PREP, MASKED_DQ, MASKED_DKDV, PROJECT_PHI, WGRAD_PARTIAL, WGRAD_REDUCE, ZERO_FILL,
           SELFTEST, COUNT };
 const char* const kNames[COUNT] = {"k_segment_state", "k_causal_fwd", "k_causal_bwd_dq", "k_causal_bwd_dkdv",
                                    "k_cross_readout", "k_cross_readout_bwd", "k_cross_state_bwd", "k_decode_step",
                                    "k_feature_map_fwd", "k_feature_map_bwd", "k_feature_map_dw_reduce",
-                                   "k_masked_fwd", "k_masked_bwd_prep", "k_masked_dq", "k_masked_dkdv",
+                                   "k_masked_fwd", "k_masked_bwd_prep", "k_masked_dq", "k_masked_dkdv", "k_project_phi",
+                                   "k_weight_grad_partial", "k_weight_grad_reduce",
                                    "k_zero_f32", "k_selftest"};
 struct Rec { int id; hipEvent_t a, b; };
 std::mutex mu;
@@ -405,6 +407,42 @@ int launch_decode(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t*
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
+}
+
+// ---- projection launcher -----------------------------------------------------------
+template <int D, int DH>
+int launch_project_phi(const rfa::half_t* x, const rfa::ProjectArgs& pa, const rfa::half_t* wf, int R, int E, int H,
+                       int np, float scale, hipStream_t st) {
+    using Cfg = rfa::ProjectCfg<D, DH>;
+    auto kern = rfa::k_project_phi<D, DH>;
+    if (int rc = set_lds(kern, Cfg::kLds)) return rc;
+    const int nrt = (R + Cfg::BM - 1) / Cfg::BM;
+    const int64_t grid = (int64_t)8 * ((nrt + 7) / 8) * H * np;
+    RFA_LAUNCH(PROJECT_PHI, kern, dim3((unsigned)grid), dim3(rfa::kThreads), Cfg::kLds, st, x, pa, wf, R, E, H, np, scale);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+// ---- weight-gradient plan -------------------------------------------------------------
+struct WGradPlan {
+    int nsplit;            // row splits (partials to add)
+    int rows_per_split;    // multiple of 64
+};
+
+// About 256-512 workgroups: 8 splits (one per XCD) times as many as the tile count leaves room for.
+WGradPlan make_wgrad_plan(int64_t R, int Eo, int Ei, int np) {
+    const int64_t tiles = (int64_t)np * (Eo / 128) * (Ei / 128);
+    const int64_t nchunks = (R + 63) / 64;
+    int64_t want = 8 * ((32 + tiles - 1) / tiles);
+    if (want > 64) want = 64;
+    if (want > nchunks) want = nchunks;
+    if (want < 1) want = 1;
+    const int64_t cps = (nchunks + want - 1) / want;
+    WGradPlan p;
+    p.rows_per_split = (int)(cps * 64);
+    p.nsplit = (int)((nchunks + cps - 1) / cps);
+    if (p.nsplit < 1) p.nsplit = 1;
+    return p;
 }
 
 // ---- feature map launchers ---------------------------------------------------------
@@ -988,6 +1026,93 @@ int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi,
     RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+// ---- projection to heads with the feature map in the epilogue -------------------------
+int rfa_project_feature_map(const void* x, const void* const* weights, const void* const* biases, void* const* y,
+                            void* const* phi, int np, const void* w_feat, int64_t R, int E, int H, int D, int d,
+                            float scale, void* stream) {
+    if (int rc = check_feature_dims("rfa_project_feature_map", R, H, D, d)) return rc;
+    if (np < 1 || np > rfa::kMaxProjections)
+        return fail(RFA_ERR_BAD_SHAPE, "rfa_project_feature_map: %d projections (1..%d supported)", np, rfa::kMaxProjections);
+    if (E < 64 || E % 64 != 0)
+        return fail(RFA_ERR_BAD_SHAPE, "rfa_project_feature_map: input width E=%d must be a positive multiple of 64", E);
+    if (R == 0) return RFA_OK;
+    if (!x || !weights || !y) return fail(RFA_ERR_NULL_POINTER, "rfa_project_feature_map: NULL tensor pointer");
+    if (!aligned16(x)) return fail(RFA_ERR_ALIGNMENT, "rfa_project_feature_map: tensors must be 16-byte aligned");
+    if ((int64_t)8 * ((R + 127) / 128 + 7) / 8 * H * np > (int64_t(1) << 31) - 1)
+        return fail(RFA_ERR_BAD_SHAPE, "rfa_project_feature_map: sizes exceed the supported range");
+    rfa::ProjectArgs pa{};
+    bool any_phi = false;
+    for (int p = 0; p < np; ++p) {
+        pa.w[p] = static_cast<const rfa::half_t*>(weights[p]);
+        pa.b[p] = biases ? static_cast<const rfa::half_t*>(biases[p]) : nullptr;
+        pa.y[p] = static_cast<rfa::half_t*>(y[p]);
+        pa.phi[p] = phi ? static_cast<rfa::half_t*>(phi[p]) : nullptr;
+        if (!pa.w[p] || !pa.y[p]) return fail(RFA_ERR_NULL_POINTER, "rfa_project_feature_map: NULL weight or output %d", p);
+        if (!aligned16(pa.w[p]) || !aligned16(pa.y[p]) || !aligned16(pa.phi[p]) ||
+            (reinterpret_cast<uintptr_t>(pa.b[p]) & 7u))
+            return fail(RFA_ERR_ALIGNMENT, "rfa_project_feature_map: tensors must be 16-byte aligned (bias: 8)");
+        any_phi = any_phi || pa.phi[p];
+    }
+    if (any_phi && !w_feat) return fail(RFA_ERR_NULL_POINTER, "rfa_project_feature_map: NULL feature matrices");
+    if (!aligned16(w_feat)) return fail(RFA_ERR_ALIGNMENT, "rfa_project_feature_map: tensors must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* xh = static_cast<const rfa::half_t*>(x);
+    auto* wfh = static_cast<const rfa::half_t*>(w_feat);
+#define RFA_CALL(DD, DH) launch_project_phi<DD, DH>(xh, pa, wfh, (int)R, E, H, np, scale, st)
+    RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+size_t rfa_linear_weight_grad_workspace_bytes(int64_t R, int E_out, int E_in, int np) {
+    if (R <= 0 || E_out <= 0 || E_in <= 0 || E_out % 128 || E_in % 128 || np < 1 || np > rfa::kMaxProjections) return 0;
+    const WGradPlan pl = make_wgrad_plan(R, E_out, E_in, np);
+    return (size_t)pl.nsplit * np * ((size_t)E_out * E_in + E_out) * 4;
+}
+
+int rfa_linear_weight_grad(const void* x, const void* const* dy, void* const* dw, void* const* db, int np, int64_t R,
+                           int E_out, int E_in, void* workspace, size_t workspace_bytes, void* stream) {
+    if (R < 0 || E_out <= 0 || E_in <= 0 || R > (int64_t(1) << 30))
+        return fail(RFA_ERR_BAD_SHAPE, "rfa_linear_weight_grad: bad sizes rows=%lld E_out=%d E_in=%d", (long long)R, E_out, E_in);
+    if (E_out % 128 || E_in % 128)
+        return fail(RFA_ERR_UNSUPPORTED, "rfa_linear_weight_grad: E_out=%d and E_in=%d must be multiples of 128", E_out, E_in);
+    if (np < 1 || np > rfa::kMaxProjections)
+        return fail(RFA_ERR_BAD_SHAPE, "rfa_linear_weight_grad: %d projections (1..%d supported)", np, rfa::kMaxProjections);
+    if (!dy || !dw) return fail(RFA_ERR_NULL_POINTER, "rfa_linear_weight_grad: NULL pointer array");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    rfa::WeightGradArgs wa{};
+    for (int p = 0; p < np; ++p) {
+        wa.dy[p] = static_cast<const rfa::half_t*>(dy[p]);
+        wa.dw[p] = static_cast<rfa::half_t*>(dw[p]);
+        wa.db[p] = db ? static_cast<rfa::half_t*>(db[p]) : nullptr;
+        if (!wa.dw[p] || (R > 0 && !wa.dy[p])) return fail(RFA_ERR_NULL_POINTER, "rfa_linear_weight_grad: NULL tensor %d", p);
+        if (!aligned16(wa.dy[p]) || !aligned16(wa.dw[p]) || (reinterpret_cast<uintptr_t>(wa.db[p]) & 7u))
+            return fail(RFA_ERR_ALIGNMENT, "rfa_linear_weight_grad: tensors must be 16-byte aligned (bias gradient: 8)");
+    }
+    if (R > 0 && !x) return fail(RFA_ERR_NULL_POINTER, "rfa_linear_weight_grad: NULL x");
+    if (!aligned16(x)) return fail(RFA_ERR_ALIGNMENT, "rfa_linear_weight_grad: tensors must be 16-byte aligned");
+    const WGradPlan pl = make_wgrad_plan(R > 0 ? R : 1, E_out, E_in, np);
+    const size_t need = (size_t)pl.nsplit * np * ((size_t)E_out * E_in + E_out) * 4;
+    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+        return fail(RFA_ERR_WORKSPACE, "rfa_linear_weight_grad: workspace of %zu bytes required, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    float* part = static_cast<float*>(workspace);
+    float* bpart = part + (size_t)pl.nsplit * np * E_out * E_in;
+    const int per_split = np * (E_out / 128) * (E_in / 128);
+    const int64_t grid = (int64_t)8 * ((pl.nsplit + 7) / 8) * per_split;
+    if (grid > (int64_t(1) << 30)) return fail(RFA_ERR_BAD_SHAPE, "rfa_linear_weight_grad: sizes exceed the supported range");
+    auto kern = rfa::k_weight_grad_partial;
+    if (int rc = set_lds(kern, rfa::WeightGradCfg::kLds)) return rc;
+    // R = 0: every split is empty and the partials come out as zeros
+    RFA_LAUNCH(WGRAD_PARTIAL, kern, dim3((unsigned)grid), dim3(rfa::kThreads), rfa::WeightGradCfg::kLds, st,
+               static_cast<const rfa::half_t*>(x), wa, part, bpart, (int)R, E_out, E_in, np, pl.nsplit, pl.rows_per_split);
+    const int64_t threads = (int64_t)np * ((int64_t)E_out * E_in + E_out) / 4;
+    RFA_LAUNCH(WGRAD_REDUCE, rfa::k_weight_grad_reduce, dim3((unsigned)((threads + 255) / 256)), dim3(rfa::kThreads), 0, st,
+               (const float*)part, (const float*)bpart, wa, E_out, E_in, np, pl.nsplit);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
 }
 
 // ---- profiling ----------------------------------------------------------------------

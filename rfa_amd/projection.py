@@ -1,0 +1,111 @@
+"""Input projections of the attention modules on the fused projection + feature-map launch.
+
+The reference modules run ``q_proj / k_proj / v_proj`` (torch.nn.Linear), view the results as
+heads and call ``random_project`` on q and k (causal_attention.py:228-247;
+cross_attention.py:66-76, :279-283).  ``project_heads`` does that chain in one kernel launch
+(``rfa_project_feature_map``) and differentiates it with the feature-map backward kernel plus
+library GEMMs for the Linear layers.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+from torch import Tensor, nn
+
+from . import rfa_hip
+
+
+def linear_param_grads(x2: Tensor, dys: Sequence[Tensor], has_bias: Sequence[bool]):
+    """(dW, db) lists of Linear layers sharing the input x2 [R, E_in], given dy [R, E_out] each:
+    one row-split MFMA launch when the sizes allow it, library GEMMs and column sums otherwise."""
+    e_out, e_in = dys[0].shape[1], x2.shape[1]
+    if (x2.is_cuda and x2.dtype == torch.float16 and all(d.dtype == torch.float16 for d in dys)
+            and rfa_hip.linear_weight_grad_supported(e_out, e_in) and 1 <= len(dys) <= 3):
+        return rfa_hip.linear_weight_grad(x2.contiguous(), [d.contiguous() for d in dys], list(has_bias))
+    return ([torch.mm(d.t(), x2) for d in dys], [d.sum(0) if b else None for d, b in zip(dys, has_bias)])
+
+
+class _ProjectHeads(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x: Tensor, w_feat: Optional[Tensor], scale: float, heads: int, want_phi: Tuple[bool, ...],
+                *params: Optional[Tensor]):
+        n = len(want_phi)
+        weights, biases = list(params[0::2]), list(params[1::2])
+        wf = None if w_feat is None else w_feat.contiguous()
+        ys, phis = rfa_hip.project_feature_map(x.contiguous(), [w.contiguous() for w in weights], biases, list(want_phi),
+                                               wf, heads, scale)
+        ctx.scale, ctx.heads, ctx.want_phi = scale, heads, want_phi
+        ctx.has_bias = tuple(b is not None for b in biases)
+        ctx.has_wf = w_feat is not None
+        ctx.save_for_backward(x, *([wf] if wf is not None else []), *weights, *[y for y, f in zip(ys, want_phi) if f])
+        return tuple(phis[p] if want_phi[p] else ys[p] for p in range(n))
+
+    @staticmethod
+    def backward(ctx, *grads: Tensor):
+        saved = list(ctx.saved_tensors)
+        x = saved.pop(0)
+        wf = saved.pop(0) if ctx.has_wf else None
+        n = len(ctx.want_phi)
+        weights, ys = saved[:n], saved[n:]
+        L, B, E = x.shape
+        x2 = x.reshape(L * B, E)
+        dx = None
+        dwf = None
+        dys = []
+        yi = 0
+        for p in range(n):
+            g = grads[p].contiguous()
+            if ctx.want_phi[p]:
+                dy, dw = rfa_hip.feature_map_backward(ys[yi], wf, g, ctx.scale)
+                yi += 1
+                dwf = dw if dwf is None else dwf + dw
+            else:
+                dy = g
+            dy2 = dy.reshape(L * B, -1)
+            dys.append(dy2)
+            if ctx.needs_input_grad[0]:
+                dx = torch.mm(dy2, weights[p]) if dx is None else dx.addmm_(dy2, weights[p])
+        dws, dbs = linear_param_grads(x2, dys, ctx.has_bias)
+        dparams = []
+        for p in range(n):
+            dparams += [dws[p], dbs[p]]
+        if dx is not None:
+            dx = dx.view(L, B, E)
+        if dwf is not None:
+            dwf = dwf.to(wf.dtype)
+        return (dx, dwf, None, None, None, *dparams)
+
+
+def fused_projection_supported(x: Tensor, layers: Sequence[nn.Linear], heads: int,
+                               w_feat: Optional[Tensor] = None) -> bool:
+    """True when the fused launch can stand in for ``[layer(x) for layer in layers]``: fp16 HIP
+    tensors, a common [out, in] weight shape with ``in`` a multiple of 64 and a head width of
+    64 or 128 (and a supported proj_dim if a feature map is asked for)."""
+    if not (x.is_cuda and x.dtype == torch.float16 and x.dim() == 3 and 1 <= len(layers) <= 3):
+        return False
+    out_dim, in_dim = layers[0].weight.shape
+    if in_dim != x.shape[-1] or in_dim % 64 != 0 or out_dim % heads != 0 or out_dim // heads not in (64, 128):
+        return False
+    for layer in layers:
+        if tuple(layer.weight.shape) != (out_dim, in_dim) or layer.weight.dtype != torch.float16:
+            return False
+        if layer.bias is not None and layer.bias.dtype != torch.float16:
+            return False
+    if w_feat is not None:
+        if w_feat.dtype != torch.float16 or w_feat.dim() != 3 or w_feat.shape[1] not in (32, 64, 128):
+            return False
+    return True
+
+
+def project_heads(x: Tensor, layers: Sequence[nn.Linear], want_phi: Sequence[bool], heads: int,
+                  w_feat: Optional[Tensor], scale: float):
+    """``[phi(layer(x)) if flag else layer(x)]`` viewed as [L, B, heads, .], in one launch.
+
+    x: [L, B, E] fp16 on a HIP device; layers: 1..3 ``nn.Linear`` with equal weight shapes;
+    w_feat: [heads, proj_dim, head_dim] (None when no flag is set).
+    """
+    params = []
+    for layer in layers:
+        params += [layer.weight, layer.bias]
+    return _ProjectHeads.apply(x, w_feat, scale, heads, tuple(bool(f) for f in want_phi), *params)

@@ -188,6 +188,86 @@ def feature_map_forward(x: Tensor, w: Tensor, scale: float) -> Tensor:
     return phi
 
 
+def project_feature_map(x: Tensor, weights, biases, want_phi, w: Optional[Tensor], heads: int, scale: float):
+    """Linear projections of x to heads, with the feature map applied to some of them, in one launch.
+
+    x fp16 [L, B, E]; weights: 1..3 fp16 [heads*d, E] (torch.nn.Linear.weight); biases: a matching
+    list of fp16 [heads*d] or None entries; want_phi: one bool per projection; w fp16 [heads, D, d]
+    (None allowed when no phi is wanted).  Returns (ys, phis): ys[p] fp16 [L, B, heads, d];
+    phis[p] fp16 [L, B, heads, 2D] or None.
+    """
+    import ctypes
+    _check_half_cuda("x", x, 3)
+    L, B, E = x.shape
+    n = len(weights)
+    _require(1 <= n <= 3 and len(biases) == n and len(want_phi) == n, ValueError,
+             "1..3 projections with one bias entry and one want_phi flag each")
+    out_dim = weights[0].shape[0]
+    _require(out_dim % heads == 0, ValueError, f"output width {out_dim} is not a multiple of heads={heads}")
+    d = out_dim // heads
+    for wt, b in zip(weights, biases):
+        _check_half_cuda("weight", wt, 2)
+        _require(tuple(wt.shape) == (out_dim, E), ValueError, f"weight {tuple(wt.shape)} must be {(out_dim, E)}")
+        _require(wt.device == x.device, RuntimeError, "x and weights must be on one device")
+        if b is not None:
+            _check_half_cuda("bias", b, 1)
+            _require(b.shape[0] == out_dim and b.device == x.device, ValueError, f"bias must be [{out_dim}] on x's device")
+    if any(want_phi):
+        _require(w is not None, ValueError, "feature matrices are needed when a phi is wanted")
+        _check_half_cuda("random_matrices", w, 3)
+        _require(w.shape[0] == heads and w.shape[2] == d and w.device == x.device, ValueError,
+                 f"random_matrices {tuple(w.shape)} must be [{heads}, D, {d}] on x's device")
+        D = w.shape[1]
+    else:
+        D = 32
+    ys = [torch.empty((L, B, heads, d), dtype=torch.float16, device=x.device) for _ in range(n)]
+    phis = [torch.empty((L, B, heads, 2 * D), dtype=torch.float16, device=x.device) if f else None for f in want_phi]
+    arr = ctypes.c_void_p * n
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().rfa_project_feature_map(
+            x.data_ptr(), arr(*[wt.data_ptr() for wt in weights]), arr(*[ptr(b) for b in biases]),
+            arr(*[t.data_ptr() for t in ys]), arr(*[ptr(t) for t in phis]), n, ptr(w) if any(want_phi) else None,
+            L * B, E, heads, D, d, float(scale), _stream_ptr(x.device)))
+    return ys, phis
+
+
+def linear_weight_grad_supported(e_out: int, e_in: int) -> bool:
+    return e_out % 128 == 0 and e_in % 128 == 0
+
+
+def linear_weight_grad(x: Tensor, dys, want_bias):
+    """(dWs, dbs) of 1..3 Linear layers that share the input: dW_p = dy_p^T x, db_p = dy_p.sum(0).
+
+    x fp16 [R, E_in]; dys: fp16 [R, E_out] each; want_bias: one bool per layer.  dWs[p] fp16
+    [E_out, E_in]; dbs[p] fp16 [E_out] or None.  E_out and E_in must be multiples of 128.
+    """
+    import ctypes
+    _check_half_cuda("x", x, 2)
+    R, e_in = x.shape
+    n = len(dys)
+    _require(1 <= n <= 3 and len(want_bias) == n, ValueError, "1..3 layers with one want_bias flag each")
+    e_out = dys[0].shape[1]
+    for dy in dys:
+        _check_half_cuda("dy", dy, 2)
+        _require(tuple(dy.shape) == (R, e_out) and dy.device == x.device, ValueError,
+                 f"dy {tuple(dy.shape)} must be {(R, e_out)} on x's device")
+    _require(linear_weight_grad_supported(e_out, e_in), ValueError,
+             f"E_out={e_out} and E_in={e_in} must be multiples of 128")
+    lib = _lib.load()
+    dws = [torch.empty((e_out, e_in), dtype=torch.float16, device=x.device) for _ in range(n)]
+    dbs = [torch.empty((e_out,), dtype=torch.float16, device=x.device) if f else None for f in want_bias]
+    arr = ctypes.c_void_p * n
+    with torch.cuda.device(x.device):
+        nbytes = lib.rfa_linear_weight_grad_workspace_bytes(max(R, 1), e_out, e_in, n)
+        ws = _workspace(nbytes, x.device)
+        _lib.check(lib.rfa_linear_weight_grad(
+            x.data_ptr(), arr(*[t.data_ptr() for t in dys]), arr(*[t.data_ptr() for t in dws]),
+            arr(*[None if t is None else t.data_ptr() for t in dbs]), n, R, e_out, e_in, ws.data_ptr(), nbytes,
+            _stream_ptr(x.device)))
+    return dws, dbs
+
+
 def feature_map_backward(x: Tensor, w: Tensor, grad_phi: Tensor, scale: float):
     """(dx fp16 [L,B,H,d], dw fp32 [H,D,d])."""
     _check_feature_args(x, w)

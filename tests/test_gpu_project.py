@@ -1,0 +1,183 @@
+"""GPU parity (through the C ABI) of the fused Linear -> heads -> feature map launch
+against torch's fp64 matmul and the CPU oracle's feature map.
+
+Tolerances: the projections y are fp16 roundings of an fp32-accumulated product, compared
+with the fp64 product of the same fp16 inputs: |dy| <= 1.5e-3 * max(1, |y|) (one fp16 ulp
+is 9.8e-4 relative).  phi is compared (a) with the oracle applied to the y the kernel itself
+returned (<= 2e-3 absolute, the feature-map bar) and (b) with the oracle applied to the
+fp64 product rounded to fp16 (<= 4e-3: an ulp of difference in y moves the angle).
+"""
+import pytest
+import torch
+
+from oracle import rfa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# L, B, E, H, d, D
+SHAPES = [(128, 2, 256, 4, 64, 64), (70, 3, 128, 2, 64, 64), (33, 1, 256, 2, 128, 128), (5, 2, 64, 1, 64, 32),
+          (1, 1, 192, 3, 64, 128), (257, 1, 128, 1, 128, 64)]
+
+
+def _randn(*shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=torch.float32)
+
+
+def _inputs(L, B, E, H, d, seed, n):
+    x = (_randn(L, B, E, seed=seed) * 0.8).half()
+    ws = [(_randn(H * d, E, seed=seed + 1 + p) / E ** 0.5 * 1.5).half() for p in range(n)]
+    bs = [(_randn(H * d, seed=seed + 11 + p) * 0.3).half() for p in range(n)]
+    return x, ws, bs
+
+
+def _linear64(x, w, b, H, d):
+    y = x.double() @ w.double().t()
+    if b is not None:
+        y = y + b.double()
+    return y.view(*x.shape[:2], H, d)
+
+
+@pytest.mark.parametrize("L,B,E,H,d,D", SHAPES)
+def test_qkv_projection_with_feature_map(L, B, E, H, d, D):
+    from rfa_amd import rfa_hip
+    x, ws, bs = _inputs(L, B, E, H, d, 900 + L, 3)
+    bs[1] = None                                       # one projection without bias
+    wf = (_randn(H, D, d, seed=77) * 0.9).half()
+    print(f"project+phi L={L} B={B} E={E} H={H} d={d} D={D}", flush=True)
+    dev = lambda t: None if t is None else t.cuda()
+    ys, phis = rfa_hip.project_feature_map(x.cuda(), [w.cuda() for w in ws], [dev(b) for b in bs],
+                                           [True, True, False], wf.cuda(), H, O.SCALE)
+    assert phis[2] is None and phis[0].shape == (L, B, H, 2 * D)
+    for p in range(3):
+        want = _linear64(x, ws[p], bs[p], H, d)
+        got = ys[p].double().cpu()
+        assert ys[p].shape == (L, B, H, d)
+        assert ((got - want).abs() <= 1.5e-3 * want.abs().clamp_min(1.0)).all(), (p, (got - want).abs().max().item())
+        if p < 2:
+            phi = phis[p].float().cpu()
+            own = O.random_project(ys[p].float().cpu(), wf.float())
+            assert (phi - own).abs().max().item() <= 2e-3
+            ref = O.random_project(want.half().float(), wf.float())
+            assert (phi - ref).abs().max().item() <= 4e-3
+
+
+def test_plain_projection_is_a_linear_layer():
+    """No phi requested: out_proj-style use, one projection, with and without bias."""
+    from rfa_amd import rfa_hip
+    L, B, E, H, d = 130, 2, 512, 8, 64
+    x, ws, bs = _inputs(L, B, E, H, d, 950, 1)
+    for b in (bs[0], None):
+        ys, phis = rfa_hip.project_feature_map(x.cuda(), [ws[0].cuda()], [None if b is None else b.cuda()], [False],
+                                               None, H, O.SCALE)
+        assert phis == [None]
+        want = _linear64(x, ws[0], b, H, d)
+        got = ys[0].double().cpu()
+        assert ((got - want).abs() <= 1.5e-3 * want.abs().clamp_min(1.0)).all()
+        ref16 = torch.nn.functional.linear(x.cuda(), ws[0].cuda(), None if b is None else b.cuda()).view(L, B, H, d)
+        assert (ys[0].float() - ref16.float()).abs().max().item() <= 4e-3      # the library GEMM, for reference
+
+
+def test_zero_rows_and_argument_checks():
+    from rfa_amd import rfa_hip
+    H, d, D, E = 2, 64, 64, 128
+    x, ws, bs = _inputs(4, 1, E, H, d, 960, 2)
+    x[1] = 0
+    ws = [w.cuda() for w in ws]
+    wf = (_randn(H, D, d, seed=78)).half().cuda()
+    ys, phis = rfa_hip.project_feature_map(x.cuda(), ws, [None, None], [True, True], wf, H, O.SCALE)
+    # a zero input row without bias projects to zero, whose phi is [0.., scale..]
+    assert (ys[0][1] == 0).all()
+    assert (phis[0][1, 0, :, :D] == 0).all() and (phis[0][1, 0, :, D:].float() - O.SCALE).abs().max() <= 1e-4
+    with pytest.raises(ValueError):
+        rfa_hip.project_feature_map(x.cuda(), ws, [None], [True, True], wf, H, O.SCALE)
+    with pytest.raises(ValueError):
+        rfa_hip.project_feature_map(x.cuda(), ws, [None, None], [True, False], None, H, O.SCALE)
+    with pytest.raises((RuntimeError, ValueError)):
+        rfa_hip.project_feature_map(x[..., :100].contiguous().cuda(), [w[:, :100].contiguous() for w in ws],
+                                    [None, None], [False, False], None, H, O.SCALE)    # E not a multiple of 64
+    with pytest.raises((RuntimeError, TypeError)):
+        rfa_hip.project_feature_map(x, [w.cpu() for w in ws], [None, None], [False, False], None, H, O.SCALE)
+
+
+@pytest.mark.parametrize("with_pad", [False, True])
+def test_causal_module_fused_projections_match_unfused_chain(with_pad):
+    """CausalAttention with the q/k/v projections + phi as one launch vs the same module running
+    nn.Linear + random_project: outputs within 4e-3, every gradient within 1e-2 (relative
+    Frobenius norm) of the unfused module's, and within 2e-2 of an fp64 autograd run of the
+    oracle chain."""
+    from rfa_amd import CausalAttention
+    torch.manual_seed(5)
+    T, B, E, H, d, D = 200, 3, 256, 4, 64, 64
+    m = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half()
+    with torch.no_grad():
+        m.sigma.mul_(1.0 + 0.1 * torch.randn_like(m.sigma))
+        m.out_proj.bias.normal_(0, 0.1)
+    W = O.make_w(d, D, H).cuda().half()
+    x0 = (torch.randn(T, B, E) * 0.7).half()
+    go = torch.randn(T, B, E).half().cuda()
+    pad = None
+    if with_pad:
+        pad = torch.zeros(B, T, dtype=torch.bool)
+        pad[1, 150:] = True
+        pad = pad.cuda()
+
+    def run(fused):
+        m.fuse_projections = fused
+        m.zero_grad(set_to_none=True)
+        x = x0.clone().cuda().requires_grad_(True)
+        y = m(x, W, key_padding_mask=pad)
+        y.backward(go)
+        return y.detach().float().cpu(), {"x": x.grad.float().cpu(),
+                                          **{n: p.grad.float().cpu() for n, p in m.named_parameters()}}
+
+    y_f, g_f = run(True)
+    y_u, g_u = run(False)
+    assert (y_f - y_u).abs().max().item() <= 4e-3
+    rel = lambda a, b: ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+    for name in g_u:
+        assert torch.isfinite(g_f[name]).all(), name
+        assert rel(g_f[name], g_u[name]) <= 1e-2, (name, rel(g_f[name], g_u[name]))
+
+    # fp64 autograd through the oracle chain with the same fp16 parameters
+    P = {n: p.detach().double().cpu().requires_grad_(True) for n, p in m.named_parameters()}
+    x = x0.double().requires_grad_(True)
+    lin = lambda n: x @ P[n + ".weight"].t() + P[n + ".bias"]
+    q, k, v = (lin(n).reshape(T, B, H, d) for n in ("q_proj", "k_proj", "v_proj"))
+    Wp = O.build_random_matrices(W.double().cpu(), 1.0, P["sigma"], True)
+    pq, pk = O.random_project(q, Wp), O.random_project(k, Wp)
+    if with_pad:
+        pk = pk.masked_fill(pad.cpu().t()[:, :, None, None], 0.0)
+    att = O.causal_forward_chunked(pq.reshape(T, B * H, 2 * D), pk.reshape(T, B * H, 2 * D), v.reshape(T, B * H, d))
+    want = att.reshape(T, B, E) @ P["out_proj.weight"].t() + P["out_proj.bias"]
+    assert (y_f.double() - want.detach()).abs().max().item() <= 1e-2
+    want.backward(go.double().cpu())
+    ref = {"x": x.grad, **{n: p.grad for n, p in P.items()}}
+    for name in ref:
+        assert rel(g_f[name].double(), ref[name]) <= 2e-2, (name, rel(g_f[name].double(), ref[name]))
+
+
+@pytest.mark.parametrize("R,Eo,Ei,n", [(8192, 512, 512, 3), (200, 128, 256, 1), (1, 128, 128, 2), (4097, 256, 128, 3),
+                                       (64, 384, 128, 1)])
+def test_linear_weight_and_bias_gradients(R, Eo, Ei, n):
+    """dW = dy^T x and db = column sums against fp64; fp16 outputs of fp32 sums: <= 1.5e-3 relative
+    to max(1, |value|) per element, and <= 1e-3 relative Frobenius error."""
+    from rfa_amd import rfa_hip
+    x = (_randn(R, Ei, seed=970 + R) * 0.5).half()
+    dys = [(_randn(R, Eo, seed=971 + p) * 0.05).half() for p in range(n)]
+    want_bias = [p != 1 for p in range(n)]
+    print(f"weight grad R={R} Eo={Eo} Ei={Ei} n={n}", flush=True)
+    dws, dbs = rfa_hip.linear_weight_grad(x.cuda(), [d.cuda() for d in dys], want_bias)
+    for p in range(n):
+        ww = dys[p].double().t() @ x.double()
+        got = dws[p].double().cpu()
+        assert ((got - ww).abs() <= 1.5e-3 * ww.abs().clamp_min(1.0)).all(), (p, (got - ww).abs().max().item())
+        assert ((got - ww).norm() / ww.norm()).item() <= 1e-3
+        if want_bias[p]:
+            wb = dys[p].double().sum(0)
+            gb = dbs[p].double().cpu()
+            assert ((gb - wb).abs() <= 1.5e-3 * wb.abs().clamp_min(1.0)).all()
+        else:
+            assert dbs[p] is None
+    with pytest.raises(ValueError):
+        rfa_hip.linear_weight_grad(x[:, :64].contiguous().cuda(), [d.cuda() for d in dys], want_bias)
