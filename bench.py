@@ -310,6 +310,57 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream):
                          "fwd_us": round(1e3 * tf, 2), "bwd_us": round(1e3 * tb, 2),
                          "fwd_hbm_gbs": round(rows * (d + 2 * D) * 2 / (tf * 1e-3) / 1e9, 1),
                          "bwd_hbm_gbs": round(rows * (2 * d + 2 * D) * 2 / (tb * 1e-3) / 1e9, 1)}
+    # ---- whole CausalAttention module (config 2 shape, embed 512): forward + backward of the module
+    # with its projections on the library's kernels, the same module on nn.Linear + separate phi
+    # launches, and the fused module replayed from a HIP graph (no host work per step)
+    from rfa_amd import CausalAttention
+    torch.manual_seed(0)
+    E = H * d
+    mod = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).to(dev).half()
+    mx = (torch.randn(T, B, E, generator=g) * 0.5).half().to(dev).requires_grad_(True)
+    mg = torch.randn(T, B, E, generator=g).half().to(dev)
+
+    def mstep():
+        mod.zero_grad(set_to_none=True)
+        mx.grad = None
+        y = mod(mx, W)
+        y.backward(mg)
+        return y
+
+    def timed(fn, n=20):
+        for _ in range(3):
+            fn()
+        return 1e3 * _event_time_ms(torch, fn, n)
+
+    fused_us = timed(mstep)
+    mod.fuse_projections = False
+    unfused_us = timed(mstep)
+    mod.fuse_projections = True
+    y_eager = mstep().detach().clone()
+    gx_eager = mx.grad.detach().clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            mstep()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    mod.zero_grad(set_to_none=True)
+    mx.grad = None
+    with torch.cuda.graph(graph):
+        y_graph = mod(mx, W)
+        y_graph.backward(mg)
+    graph_us = timed(graph.replay)
+    mstep()                                      # eager work between replays
+    graph.replay()
+    torch.cuda.synchronize()
+    ex["module_step"] = {"workload": "CausalAttention(embed 512, 8 heads) forward + backward on [1024, 8, 512] fp16",
+                         "eager_us": round(fused_us, 1), "eager_library_projections_us": round(unfused_us, 1),
+                         "hip_graph_replay_us": round(graph_us, 1),
+                         "graph_equals_eager": bool(torch.equal(y_graph, y_eager) and torch.equal(mx.grad, gx_eager))}
+    del graph, mod
+
     # ---- plain device copy of 512 MiB (larger than the 256 MiB last-level cache): the HBM
     # bandwidth a trivial kernel reaches here, and the known-size dispatch against which the
     # rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled

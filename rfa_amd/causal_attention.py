@@ -18,7 +18,7 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import rfa_hip
-from .projection import fused_projection_supported, project_heads
+from .projection import fused_projection_supported, linear_out, project_heads
 from .rfa import RFA
 from .utils import (EPS, SCALE, build_random_matrices, random_project,
                     upgrade_state_dict_named)
@@ -204,7 +204,7 @@ class CausalAttention(nn.Module):
             else:
                 attn = masked_rfa(phi_q=phi_q, phi_k=phi_k, v=v, attn_mask=attn_mask,
                                   key_padding_mask=key_padding_mask)
-            return self.out_proj(attn)
+            return linear_out(attn, self.out_proj)
         q = self._heads(self.q_proj(x), tgt_len, bsz)
         k = self._heads(self.k_proj(x), tgt_len, bsz)
         v = self._heads(self.v_proj(x), tgt_len, bsz)
@@ -248,4 +248,4 @@ class CausalAttention(nn.Module):
             else:
                 attn = masked_rfa(phi_q=phi_q, phi_k=phi_k, v=v, attn_mask=attn_mask,
                                   key_padding_mask=key_padding_mask)
-        return self.out_proj(attn)
+        return linear_out(attn, self.out_proj)

@@ -15,7 +15,8 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import rfa_hip
-from .utils import (EPS, CrossAttentionState, build_random_matrices, load_random_matrices, random_project,
+from .projection import fused_projection_supported, linear_out, project_heads
+from .utils import (EPS, SCALE, CrossAttentionState, build_random_matrices, load_random_matrices, random_project,
                     sample_random_matrices, upgrade_state_dict_named)
 
 
@@ -72,6 +73,7 @@ class CrossAttentionProjectLayer(nn.Module):
             self.sigma = Parameter(Tensor(num_heads, 1, head_dim))
         self.reset_parameters()
         self.upgrade_state_dict_named = upgrade_state_dict_named
+        self.fuse_projections = True      # k/v projections + view to heads + phi(k) as one launch when possible
 
     def reset_parameters(self):
         nn.init.xavier_uniform_(self.k_proj.weight, gain=1 / math.sqrt(2))
@@ -85,12 +87,17 @@ class CrossAttentionProjectLayer(nn.Module):
         Returns (s [bsz, heads, 2*proj_dim, head_dim], z [bsz, heads, 2*proj_dim], W', tau)
         (reference cross_attention.py:52-106)."""
         src_len, bsz, _ = encoder_output.size()
-        k = self.k_proj(encoder_output).contiguous().view(src_len, bsz, self.num_heads, self.head_dim)
-        v = self.v_proj(encoder_output).contiguous().view(src_len, bsz, self.num_heads, self.head_dim)
         w = build_random_matrices(random_matrices=random_matrices, tau=self.tau,
                                   sigma=self.sigma if self.reparam_proj else None,
                                   reparam_proj=self.reparam_proj)
-        phi_k = random_project(x=k, random_matrices=w)
+        kv = (self.k_proj, self.v_proj)
+        if self.fuse_projections and fused_projection_supported(encoder_output, kv, self.num_heads, w):
+            # both projections, the view to heads and phi(k) in one launch
+            phi_k, v = project_heads(encoder_output, kv, (True, False), self.num_heads, w, SCALE)
+        else:
+            k = self.k_proj(encoder_output).contiguous().view(src_len, bsz, self.num_heads, self.head_dim)
+            v = self.v_proj(encoder_output).contiguous().view(src_len, bsz, self.num_heads, self.head_dim)
+            phi_k = random_project(x=k, random_matrices=w)
         pad = None
         if mask is not None:
             pad = mask.reshape(src_len, bsz).transpose(0, 1).contiguous()   # [bsz, src_len]
@@ -158,6 +165,7 @@ class CrossAttention(nn.Module):
         self.out_proj = nn.Linear(embed_dim, embed_dim, bias=True)
         self.reset_parameters()
         self.upgrade_state_dict_named = upgrade_state_dict_named
+        self.fuse_projections = True      # q projection + view to heads + phi(q) as one launch when possible
 
     def reset_parameters(self):
         for proj in (self.q_proj, self.out_proj):
@@ -176,7 +184,12 @@ class CrossAttention(nn.Module):
         s, z, random_matrices, tau = state
         tgt_len, bsz, embed_dim = query.size()
         assert embed_dim == self.embed_dim
-        q = self.q_proj(query).contiguous().view(tgt_len, bsz, self.num_heads, self.head_dim)
-        attn = self.rfa(q, s, z, random_matrices)
+        if self.fuse_projections and fused_projection_supported(query, (self.q_proj,), self.num_heads, random_matrices):
+            # q projection, the view to heads and phi(q) in one launch
+            (phi_q,) = project_heads(query, (self.q_proj,), (True,), self.num_heads, random_matrices, SCALE)
+            attn = _CrossReadout.apply(phi_q, s, z)
+        else:
+            q = self.q_proj(query).contiguous().view(tgt_len, bsz, self.num_heads, self.head_dim)
+            attn = self.rfa(q, s, z, random_matrices)
         assert list(attn.size()) == [tgt_len, bsz, self.num_heads, self.head_dim]
-        return self.out_proj(attn.contiguous().view(tgt_len, bsz, self.num_heads * self.head_dim))
+        return linear_out(attn.contiguous().view(tgt_len, bsz, self.num_heads * self.head_dim), self.out_proj)

@@ -410,9 +410,37 @@ int launch_decode(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t*
 }
 
 // ---- projection launcher -----------------------------------------------------------
+template <int D, int DH, int NKS>
+int launch_project_rows(const rfa::half_t* x, const rfa::ProjectArgs& pa, const rfa::half_t* wf, int R, int H, int np,
+                        float scale, hipStream_t st) {
+    // rows of x in registers; split the H * np pairs of a row tile over enough groups to fill the CUs
+    using Cfg = rfa::ProjectRowCfg<D, DH, NKS>;
+    auto kern = rfa::k_project_phi_rows<D, DH, NKS>;
+    if (int rc = set_lds(kern, Cfg::kLds)) return rc;
+    const int nrt = (R + Cfg::BM - 1) / Cfg::BM;
+    const int pairs = H * np;
+    int ngroups = (256 + nrt - 1) / nrt;
+    if (ngroups > pairs) ngroups = pairs;
+    const int ppg = (pairs + ngroups - 1) / ngroups;
+    ngroups = (pairs + ppg - 1) / ppg;
+    const int64_t grid = (int64_t)8 * ((nrt + 7) / 8) * ngroups;
+    RFA_LAUNCH(PROJECT_PHI, kern, dim3((unsigned)grid), dim3(rfa::kThreads), Cfg::kLds, st, x, pa, wf, R, H, np, ngroups,
+               ppg, scale);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
 template <int D, int DH>
 int launch_project_phi(const rfa::half_t* x, const rfa::ProjectArgs& pa, const rfa::half_t* wf, int R, int E, int H,
                        int np, float scale, hipStream_t st) {
+    if constexpr (DH == 64 && D <= 64) {
+        if (!getenv("RFA_HIP_PROJECT_STREAMING")) {
+            if (E == 128) return launch_project_rows<D, DH, 4>(x, pa, wf, R, H, np, scale, st);
+            if (E == 256) return launch_project_rows<D, DH, 8>(x, pa, wf, R, H, np, scale, st);
+            if (E == 384) return launch_project_rows<D, DH, 12>(x, pa, wf, R, H, np, scale, st);
+            if (E == 512) return launch_project_rows<D, DH, 16>(x, pa, wf, R, H, np, scale, st);
+        }
+    }
     using Cfg = rfa::ProjectCfg<D, DH>;
     auto kern = rfa::k_project_phi<D, DH>;
     if (int rc = set_lds(kern, Cfg::kLds)) return rc;

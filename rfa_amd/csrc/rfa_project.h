@@ -208,6 +208,213 @@ __global__ __launch_bounds__(kThreads) void k_project_phi(
 }
 
 // ---------------------------------------------------------------------------
+// Same computation for narrow inputs (E = 32 * NKS <= 512, DH = 64): a workgroup keeps its 128
+// rows of x in registers for its whole life -- wave w holds rows [32w, 32w + 32) as MFMA B
+// operands, 2 * NKS registers of 8 halves -- and walks a list of (head, projection) pairs whose
+// weight rows ([DH][E] each) arrive whole in a two-buffer LDS ring, one pair ahead.  No barrier
+// inside a pair's contraction or its epilogue.
+//   grid = 8 * ceil(nrt / 8) * ngroups; group g of a row tile takes pairs [g * ppg, (g + 1) * ppg)
+//   of the H * np pairs, pair index hp -> head hp / np, projection hp % np.
+// LDS: [ring: 2 x DH x (E + 8); first used to stage the x tile][staging rows of the waves][w' of the head]
+// ---------------------------------------------------------------------------
+// 16 bytes as a native vector: assignments are plain vector loads and stores (the uint4 class
+// is copied with memcpy, which keeps registers that stay in flight across loop iterations in
+// private memory)
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Orders this wave's LDS accesses for the compiler only (the hardware runs one wave's LDS
+// instructions in order); unlike a fence it does not wait for outstanding global loads/stores.
+__device__ __forceinline__ void wave_lds_order() {
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");
+}
+
+template <int D, int DH, int NKS>
+struct ProjectRowCfg {
+    static_assert(DH == 64, "one 64-wide head per pair");
+    static constexpr int BM = 128, E = 32 * NKS;
+    static constexpr int LDE = E + 8;
+    static constexpr int LDW = DH + lds_pad(DH);
+    static constexpr int LDP = (2 * D > DH ? 2 * D : DH) + 16;
+    static constexpr int kSliceHalves = DH * LDE;
+    static constexpr int SP = DH * E / 8 / kThreads;        // 16-byte pieces per thread and slice
+    static constexpr size_t kLds = (size_t)(2 * kSliceHalves + 4 * 16 * LDP + D * LDW) * 2;
+    static_assert(2 * kSliceHalves >= BM * LDE, "the x tile is staged in the ring");
+    static_assert(kLds <= 160 * 1024, "LDS budget");
+};
+
+template <int D, int DH, int NKS>
+__global__ __launch_bounds__(kThreads) void k_project_phi_rows(
+    const half_t* __restrict__ x, ProjectArgs pa, const half_t* __restrict__ wf, int R, int H, int np,
+    int ngroups, int ppg, float scale) {
+    using Cfg = ProjectRowCfg<D, DH, NKS>;
+    constexpr int BM = Cfg::BM, E = Cfg::E, LDE = Cfg::LDE, LDW = Cfg::LDW, LDP = Cfg::LDP, SP = Cfg::SP;
+    constexpr int NCT = DH / 16, PPR = E / 8;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    half_t* ring = reinterpret_cast<half_t*>(smem_raw);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int i = lane & 15, G = lane >> 4;
+    half_t* Ps = ring + 2 * Cfg::kSliceHalves + wv * 16 * LDP;
+    half_t* Wfs = ring + 2 * Cfg::kSliceHalves + 4 * 16 * LDP;
+
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int row0 = (xcd + 8 * (slot / ngroups)) * BM;
+    const int grp = slot % ngroups;
+    const int pairs = H * np;
+    const int hp_begin = grp * ppg, hp_end = min(hp_begin + ppg, pairs);
+    if (row0 >= R || hp_begin >= hp_end) return;
+    RFA_TICK_INIT();
+
+    // weight rows of pair hp: piece -> (row, 16-byte column)
+    u32x4 wr[SP];
+    auto slice_g2r = [&](int hp) {
+        const half_t* __restrict__ src = pick3(pa.w, hp % np) + (int64_t)(hp / np) * DH * E;
+#pragma unroll
+        for (int it = 0; it < SP; ++it) wr[it] = *reinterpret_cast<const u32x4*>(src + (int64_t)(tid + kThreads * it) * 8);
+    };
+    auto slice_r2s = [&](half_t* buf) {
+#pragma unroll
+        for (int it = 0; it < SP; ++it) {
+            const int pc = tid + kThreads * it;
+            *reinterpret_cast<u32x4*>(buf + (pc / PPR) * LDE + (pc % PPR) * 8) = wr[it];
+        }
+    };
+    // Workgroups of different row tiles walk their pairs in rotated order, so that the CUs of an
+    // XCD do not all ask the L2 for the same weight rows at the same time.
+    const int cnt = hp_end - hp_begin;
+    const int rot = (row0 / BM) % cnt;
+    auto pair_at = [&](int j) { return hp_begin + (j + rot) % cnt; };
+    slice_g2r(pair_at(0));
+
+    // x tile -> ring (coalesced rows) -> this wave's rows as B operands
+    {
+        constexpr int XP = BM * PPR / kThreads, BATCH = XP % 16 == 0 ? 16 : 8;
+        static_assert(XP % BATCH == 0, "x tile pieces");
+#pragma unroll
+        for (int base = 0; base < XP; base += BATCH) {
+            u32x4 v[BATCH];
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b) {
+                const int pc = tid + kThreads * (base + b);
+                const int r = min(row0 + pc / PPR, R - 1);
+                v[b] = *reinterpret_cast<const u32x4*>(x + (int64_t)r * E + (pc % PPR) * 8);
+            }
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b) {
+                const int pc = tid + kThreads * (base + b);
+                *reinterpret_cast<u32x4*>(ring + (pc / PPR) * LDE + (pc % PPR) * 8) = v[b];
+            }
+        }
+    }
+    __syncthreads();
+    h8 xb[2][NKS];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) xb[a][ks] = row8(ring, LDE, 32 * wv + 16 * a + i, 32 * ks, G);
+    __syncthreads();
+    slice_r2s(ring);
+    // wf is NULL when no projection asks for phi
+    int h_loaded = pair_at(0) / np;
+    if (wf) load_w_to_lds<D, DH>(Wfs, wf + (int64_t)h_loaded * D * DH, tid);
+    __syncthreads();
+    RFA_TICK(0);
+
+    for (int j = 0; j < cnt; ++j) {
+        const int hp = pair_at(j);
+        const int h = hp / np, p = hp % np;
+        const half_t* Ws = ring + (j & 1) * Cfg::kSliceHalves;
+        // the bias before the weight prefetch: loads return in order, and the epilogue must not
+        // have to wait for the next pair's weights to see its bias
+        const half_t* bias = pick3(pa.b, p);
+        h4 bv[NCT];
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bv[ct][e] = (half_t)0.f;
+            if (bias) bv[ct] = *reinterpret_cast<const h4*>(bias + h * DH + 16 * ct + 4 * G);
+        }
+        const int hp_next = pair_at(min(j + 1, cnt - 1));     // the last pair re-reads its own rows
+        slice_g2r(hp_next);
+
+        f4 acc[2][NCT];
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int c = 0; c < NCT; ++c) acc[a][c] = f4_zero();
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct) {
+                const h8 wa = row8(Ws, LDE, 16 * ct + i, 32 * ks, G);
+                acc[0][ct] = mfma32(wa, xb[0][ks], acc[0][ct]);
+                acc[1][ct] = mfma32(wa, xb[1][ks], acc[1][ct]);
+            }
+        RFA_TICK(1);
+
+        half_t* phi = pick3(pa.phi, p);
+        half_t* y = pick3(pa.y, p);
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            const int r0 = row0 + 32 * wv + 16 * a;
+            h8 op[DH / 32];
+            float ss = 0.f;
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct) {
+                f4 t = acc[a][ct];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) t[e] += (float)bv[ct][e];
+                const h4 yh = to_h4(t);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    ss += (float)yh[e] * (float)yh[e];
+                    op[ct / 2][4 * (ct % 2) + e] = yh[e];
+                }
+                *reinterpret_cast<h4*>(Ps + i * LDP + 16 * ct + 4 * G) = yh;
+            }
+            wave_lds_order();
+            wave_rows_s2g<DH>(Ps, LDP, y, r0, R, H, h, lane);
+            wave_lds_order();
+            if (phi) {
+                ss = sum_over_groups(ss);
+                const float inv = 1.0f / (sqrtf(ss) + 1e-3f);
+#pragma unroll
+                for (int jt = 0; jt < D / 16; ++jt) {
+                    f4 u = f4_zero();
+#pragma unroll
+                    for (int pr = 0; pr < DH / 32; ++pr)
+                        u = mfma32(row_split8(Wfs, LDW, 16 * jt + i, 32 * pr, G), op[pr], u);
+                    h4 sv, cv;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float s_, c_;
+                        fast_sincos(u[e] * inv, s_, c_);
+                        sv[e] = (half_t)(scale * s_);
+                        cv[e] = (half_t)(scale * c_);
+                    }
+                    *reinterpret_cast<h4*>(Ps + i * LDP + 16 * jt + 4 * G) = sv;
+                    *reinterpret_cast<h4*>(Ps + i * LDP + D + 16 * jt + 4 * G) = cv;
+                }
+                wave_lds_order();
+                wave_rows_s2g<2 * D>(Ps, LDP, phi, r0, R, H, h, lane);
+                wave_lds_order();
+            }
+        }
+        RFA_TICK(2);
+        __syncthreads();                              // everyone is done with this pair's buffer and w'
+        const int h_next = hp_next / np;
+        if (h_next != h_loaded) {
+            h_loaded = h_next;
+            if (wf) load_w_to_lds<D, DH>(Wfs, wf + (int64_t)h_next * D * DH, tid);
+        }
+        slice_r2s(ring + ((j + 1) & 1) * Cfg::kSliceHalves);
+        __syncthreads();
+        RFA_TICK(3);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Weight and bias gradients of those Linear layers:
 //     dW_p[o][c] = sum_r dy_p[r][o] * x[r][c],      db_p[o] = sum_r dy_p[r][o]
 // (what autograd computes for torch.nn.Linear).  The contraction runs over the R rows, far

@@ -109,3 +109,34 @@ def project_heads(x: Tensor, layers: Sequence[nn.Linear], want_phi: Sequence[boo
     for layer in layers:
         params += [layer.weight, layer.bias]
     return _ProjectHeads.apply(x, w_feat, scale, heads, tuple(bool(f) for f in want_phi), *params)
+
+
+class _LinearOut(torch.autograd.Function):
+    """y = x W^T + b with the library GEMM forward and the row-split weight/bias-gradient kernel
+    backward (the library's choice for dy^T x with a long row count is several times slower)."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, weight: Tensor, bias: Optional[Tensor]):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, dy: Tensor):
+        x, weight = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1])
+        x2 = x.reshape(-1, x.shape[-1])
+        dx = torch.mm(dy2, weight).view(x.shape) if ctx.needs_input_grad[0] else None
+        dws, dbs = linear_param_grads(x2, [dy2], [ctx.has_bias])
+        return dx, dws[0], dbs[0]
+
+
+def linear_out(x: Tensor, layer: nn.Linear) -> Tensor:
+    """``layer(x)`` (the modules' out_proj, causal_attention.py:278, cross_attention.py:298); fp16 HIP
+    tensors with widths that are multiples of 128 take the row-split gradient kernel in backward."""
+    w = layer.weight
+    if (x.is_cuda and x.dtype == torch.float16 and w.dtype == torch.float16 and torch.is_grad_enabled()
+            and (w.requires_grad or x.requires_grad) and rfa_hip.linear_weight_grad_supported(*w.shape)
+            and (layer.bias is None or layer.bias.dtype == torch.float16)):
+        return _LinearOut.apply(x, w, layer.bias)
+    return layer(x)

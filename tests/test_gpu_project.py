@@ -15,7 +15,7 @@ from oracle import rfa_oracle as O
 pytestmark = pytest.mark.gpu
 
 # L, B, E, H, d, D
-SHAPES = [(128, 2, 256, 4, 64, 64), (70, 3, 128, 2, 64, 64), (33, 1, 256, 2, 128, 128), (5, 2, 64, 1, 64, 32),
+SHAPES = [(128, 2, 256, 4, 64, 64), (300, 2, 512, 8, 64, 64), (70, 3, 128, 2, 64, 64), (33, 1, 256, 2, 128, 128), (5, 2, 64, 1, 64, 32),
           (1, 1, 192, 3, 64, 128), (257, 1, 128, 1, 128, 64)]
 
 
@@ -38,9 +38,16 @@ def _linear64(x, w, b, H, d):
     return y.view(*x.shape[:2], H, d)
 
 
+@pytest.mark.parametrize("streaming", [False, True])
 @pytest.mark.parametrize("L,B,E,H,d,D", SHAPES)
-def test_qkv_projection_with_feature_map(L, B, E, H, d, D):
+def test_qkv_projection_with_feature_map(L, B, E, H, d, D, streaming, monkeypatch):
+    """Both kernels: the one that keeps its rows of x in LDS (picked when they fit) and the one
+    that streams x and the weights together (forced by RFA_HIP_PROJECT_STREAMING)."""
     from rfa_amd import rfa_hip
+    if streaming:
+        monkeypatch.setenv("RFA_HIP_PROJECT_STREAMING", "1")
+    else:
+        monkeypatch.delenv("RFA_HIP_PROJECT_STREAMING", raising=False)
     x, ws, bs = _inputs(L, B, E, H, d, 900 + L, 3)
     bs[1] = None                                       # one projection without bias
     wf = (_randn(H, D, d, seed=77) * 0.9).half()
@@ -181,3 +188,93 @@ def test_linear_weight_and_bias_gradients(R, Eo, Ei, n):
             assert dbs[p] is None
     with pytest.raises(ValueError):
         rfa_hip.linear_weight_grad(x[:, :64].contiguous().cuda(), [d.cuda() for d in dys], want_bias)
+
+
+def test_cross_modules_fused_projections_match_unfused_chain():
+    """CrossAttentionProjectLayer + CrossAttention with their projections on the fused launch vs
+    the same modules on nn.Linear + random_project: output within 4e-3, gradients within 1e-2."""
+    from rfa_amd import CrossAttention, CrossAttentionProjectLayer
+    torch.manual_seed(6)
+    S, T, B, E, H, d, D = 150, 70, 2, 256, 4, 64, 64
+    proj = CrossAttentionProjectLayer(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half()
+    att = CrossAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half()
+    with torch.no_grad():
+        proj.sigma.mul_(1.0 + 0.1 * torch.randn_like(proj.sigma))
+        att.q_proj.bias.normal_(0, 0.1)
+    W = O.make_w(d, D, H).cuda().half()
+    enc0 = (torch.randn(S, B, E) * 0.7).half()
+    q0 = (torch.randn(T, B, E) * 0.7).half()
+    go = torch.randn(T, B, E).half().cuda()
+    mask = torch.zeros(S, B, 1, 1, dtype=torch.bool)
+    mask[120:, 1] = True
+    mask = mask.cuda()
+
+    def run(fused):
+        proj.fuse_projections = att.fuse_projections = fused
+        proj.zero_grad(set_to_none=True)
+        att.zero_grad(set_to_none=True)
+        enc = enc0.clone().cuda().requires_grad_(True)
+        q = q0.clone().cuda().requires_grad_(True)
+        y = att(q, proj(encoder_output=enc, random_matrices=W, mask=mask))
+        y.backward(go)
+        grads = {"enc": enc.grad, "q": q.grad}
+        grads.update({"proj." + n: p.grad for n, p in proj.named_parameters()})
+        grads.update({"att." + n: p.grad for n, p in att.named_parameters()})
+        return y.detach().float().cpu(), {k: v.float().cpu() for k, v in grads.items()}
+
+    y_f, g_f = run(True)
+    y_u, g_u = run(False)
+    assert (y_f - y_u).abs().max().item() <= 4e-3
+    for name in g_u:
+        r = ((g_f[name] - g_u[name]).norm() / g_u[name].norm().clamp_min(1e-30)).item()
+        assert torch.isfinite(g_f[name]).all() and r <= 1e-2, (name, r)
+
+
+def test_module_step_replays_from_a_hip_graph():
+    """Forward + backward of CausalAttention captured once and replayed: every replay, with eager
+    steps and synchronisations in between, gives bit-identical output and gradients to the eager step."""
+    from rfa_amd import CausalAttention
+    torch.manual_seed(7)
+    T, B, E, H, d, D = 320, 2, 256, 4, 64, 64
+    m = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half()
+    W = O.make_w(d, D, H).cuda().half()
+    x = (torch.randn(T, B, E) * 0.6).half().cuda().requires_grad_(True)
+    go = torch.randn(T, B, E).half().cuda()
+
+    def step():
+        m.zero_grad(set_to_none=True)
+        x.grad = None
+        y = m(x, W)
+        y.backward(go)
+        return y
+
+    y_e = step().detach().clone()
+    want = {"x": x.grad.detach().clone(), **{n: p.grad.detach().clone() for n, p in m.named_parameters()}}
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    m.zero_grad(set_to_none=True)
+    x.grad = None
+    with torch.cuda.graph(graph):
+        y_g = m(x, W)
+        y_g.backward(go)
+    captured = {"x": x.grad, **{n: p.grad for n, p in m.named_parameters()}}   # the graph's output buffers
+    for rep in range(3):
+        for t in captured.values():
+            t.zero_()
+        y_g.detach().zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_g, y_e), rep
+        for name, t in captured.items():
+            assert torch.equal(t, want[name]), (rep, name)
+        # eager work between the replays; it rebinds .grad, the graph keeps writing its own buffers
+        grads_before = {k: v for k, v in captured.items()}
+        step()
+        torch.cuda.synchronize()
+        captured = grads_before
