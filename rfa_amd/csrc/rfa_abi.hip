@@ -41,13 +41,13 @@ int fail(int code, const char* fmt, ...) {
 // ---- optional per-kernel timing with HIP events ------------------------------------
 namespace prof {
 enum Id { SEG_STATE, CAUSAL_FWD, CAUSAL_BWD_DQ, CAUSAL_BWD_DKDV, CROSS_READOUT, CROSS_READOUT_BWD,
-          CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, MASKED_FWD, MASKED_PREP, MASKED_DQ, MASKED_DKDV, PROJECT_PHI, WGRAD_PARTIAL, WGRAD_REDUCE, ZERO_FILL,
+          CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, MASKED_FWD, MASKED_PREP, MASKED_DQ, MASKED_DKDV, PROJECT_PHI, WGRAD_PARTIAL, WGRAD_REDUCE, TOTALS_SCAN, ZERO_FILL,
           SELFTEST, COUNT };
 const char* const kNames[COUNT] = {"k_segment_state", "k_causal_fwd", "k_causal_bwd_dq", "k_causal_bwd_dkdv",
                                    "k_cross_readout", "k_cross_readout_bwd", "k_cross_state_bwd", "k_decode_step",
                                    "k_feature_map_fwd", "k_feature_map_bwd", "k_feature_map_dw_reduce",
                                    "k_masked_fwd", "k_masked_bwd_prep", "k_masked_dq", "k_masked_dkdv", "k_project_phi",
-                                   "k_weight_grad_partial", "k_weight_grad_reduce",
+                                   "k_weight_grad_partial", "k_weight_grad_reduce", "k_totals_scan",
                                    "k_zero_f32", "k_selftest"};
 struct Rec { int id; hipEvent_t a, b; };
 std::mutex mu;
@@ -157,6 +157,23 @@ int set_lds(Kern kern, size_t bytes) {
     return RFA_OK;
 }
 
+// Whether the consumers read one pre-scanned state (k_totals_scan) instead of adding up the
+// segment totals themselves, (nseg - 1) / 2 states of K * d floats on average per workgroup:
+// worth its pass over the totals from 128 KiB of such reads on.
+// RFA_HIP_PREFIX=0/1 overrides (the forward and the backward of a saved pair must agree).
+bool use_scanned_totals(int nseg, int K, int d) {
+    if (nseg < 2) return false;
+    if (const char* env = getenv("RFA_HIP_PREFIX")) return env[0] == '1';
+    return (int64_t)(nseg - 1) * K * d * 2 >= 128 * 1024;
+}
+
+template <bool REVERSE>
+void launch_totals_scan(float* a, int64_t Ma, float* b, int64_t Mb, int N, int nseg, hipStream_t st) {
+    const int64_t threads = (Ma + Mb) / 4;
+    RFA_LAUNCH(TOTALS_SCAN, rfa::k_totals_scan<REVERSE>, dim3((unsigned)((threads + 255) / 256), (unsigned)N),
+               dim3(rfa::kThreads), 0, st, a, Ma, b, Mb, nseg);
+}
+
 template <int KD, int DH>
 int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, rfa::half_t* out,
                    int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, float* savedS, float* savedZ,
@@ -176,16 +193,18 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(64 * NW), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
+    const int prefixed = use_scanned_totals(p.nseg, KD, DH) ? 1 : 0;
+    if (prefixed) launch_totals_scan<false>(wsS, (int64_t)KD * DH, wsZ, KD, N, p.nseg, st);
     if constexpr (PIPE) {
         auto kern = rfa::k_causal_fwd_pipe<KD, DH>;
         if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(512), rfa::FwdPipeCfg<KD, DH>::kLds, st, q, k, v, out,
-                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len);
+                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, prefixed);
     } else {
         auto kern = rfa::k_causal_fwd<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q, k, v, out,
-                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len);
+                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, prefixed);
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -194,8 +213,22 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
 template <int KD, int DH>
 int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v,
                     const rfa::half_t* g, const rfa::half_t* out, rfa::half_t* dq, rfa::half_t* dk,
-                    rfa::half_t* dv, int T, int N, const ScanPlan& p, char* ws, const Workspace& wl,
+                    rfa::half_t* dv, int T, int N, const ScanPlan& pf, char* ws, const Workspace& wl,
                     const float* savedS, const float* savedZ, const float* savedDen, hipStream_t st) {
+    // pf is the forward's cut into segments (that of the saved totals).  Where both sweeps run as two
+    // workgroups per (sequence, segment) and the totals are scanned, the backward takes segments
+    // twice as long: half as many workgroups already cover the CUs, in one round instead of two.
+    ScanPlan p = pf;
+    const int prefixed_s = use_scanned_totals(pf.nseg, KD, DH) ? 1 : 0;
+    int s_ratio = 1;
+    if constexpr (KD >= 256 && DH >= 128) {
+        if (savedS && prefixed_s && pf.nseg >= 4 && pf.nseg % 2 == 0 && !getenv("RFA_HIP_NSEG_SAME")) {
+            p.nseg = pf.nseg / 2;
+            p.seg_len = 2 * pf.seg_len;
+            s_ratio = 2;
+        }
+    }
+    const int prefixed = (s_ratio == 1) ? prefixed_s : (use_scanned_totals(p.nseg, KD, DH) ? 1 : 0);   // of dR, dr
     constexpr int NW = causal_waves(KD, DH);
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
@@ -206,7 +239,7 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
     float* gz = reinterpret_cast<float*>(ws + wl.gz);
     const float* inS = wsS;
     const float* inZ = wsZ;
-    if (savedS) {          // segment totals handed over by the forward pass
+    if (savedS) {          // segment totals handed over by the forward pass (already scanned if prefixed_s)
         inS = savedS;
         inZ = savedZ;
     } else if (p.nseg > 1) {
@@ -214,6 +247,7 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         if (int rc = set_lds(kern, Cfg::kSegStateLds)) return rc;
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(64 * NW), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
+        if (prefixed_s) launch_totals_scan<false>(wsS, (int64_t)KD * DH, wsZ, KD, N, p.nseg, st);
     }
     const float* den_in = den;
     if (savedDen) {
@@ -227,14 +261,14 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
             auto kern = rfa::k_causal_bwd_dq_saved<KL, DH, NWQ, fwd_state_waves_v<KD, DH>, KD>;
             if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
             RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(2 * N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g,
-                       out, savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len);
+                       out, savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len, prefixed_s, pf.nseg, s_ratio);
         } else {
             constexpr int NWQ = dq_waves(KD, DH);
             using CfgQ = rfa::CausalCfg<KD, DH, NWQ>;
             auto kern = rfa::k_causal_bwd_dq_saved<KD, DH, NWQ, fwd_state_waves_v<KD, DH>>;
             if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
             RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g, out,
-                       savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len);
+                       savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len, prefixed_s, pf.nseg, s_ratio);
         }
         den_in = savedDen;
     } else {
@@ -243,8 +277,10 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         auto kern = rfa::k_causal_bwd_dq<KD, DH, NWQ, true>;
         if (int rc = set_lds(kern, CfgQ::kBwdDqLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqLds, st, q, k, v, g,
-                           dq, inS, inZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len);
+                           dq, inS, inZ, wsR, wsr, den, gz, T, N, p.nseg, p.seg_len, prefixed_s);
     }
+    // the dQ sweep left the totals of dR, dr of segments 1 .. nseg - 1
+    if (prefixed) launch_totals_scan<true>(wsR, (int64_t)KD * DH, wsr, KD, N, p.nseg, st);
     if constexpr (KD >= 256) {
         // two copies of R in one workgroup would not fit the register file: dK and dV in separate
         // workgroups (one copy each); measured 2.5x (d = 64) and 1.7x (d = 128) faster at K = 256,
@@ -254,7 +290,7 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         auto kern = rfa::k_causal_bwd_dkdv_roles<KD, DH, NWR>;
         if (int rc = set_lds(kern, CfgR::kLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(2 * N * p.nseg), dim3(64 * NWR), CfgR::kLds, st, q, k, v, g, dk, dv,
-                   (const float*)wsR, (const float*)wsr, den_in, (const float*)gz, T, N, p.nseg, p.seg_len);
+                   (const float*)wsR, (const float*)wsr, den_in, (const float*)gz, T, N, p.nseg, p.seg_len, prefixed);
     } else
     if constexpr (NW == 4 && KD <= 128) {
         // 8 waves with the state phase split by role (dK waves / dV waves): two waves per SIMD
@@ -263,12 +299,12 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         auto kern = rfa::k_causal_bwd_dkdv<KD, DH, 8, true, true>;
         if (int rc = set_lds(kern, CfgK::kBwdDkLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(512), CfgK::kBwdDkLds, st, q, k, v, g,
-                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
+                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len, prefixed);
     } else {
         auto kern = rfa::k_causal_bwd_dkdv<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDkLds, st, q, k, v, g,
-                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len);
+                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len, prefixed);
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -320,7 +356,7 @@ int launch_cross_readout(const rfa::half_t* q, const float* s, const float* z, r
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
     RFA_LAUNCH(CROSS_READOUT, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q,
                        (const rfa::half_t*)nullptr, (const rfa::half_t*)nullptr, out, s, z, (float*)nullptr,
-                       (float*)nullptr, (float*)nullptr, T, N, p.nseg, p.seg_len);
+                       (float*)nullptr, (float*)nullptr, T, N, p.nseg, p.seg_len, 0);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -335,7 +371,7 @@ int launch_cross_readout_bwd(const rfa::half_t* q, const float* s, const float* 
     if (int rc = set_lds(kern, Cfg::kBwdDqLds)) return rc;
     RFA_LAUNCH(CROSS_READOUT_BWD, kern, dim3(N), dim3(64 * NW), Cfg::kBwdDqLds, st, q, (const rfa::half_t*)nullptr,
                        (const rfa::half_t*)nullptr, g, dq, s, z, ds, dz, (float*)nullptr, (float*)nullptr, T, N,
-                       1, seg_len);
+                       1, seg_len, 0);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -351,7 +387,7 @@ int launch_cross_state_bwd(const rfa::half_t* k, const rfa::half_t* v, const uin
     if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
     RFA_LAUNCH(CROSS_STATE_BWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDkLds, st,
                        (const rfa::half_t*)nullptr, k, v, (const rfa::half_t*)nullptr, dk, dv, ds, dz,
-                       (const float*)nullptr, (const float*)nullptr, mask, H, T, N, p.nseg, p.seg_len);
+                       (const float*)nullptr, (const float*)nullptr, mask, H, T, N, p.nseg, p.seg_len, 0);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }

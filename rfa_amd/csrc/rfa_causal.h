@@ -214,7 +214,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
     float* __restrict__ den_out, float* __restrict__ final_s, float* __restrict__ final_z, int T, int N,
-    int nseg, int seg_len) {
+    int nseg, int seg_len, int prefixed) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = Cfg::DS;
@@ -262,9 +262,11 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
 #pragma unroll
     for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
     const h8 ones = h8_ones();
-    const int n_states = CAUSAL ? seg : 1;          // states to sum
+    // states to sum: every earlier segment's total, or the one exclusive prefix k_totals_scan left
+    const int s_begin = (CAUSAL && prefixed) ? seg : 0;
+    const int n_states = CAUSAL ? (prefixed ? seg + 1 : seg) : 1;
     const int state_stride = CAUSAL ? nseg : 1;     // states stored per sequence
-    for (int s = 0; s < n_states; ++s) {
+    for (int s = s_begin; s < n_states; ++s) {
         const float* si = wsS + ((int64_t)(n * state_stride + s) * KD) * DH;
         if (CAUSAL) {
             const f4* sf = reinterpret_cast<const f4*>(si) + (int64_t)w * NKT * NCT * 64;
@@ -490,7 +492,7 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
     float* __restrict__ den_out, float* __restrict__ final_s, float* __restrict__ final_z, int T, int N,
-    int nseg, int seg_len) {
+    int nseg, int seg_len, int prefixed) {
     using Cfg = FwdPipeCfg<KD, DH>;
     constexpr int NT = 256;      // threads per group
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = DH / 4;
@@ -527,7 +529,7 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
         f4 zacc[NKTW];      // z for feature tiles kt = w*NKTW + a, element k = 16kt + 4G + e
 #pragma unroll
         for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
-        for (int s = 0; s < seg; ++s) {
+        for (int s = prefixed ? seg : 0; s < (prefixed ? seg + 1 : seg); ++s) {
 #pragma unroll
             for (int a = 0; a < NKTW; ++a)
                 zacc[a] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * nseg + s) * KD + 16 * (w * NKTW + a) + 4 * G);
@@ -629,7 +631,7 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
         for (int a = 0; a < NKT; ++a)
 #pragma unroll
             for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
-        for (int s = 0; s < seg; ++s) {
+        for (int s = prefixed ? seg : 0; s < (prefixed ? seg + 1 : seg); ++s) {
             const f4* sf = reinterpret_cast<const f4*>(wsS + ((int64_t)(n * nseg + s) * KD) * DH) + (int64_t)w * NKT * NCT * 64;
 #pragma unroll
             for (int kt = 0; kt < NKT; ++kt)
@@ -742,7 +744,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, half_t* __restrict__ dq, const float* __restrict__ wsS,
     const float* __restrict__ wsZ, float* __restrict__ wsR, float* __restrict__ wsr,
-    float* __restrict__ den_ws, float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len) {
+    float* __restrict__ den_ws, float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len, int prefixed) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS;
@@ -786,9 +788,10 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
 #pragma unroll
     for (int b = 0; b < NKT; ++b) { zacc[b] = f4_zero(); racc[b] = f4_zero(); }
     const h8 ones = h8_ones();
-    const int n_states = CAUSAL ? seg : 1;
+    const int s_begin = (CAUSAL && prefixed) ? seg : 0;
+    const int n_states = CAUSAL ? (prefixed ? seg + 1 : seg) : 1;
     const int state_stride = CAUSAL ? nseg : 1;
-    for (int s = 0; s < n_states; ++s) {
+    for (int s = s_begin; s < n_states; ++s) {
         const float* si = wsS + ((int64_t)(n * state_stride + s) * KD) * DH;
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct)
@@ -1078,7 +1081,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     const half_t* __restrict__ g, const half_t* __restrict__ o, const float* __restrict__ den_raw,
     half_t* __restrict__ dq, const float* __restrict__ wsS, const float* __restrict__ wsZ,
     float* __restrict__ wsR, float* __restrict__ wsr, float* __restrict__ gz_ws, int T, int N, int nseg,
-    int seg_len) {
+    int seg_len, int prefixed, int s_nseg, int s_ratio) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS;
@@ -1129,9 +1132,12 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     // in (k_segment_state<FRAG = true> for NWF waves: [wave][kt][ct][lane][4], element
     // (k = 16kt + 4G + e, c = wave*DSF + 16ct + i)); this wave needs (c = 16ct + 4G + e,
     // k = w*KS + 16kt + row), i.e. four scalar loads per tile, once per workgroup.
+    // The forward may have cut the sequence into s_ratio times as many segments as this sweep
+    // (s_nseg per sequence; only with scanned totals, where slot seg * s_ratio is the state at
+    // this segment's first step).
     constexpr int DSF = DH / NWF, NCTF = DSF / 16, NKTF = KDG / 16;
-    for (int s = 0; s < seg; ++s) {
-        const float* si = wsS + ((int64_t)(n * nseg + s) * KDG) * DH;
+    for (int s = prefixed ? seg : 0; s < (prefixed ? seg + 1 : seg); ++s) {
+        const float* si = wsS + ((int64_t)(n * s_nseg + s * s_ratio) * KDG) * DH;
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct) {
             const int wf = (16 * ct) / DSF, ctf = ((16 * ct) % DSF) / 16;
@@ -1145,7 +1151,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
         }
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
-            zacc[kt] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * nseg + s) * KDG + koff + w * KS + 16 * kt + 4 * G);
+            zacc[kt] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * s_nseg + s * s_ratio) * KDG + koff + w * KS + 16 * kt + 4 * G);
     }
 
     RFA_TICK_INIT();
@@ -1352,7 +1358,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     const half_t* __restrict__ g, half_t* __restrict__ dk, half_t* __restrict__ dv,
     const float* __restrict__ wsR, const float* __restrict__ wsr, const float* __restrict__ den_ws,
     const float* __restrict__ gz_ws, const uint8_t* __restrict__ pad_mask, int H, int T, int N,
-    int nseg, int seg_len) {
+    int nseg, int seg_len, int prefixed) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     static_assert(!SPLIT || NW == 8, "the role split needs 8 waves");
@@ -1402,7 +1408,8 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
 #pragma unroll
     for (int b = 0; b < NKT; ++b) racc[b] = f4_zero();
     const uint8_t* mrow = (!CAUSAL && pad_mask) ? pad_mask + (int64_t)(n / H) * T : nullptr;
-    const int s_first = CAUSAL ? seg + 1 : 0, s_last = CAUSAL ? nseg : 1;
+    // later segments' totals, or the one exclusive suffix k_totals_scan left
+    const int s_first = CAUSAL ? (prefixed ? seg : seg + 1) : 0, s_last = CAUSAL ? (prefixed ? seg + 1 : nseg) : 1;
     const int state_stride = CAUSAL ? nseg : 1;
     for (int s = s_first; s < s_last; ++s) {
         const float* ri = wsR + ((int64_t)(n * state_stride + s) * KD) * DH;
@@ -1668,7 +1675,7 @@ __device__ __forceinline__ void dkdv_role_dk(
     unsigned char* smem_raw, int bid, const half_t* __restrict__ q, const half_t* __restrict__ v,
     const half_t* __restrict__ g, half_t* __restrict__ dk, const float* __restrict__ wsR,
     const float* __restrict__ wsr, const float* __restrict__ den_ws, const float* __restrict__ gz_ws, int T,
-    int N, int nseg, int seg_len) {
+    int N, int nseg, int seg_len, int prefixed) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = KD / NW;
@@ -1703,7 +1710,7 @@ __device__ __forceinline__ void dkdv_role_dk(
     f4 racc[NKT];
 #pragma unroll
     for (int b = 0; b < NKT; ++b) racc[b] = f4_zero();
-    for (int s = seg + 1; s < nseg; ++s) {
+    for (int s = prefixed ? seg : seg + 1; s < (prefixed ? seg + 1 : nseg); ++s) {
         const float* ri = wsR + ((int64_t)(n * nseg + s) * KD) * DH;
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct)
@@ -1843,7 +1850,7 @@ template <int KD, int DH, int NW>
 __device__ __forceinline__ void dkdv_role_dv(
     unsigned char* smem_raw, int bid, const half_t* __restrict__ q, const half_t* __restrict__ k,
     const half_t* __restrict__ g, half_t* __restrict__ dv, const float* __restrict__ wsR,
-    const float* __restrict__ den_ws, int T, int N, int nseg, int seg_len) {
+    const float* __restrict__ den_ws, int T, int N, int nseg, int seg_len, int prefixed) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = DH / NW;
@@ -1873,7 +1880,7 @@ __device__ __forceinline__ void dkdv_role_dv(
     for (int a = 0; a < NKT2; ++a)
 #pragma unroll
         for (int b = 0; b < NCT2; ++b) RR[a][b] = f4_zero();
-    for (int s = seg + 1; s < nseg; ++s) {
+    for (int s = prefixed ? seg : seg + 1; s < (prefixed ? seg + 1 : nseg); ++s) {
         const float* ri = wsR + ((int64_t)(n * nseg + s) * KD) * DH;
 #pragma unroll
         for (int kt = 0; kt < NKT2; ++kt)
@@ -1995,13 +2002,67 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv_roles(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, half_t* __restrict__ dk, half_t* __restrict__ dv,
     const float* __restrict__ wsR, const float* __restrict__ wsr, const float* __restrict__ den_ws,
-    const float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len) {
+    const float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len, int prefixed) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int nsq = N * nseg;
     if ((int)blockIdx.x < nsq)
-        dkdv_role_dk<KD, DH, NW>(smem_raw, blockIdx.x, q, v, g, dk, wsR, wsr, den_ws, gz_ws, T, N, nseg, seg_len);
+        dkdv_role_dk<KD, DH, NW>(smem_raw, blockIdx.x, q, v, g, dk, wsR, wsr, den_ws, gz_ws, T, N, nseg, seg_len, prefixed);
     else
-        dkdv_role_dv<KD, DH, NW>(smem_raw, blockIdx.x - nsq, q, k, g, dv, wsR, den_ws, T, N, nseg, seg_len);
+        dkdv_role_dv<KD, DH, NW>(smem_raw, blockIdx.x - nsq, q, k, g, dv, wsR, den_ws, T, N, nseg, seg_len, prefixed);
+}
+
+// ---------------------------------------------------------------------------
+// Exclusive scan of the segment totals over the segment axis, in place.  A consumer of segment
+// s otherwise adds up the totals of every earlier (forward sweeps) or later (reverse sweep)
+// segment itself, (nseg - 1) / 2 state reads on average per workgroup; with many segments of a
+// large state one pass over the totals is cheaper.
+//   a [N][nseg][Ma], b [N][nseg][Mb] fp32 (Ma, Mb multiples of 4; b may be NULL)
+//   REVERSE = false: slot s <- sum of slots s' < s; slot nseg - 1 is never read (no total is
+//                    stored for the last segment)
+//   REVERSE = true : slot s <- sum of slots s' > s; slot 0 is never read
+// grid = (ceil((Ma + Mb) / 4 / 256), N); one thread owns four consecutive elements of every slot.
+// ---------------------------------------------------------------------------
+constexpr int kMaxSegments = 16;
+
+template <bool REVERSE>
+__global__ __launch_bounds__(kThreads) void k_totals_scan(float* __restrict__ a, int64_t Ma, float* __restrict__ b,
+                                                          int64_t Mb, int nseg) {
+    int64_t e = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 4;
+    float* base;
+    int64_t M;
+    if (e < Ma) {
+        base = a; M = Ma;
+    } else {
+        e -= Ma;
+        if (!b || e >= Mb) return;
+        base = b; M = Mb;
+    }
+    float* col = base + (int64_t)blockIdx.y * nseg * M + e;
+    f4 t[kMaxSegments];
+#pragma unroll
+    for (int s = 0; s < kMaxSegments; ++s) {
+        const bool live = REVERSE ? (s >= 1 && s < nseg) : (s < nseg - 1);
+        t[s] = f4_zero();
+        if (live) t[s] = *reinterpret_cast<const f4*>(col + (int64_t)s * M);
+    }
+    f4 run = f4_zero();
+    if (REVERSE) {
+#pragma unroll
+        for (int s = kMaxSegments - 1; s >= 0; --s) {
+            if (s < nseg) {
+                *reinterpret_cast<f4*>(col + (int64_t)s * M) = run;
+                run[0] += t[s][0]; run[1] += t[s][1]; run[2] += t[s][2]; run[3] += t[s][3];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < kMaxSegments; ++s) {
+            if (s < nseg) {
+                *reinterpret_cast<f4*>(col + (int64_t)s * M) = run;
+                run[0] += t[s][0]; run[1] += t[s][1]; run[2] += t[s][2]; run[3] += t[s][3];
+            }
+        }
+    }
 }
 
 }  // namespace rfa

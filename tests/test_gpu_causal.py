@@ -128,17 +128,24 @@ def test_saved_pair_clamped_and_unclamped_rows():
             assert _rel(a, b) <= GRAD_RTOL, (scale, name, _rel(a, b))
 
 
-@pytest.mark.parametrize("nseg", [1, 2, 3, 8, 16])
-def test_every_segment_count_gives_the_same_answer(nseg, monkeypatch):
+@pytest.mark.parametrize("nseg,scanned", [(1, None), (2, None), (3, None), (8, None), (16, None),
+                                          (2, "1"), (3, "1"), (11, "1"), (8, "0"), (1, "1")])
+def test_every_segment_count_gives_the_same_answer(nseg, scanned, monkeypatch):
     """RFA_HIP_NSEG overrides the number of time segments per sequence; the plain pair, the
     saved pair and the prefill state must meet the oracle for any of them (ragged last segment,
-    single-chunk segments, one segment for the whole sequence)."""
+    single-chunk segments, one segment for the whole sequence).  RFA_HIP_PREFIX forces the
+    consumers to add up the segment totals themselves ("0") or to read totals that a scan
+    kernel turned into running sums first ("1"); unset, five segments or more take the scan."""
     from rfa_amd import rfa_hip
     monkeypatch.setenv("RFA_HIP_NSEG", str(nseg))
+    if scanned is None:
+        monkeypatch.delenv("RFA_HIP_PREFIX", raising=False)
+    else:
+        monkeypatch.setenv("RFA_HIP_PREFIX", scanned)
     T, B, H, d, D = 700, 1, 3, 64, 64
     cpu = _features(T, B, H, d, D, seed=5000)
     pq, pk, v, g = (t.cuda() for t in cpu)
-    print(f"causal nseg={nseg} T={T}", flush=True)
+    print(f"causal nseg={nseg} scanned={scanned} T={T}", flush=True)
     ref = _oracle_fwd(*cpu[:3])
     want = _oracle_bwd(*cpu)
     out, saved = rfa_hip.forward_save(pq, pk, v)
@@ -151,3 +158,28 @@ def test_every_segment_count_gives_the_same_answer(nseg, monkeypatch):
     assert torch.equal(o2, out)
     _, s_ref, z_ref = O.causal_forward_loop(cpu[0].float(), cpu[1].float(), cpu[2].float())
     assert _rel(s.cpu(), s_ref) < 1e-5 and _rel(z.cpu(), z_ref) < 1e-5
+
+
+@pytest.mark.parametrize("nseg,same", [(8, False), (4, False), (6, False), (8, True), (5, False)])
+def test_wide_state_backward_on_half_as_many_segments(nseg, same, monkeypatch):
+    """K = 256, d = 128: with scanned totals the saved-pair backward runs on segments twice as long
+    as the forward's (even segment counts; RFA_HIP_NSEG_SAME keeps them equal); out and gradients
+    must meet the oracle either way, and the plain pair as well."""
+    from rfa_amd import rfa_hip
+    monkeypatch.setenv("RFA_HIP_NSEG", str(nseg))
+    monkeypatch.delenv("RFA_HIP_PREFIX", raising=False)
+    if same:
+        monkeypatch.setenv("RFA_HIP_NSEG_SAME", "1")
+    else:
+        monkeypatch.delenv("RFA_HIP_NSEG_SAME", raising=False)
+    T, B, H, d, D = 1100, 1, 2, 128, 128
+    cpu = _features(T, B, H, d, D, seed=5100)
+    pq, pk, v, g = (t.cuda() for t in cpu)
+    print(f"causal wide nseg={nseg} same={same} T={T}", flush=True)
+    ref = _oracle_fwd(*cpu[:3])
+    want = _oracle_bwd(*cpu)
+    out, saved = rfa_hip.forward_save(pq, pk, v)
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_ATOL
+    for pair in (rfa_hip.backward_saved(pq, pk, v, g, out, saved), rfa_hip.backward(pq, pk, v, g)):
+        for name, a, b in zip(("dq", "dk", "dv"), pair, want):
+            assert _rel(a.float().cpu(), b) <= GRAD_RTOL, (nseg, name)
