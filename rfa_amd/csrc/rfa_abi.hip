@@ -364,7 +364,7 @@ int launch_cross_readout(const rfa::half_t* q, const float* s, const float* z, r
 template <int KD, int DH>
 int launch_cross_readout_bwd(const rfa::half_t* q, const float* s, const float* z, const rfa::half_t* g,
                              rfa::half_t* dq, float* ds, float* dz, int T, int N, hipStream_t st) {
-    constexpr int NW = causal_waves(KD, DH);
+    constexpr int NW = dq_waves(KD, DH);
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     const int seg_len = ((T + rfa::kChunk - 1) / rfa::kChunk) * rfa::kChunk;
     auto kern = rfa::k_causal_bwd_dq<KD, DH, NW, false>;
@@ -380,7 +380,7 @@ template <int KD, int DH>
 int launch_cross_state_bwd(const rfa::half_t* k, const rfa::half_t* v, const uint8_t* mask, int H,
                            const float* ds, const float* dz, rfa::half_t* dk, rfa::half_t* dv, int T, int N,
                            hipStream_t st) {
-    constexpr int NW = causal_waves(KD, DH);
+    constexpr int NW = causal_waves(KD, DH);    // the 8-wave role split of the causal sweep measured slower here
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     const ScanPlan p = make_free_plan(T, N);
     auto kern = rfa::k_causal_bwd_dkdv<KD, DH, NW, false>;
