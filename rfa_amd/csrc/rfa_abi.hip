@@ -512,7 +512,7 @@ WGradPlan make_wgrad_plan(int64_t R, int Eo, int Ei, int np) {
 // ---- feature map launchers ---------------------------------------------------------
 int feature_bwd_blocks(int64_t R, int H) {
     const int64_t nrb = (R + 63) / 64;
-    int64_t nblk = (256 + H - 1) / H;   // about one workgroup per CU; few partial sums to reduce
+    int64_t nblk = (512 + H - 1) / H;   // about two workgroups per CU; few partial sums to reduce
     if (nblk > nrb) nblk = nrb;
     if (nblk < 1) nblk = 1;
     return (int)nblk;
