@@ -17,22 +17,49 @@ from torch import Tensor
 from . import _lib
 
 
-def _require(cond: bool, exc, msg: str):
+def _require(cond: bool, exc, msg):
+    # msg is a callable so that the text is only built when the check fails
     if not cond:
-        raise exc(msg)
+        raise exc(msg())
 
 
 def _check_half_cuda(name: str, t: Tensor, ndim: int):
-    _require(isinstance(t, Tensor), TypeError, f"{name} must be a torch.Tensor")
+    _require(isinstance(t, Tensor), TypeError, lambda: f"{name} must be a torch.Tensor")
     _require(t.is_cuda, RuntimeError,
-             f"{name} must live on a HIP device (got {t.device}); the kernels have no CPU path")
-    _require(t.dtype == torch.float16, TypeError, f"{name} must be float16 (got {t.dtype})")
-    _require(t.dim() == ndim, ValueError, f"{name} must have {ndim} dims (got {tuple(t.shape)})")
-    _require(t.is_contiguous(), ValueError, f"{name} must be contiguous")
+             lambda: f"{name} must live on a HIP device (got {t.device}); the kernels have no CPU path")
+    _require(t.dtype == torch.float16, TypeError, lambda: f"{name} must be float16 (got {t.dtype})")
+    _require(t.dim() == ndim, ValueError, lambda: f"{name} must have {ndim} dims (got {tuple(t.shape)})")
+    _require(t.is_contiguous(), ValueError, lambda: f"{name} must be contiguous")
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream_ptr(device) -> int:
+    # the raw-stream accessor skips the Stream object; same value as current_stream(device).cuda_stream
+    if _raw_stream is not None:
+        index = device if isinstance(device, int) else device.index
+        if index is not None:
+            return _raw_stream(index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _on_device:
+    """``with _on_device(dev):`` makes dev the current device for the launch; a no-op (no context
+    switch, no driver call) when it already is, which is the common case."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, device):
+        self.ctx = None if device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
 
 
 def _workspace(nbytes: int, device) -> Tensor:
@@ -53,10 +80,10 @@ def _check_qkv(q: Tensor, k: Tensor, v: Tensor):
     _check_half_cuda("q", q, 3)
     _check_half_cuda("k", k, 3)
     _check_half_cuda("v", v, 3)
-    _require(q.shape == k.shape, ValueError, f"q {tuple(q.shape)} and k {tuple(k.shape)} differ")
+    _require(q.shape == k.shape, ValueError, lambda: f"q {tuple(q.shape)} and k {tuple(k.shape)} differ")
     _require(v.shape[:2] == q.shape[:2], ValueError,
-             f"v {tuple(v.shape)} does not match q {tuple(q.shape)} in [tgt_len, bsz*heads]")
-    _require(q.device == k.device == v.device, RuntimeError, "q, k, v must be on one device")
+             lambda: f"v {tuple(v.shape)} does not match q {tuple(q.shape)} in [tgt_len, bsz*heads]")
+    _require(q.device == k.device == v.device, RuntimeError, lambda: "q, k, v must be on one device")
 
 
 def forward(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
@@ -69,7 +96,7 @@ def forward(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
     T, N, K = q.shape
     d = v.shape[2]
     out = torch.empty_like(v)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         nbytes = lib.rfa_causal_forward_workspace_bytes(T, N, K, d)
         ws = _workspace(nbytes, q.device)
         _lib.check(lib.rfa_causal_forward(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
@@ -89,7 +116,7 @@ def prefill(q: Tensor, k: Tensor, v: Tensor):
     out = torch.empty_like(v)
     s = torch.empty((N, K, d), dtype=torch.float32, device=q.device)
     z = torch.empty((N, K), dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         nbytes = lib.rfa_causal_forward_workspace_bytes(T, N, K, d)
         ws = _workspace(nbytes, q.device)
         _lib.check(lib.rfa_causal_prefill(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), s.data_ptr(),
@@ -104,7 +131,7 @@ def forward_save(q: Tensor, k: Tensor, v: Tensor):
     T, N, K = q.shape
     d = v.shape[2]
     out = torch.empty_like(v)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         nbytes = lib.rfa_causal_forward_workspace_bytes(T, N, K, d)
         sbytes = lib.rfa_causal_saved_state_bytes(T, N, K, d)
         ws = _workspace(nbytes, q.device)
@@ -121,15 +148,15 @@ def backward_saved(q: Tensor, k: Tensor, v: Tensor, grad_attn: Tensor, out: Tens
     _check_half_cuda("grad_attn", grad_attn, 3)
     _check_half_cuda("out", out, 3)
     _require(grad_attn.shape == v.shape, ValueError,
-             f"grad_attn {tuple(grad_attn.shape)} must match v {tuple(v.shape)}")
-    _require(out.shape == v.shape, ValueError, f"out {tuple(out.shape)} must match v {tuple(v.shape)}")
+             lambda: f"grad_attn {tuple(grad_attn.shape)} must match v {tuple(v.shape)}")
+    _require(out.shape == v.shape, ValueError, lambda: f"out {tuple(out.shape)} must match v {tuple(v.shape)}")
     _require(saved.is_cuda and saved.dtype == torch.uint8 and saved.is_contiguous(), TypeError,
-             "saved must be the byte buffer returned by forward_save")
+             lambda: "saved must be the byte buffer returned by forward_save")
     lib = _lib.load()
     T, N, K = q.shape
     d = v.shape[2]
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         nbytes = lib.rfa_causal_backward_workspace_bytes(T, N, K, d)
         ws = _workspace(nbytes, q.device)
         _lib.check(lib.rfa_causal_backward_saved(q.data_ptr(), k.data_ptr(), v.data_ptr(), grad_attn.data_ptr(),
@@ -147,12 +174,12 @@ def backward(q: Tensor, k: Tensor, v: Tensor, grad_attn: Tensor) -> List[Tensor]
     _check_qkv(q, k, v)
     _check_half_cuda("grad_attn", grad_attn, 3)
     _require(grad_attn.shape == v.shape, ValueError,
-             f"grad_attn {tuple(grad_attn.shape)} must match v {tuple(v.shape)}")
+             lambda: f"grad_attn {tuple(grad_attn.shape)} must match v {tuple(v.shape)}")
     lib = _lib.load()
     T, N, K = q.shape
     d = v.shape[2]
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         nbytes = lib.rfa_causal_backward_workspace_bytes(T, N, K, d)
         ws = _workspace(nbytes, q.device)
         _lib.check(lib.rfa_causal_backward(q.data_ptr(), k.data_ptr(), v.data_ptr(), grad_attn.data_ptr(),
@@ -172,8 +199,8 @@ def _check_feature_args(x: Tensor, w: Tensor):
     _check_half_cuda("x", x, 4)
     _check_half_cuda("random_matrices", w, 3)
     _require(w.shape[0] == x.shape[2] and w.shape[2] == x.shape[3], ValueError,
-             f"random_matrices {tuple(w.shape)} must be [num_heads, proj_dim, head_dim] for x {tuple(x.shape)}")
-    _require(x.device == w.device, RuntimeError, "x and random_matrices must be on one device")
+             lambda: f"random_matrices {tuple(w.shape)} must be [num_heads, proj_dim, head_dim] for x {tuple(x.shape)}")
+    _require(x.device == w.device, RuntimeError, lambda: "x and random_matrices must be on one device")
 
 
 def feature_map_forward(x: Tensor, w: Tensor, scale: float) -> Tensor:
@@ -182,7 +209,7 @@ def feature_map_forward(x: Tensor, w: Tensor, scale: float) -> Tensor:
     L, B, H, d = x.shape
     D = w.shape[1]
     phi = torch.empty((L, B, H, 2 * D), dtype=torch.float16, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _lib.check(_lib.load().rfa_feature_map_forward(
             x.data_ptr(), w.data_ptr(), phi.data_ptr(), L * B, H, D, d, float(scale), _stream_ptr(x.device)))
     return phi
@@ -201,22 +228,22 @@ def project_feature_map(x: Tensor, weights, biases, want_phi, w: Optional[Tensor
     L, B, E = x.shape
     n = len(weights)
     _require(1 <= n <= 3 and len(biases) == n and len(want_phi) == n, ValueError,
-             "1..3 projections with one bias entry and one want_phi flag each")
+             lambda: "1..3 projections with one bias entry and one want_phi flag each")
     out_dim = weights[0].shape[0]
-    _require(out_dim % heads == 0, ValueError, f"output width {out_dim} is not a multiple of heads={heads}")
+    _require(out_dim % heads == 0, ValueError, lambda: f"output width {out_dim} is not a multiple of heads={heads}")
     d = out_dim // heads
     for wt, b in zip(weights, biases):
         _check_half_cuda("weight", wt, 2)
-        _require(tuple(wt.shape) == (out_dim, E), ValueError, f"weight {tuple(wt.shape)} must be {(out_dim, E)}")
-        _require(wt.device == x.device, RuntimeError, "x and weights must be on one device")
+        _require(tuple(wt.shape) == (out_dim, E), ValueError, lambda: f"weight {tuple(wt.shape)} must be {(out_dim, E)}")
+        _require(wt.device == x.device, RuntimeError, lambda: "x and weights must be on one device")
         if b is not None:
             _check_half_cuda("bias", b, 1)
-            _require(b.shape[0] == out_dim and b.device == x.device, ValueError, f"bias must be [{out_dim}] on x's device")
+            _require(b.shape[0] == out_dim and b.device == x.device, ValueError, lambda: f"bias must be [{out_dim}] on x's device")
     if any(want_phi):
-        _require(w is not None, ValueError, "feature matrices are needed when a phi is wanted")
+        _require(w is not None, ValueError, lambda: "feature matrices are needed when a phi is wanted")
         _check_half_cuda("random_matrices", w, 3)
         _require(w.shape[0] == heads and w.shape[2] == d and w.device == x.device, ValueError,
-                 f"random_matrices {tuple(w.shape)} must be [{heads}, D, {d}] on x's device")
+                 lambda: f"random_matrices {tuple(w.shape)} must be [{heads}, D, {d}] on x's device")
         D = w.shape[1]
     else:
         D = 32
@@ -224,7 +251,7 @@ def project_feature_map(x: Tensor, weights, biases, want_phi, w: Optional[Tensor
     phis = [torch.empty((L, B, heads, 2 * D), dtype=torch.float16, device=x.device) if f else None for f in want_phi]
     arr = ctypes.c_void_p * n
     ptr = lambda t: None if t is None else t.data_ptr()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _lib.check(_lib.load().rfa_project_feature_map(
             x.data_ptr(), arr(*[wt.data_ptr() for wt in weights]), arr(*[ptr(b) for b in biases]),
             arr(*[t.data_ptr() for t in ys]), arr(*[ptr(t) for t in phis]), n, ptr(w) if any(want_phi) else None,
@@ -246,19 +273,19 @@ def linear_weight_grad(x: Tensor, dys, want_bias):
     _check_half_cuda("x", x, 2)
     R, e_in = x.shape
     n = len(dys)
-    _require(1 <= n <= 3 and len(want_bias) == n, ValueError, "1..3 layers with one want_bias flag each")
+    _require(1 <= n <= 3 and len(want_bias) == n, ValueError, lambda: "1..3 layers with one want_bias flag each")
     e_out = dys[0].shape[1]
     for dy in dys:
         _check_half_cuda("dy", dy, 2)
         _require(tuple(dy.shape) == (R, e_out) and dy.device == x.device, ValueError,
-                 f"dy {tuple(dy.shape)} must be {(R, e_out)} on x's device")
+                 lambda: f"dy {tuple(dy.shape)} must be {(R, e_out)} on x's device")
     _require(linear_weight_grad_supported(e_out, e_in), ValueError,
-             f"E_out={e_out} and E_in={e_in} must be multiples of 128")
+             lambda: f"E_out={e_out} and E_in={e_in} must be multiples of 128")
     lib = _lib.load()
     dws = [torch.empty((e_out, e_in), dtype=torch.float16, device=x.device) for _ in range(n)]
     dbs = [torch.empty((e_out,), dtype=torch.float16, device=x.device) if f else None for f in want_bias]
     arr = ctypes.c_void_p * n
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         nbytes = lib.rfa_linear_weight_grad_workspace_bytes(max(R, 1), e_out, e_in, n)
         ws = _workspace(nbytes, x.device)
         _lib.check(lib.rfa_linear_weight_grad(
@@ -275,11 +302,11 @@ def feature_map_backward(x: Tensor, w: Tensor, grad_phi: Tensor, scale: float):
     D = w.shape[1]
     _check_half_cuda("grad_phi", grad_phi, 4)
     _require(tuple(grad_phi.shape) == (L, B, H, 2 * D), ValueError,
-             f"grad_phi {tuple(grad_phi.shape)} must be {(L, B, H, 2 * D)}")
+             lambda: f"grad_phi {tuple(grad_phi.shape)} must be {(L, B, H, 2 * D)}")
     lib = _lib.load()
     dx = torch.empty_like(x)
     dw = torch.empty((H, D, d), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         nbytes = lib.rfa_feature_map_backward_workspace_bytes(L * B, H, D, d)
         ws = _workspace(nbytes, x.device)
         _lib.check(lib.rfa_feature_map_backward(
@@ -292,18 +319,18 @@ def feature_map_backward(x: Tensor, w: Tensor, grad_phi: Tensor, scale: float):
 # cross attention
 # ---------------------------------------------------------------------------
 def _check_f32_cuda(name: str, t: Tensor, shape):
-    _require(isinstance(t, Tensor) and t.is_cuda, RuntimeError, f"{name} must live on a HIP device")
-    _require(t.dtype == torch.float32, TypeError, f"{name} must be float32 (got {t.dtype})")
-    _require(tuple(t.shape) == tuple(shape), ValueError, f"{name} must have shape {tuple(shape)} (got {tuple(t.shape)})")
-    _require(t.is_contiguous(), ValueError, f"{name} must be contiguous")
+    _require(isinstance(t, Tensor) and t.is_cuda, RuntimeError, lambda: f"{name} must live on a HIP device")
+    _require(t.dtype == torch.float32, TypeError, lambda: f"{name} must be float32 (got {t.dtype})")
+    _require(tuple(t.shape) == tuple(shape), ValueError, lambda: f"{name} must have shape {tuple(shape)} (got {tuple(t.shape)})")
+    _require(t.is_contiguous(), ValueError, lambda: f"{name} must be contiguous")
 
 
 def _mask_arg(mask, B: int, S: int, device):
     """key_padding_mask [B, S] (non-zero = pad) -> (uint8 tensor kept alive, pointer)."""
     if mask is None:
         return None, None
-    _require(tuple(mask.shape) == (B, S), ValueError, f"key_padding_mask must be [{B}, {S}] (got {tuple(mask.shape)})")
-    _require(mask.device == device, RuntimeError, "key_padding_mask must be on the tensors' device")
+    _require(tuple(mask.shape) == (B, S), ValueError, lambda: f"key_padding_mask must be [{B}, {S}] (got {tuple(mask.shape)})")
+    _require(mask.device == device, RuntimeError, lambda: "key_padding_mask must be on the tensors' device")
     m = (mask != 0).to(torch.uint8).contiguous()
     return m, m.data_ptr()
 
@@ -312,13 +339,13 @@ def cross_state(phi_k: Tensor, v: Tensor, key_padding_mask=None):
     """phi_k fp16 [S, B, H, K], v fp16 [S, B, H, d], mask [B, S] -> (s fp32 [B,H,K,d], z fp32 [B,H,K])."""
     _check_half_cuda("phi_k", phi_k, 4)
     _check_half_cuda("v", v, 4)
-    _require(phi_k.shape[:3] == v.shape[:3], ValueError, "phi_k and v must agree in [src_len, bsz, heads]")
+    _require(phi_k.shape[:3] == v.shape[:3], ValueError, lambda: "phi_k and v must agree in [src_len, bsz, heads]")
     S, B, H, K = phi_k.shape
     d = v.shape[3]
     s = torch.empty((B, H, K, d), dtype=torch.float32, device=v.device)
     z = torch.empty((B, H, K), dtype=torch.float32, device=v.device)
     keep, mptr = _mask_arg(key_padding_mask, B, S, v.device)
-    with torch.cuda.device(v.device):
+    with _on_device(v.device):
         _lib.check(_lib.load().rfa_cross_state(phi_k.data_ptr(), v.data_ptr(), mptr, s.data_ptr(), z.data_ptr(),
                                                S, B, H, K, d, _stream_ptr(v.device)))
     return s, z
@@ -333,7 +360,7 @@ def cross_state_backward(phi_k: Tensor, v: Tensor, ds: Tensor, dz: Tensor, key_p
     _check_f32_cuda("dz", dz, (B, H, K))
     dphi_k, dv = torch.empty_like(phi_k), torch.empty_like(v)
     keep, mptr = _mask_arg(key_padding_mask, B, S, v.device)
-    with torch.cuda.device(v.device):
+    with _on_device(v.device):
         _lib.check(_lib.load().rfa_cross_state_backward(
             phi_k.data_ptr(), v.data_ptr(), mptr, ds.data_ptr(), dz.data_ptr(), dphi_k.data_ptr(), dv.data_ptr(),
             S, B, H, K, d, _stream_ptr(v.device)))
@@ -344,12 +371,12 @@ def cross_readout(phi_q: Tensor, s: Tensor, z: Tensor) -> Tensor:
     """phi_q fp16 [T, B, H, K], s fp32 [B,H,K,d], z fp32 [B,H,K] -> attn fp16 [T, B, H, d]."""
     _check_half_cuda("phi_q", phi_q, 4)
     T, B, H, K = phi_q.shape
-    _require(s.dim() == 4, ValueError, "s must be [bsz, heads, 2*proj_dim, head_dim]")
+    _require(s.dim() == 4, ValueError, lambda: "s must be [bsz, heads, 2*proj_dim, head_dim]")
     d = s.shape[3]
     _check_f32_cuda("s", s, (B, H, K, d))
     _check_f32_cuda("z", z, (B, H, K))
     out = torch.empty((T, B, H, d), dtype=torch.float16, device=phi_q.device)
-    with torch.cuda.device(phi_q.device):
+    with _on_device(phi_q.device):
         _lib.check(_lib.load().rfa_cross_readout(phi_q.data_ptr(), s.data_ptr(), z.data_ptr(), out.data_ptr(),
                                                  T, B * H, K, d, _stream_ptr(phi_q.device)))
     return out
@@ -362,10 +389,10 @@ def cross_readout_backward(phi_q: Tensor, s: Tensor, z: Tensor, grad_attn: Tenso
     _check_f32_cuda("s", s, (B, H, K, d))
     _check_f32_cuda("z", z, (B, H, K))
     _check_half_cuda("grad_attn", grad_attn, 4)
-    _require(tuple(grad_attn.shape) == (T, B, H, d), ValueError, "grad_attn must be [tgt_len, bsz, heads, head_dim]")
+    _require(tuple(grad_attn.shape) == (T, B, H, d), ValueError, lambda: "grad_attn must be [tgt_len, bsz, heads, head_dim]")
     dphi_q = torch.empty_like(phi_q)
     ds, dz = torch.empty_like(s), torch.empty_like(z)
-    with torch.cuda.device(phi_q.device):
+    with _on_device(phi_q.device):
         _lib.check(_lib.load().rfa_cross_readout_backward(
             phi_q.data_ptr(), s.data_ptr(), z.data_ptr(), grad_attn.data_ptr(), dphi_q.data_ptr(),
             ds.data_ptr(), dz.data_ptr(), T, B * H, K, d, _stream_ptr(phi_q.device)))
@@ -383,7 +410,7 @@ def incremental(phi_q: Tensor, phi_k: Tensor, v: Tensor, s: Tensor, z: Tensor) -
     _check_f32_cuda("s", s, (N, K, d))
     _check_f32_cuda("z", z, (N, K))
     out = torch.empty_like(v)
-    with torch.cuda.device(v.device):
+    with _on_device(v.device):
         _lib.check(_lib.load().rfa_incremental(phi_q.data_ptr(), phi_k.data_ptr(), v.data_ptr(), s.data_ptr(),
                                                z.data_ptr(), out.data_ptr(), steps, N, K, d, _stream_ptr(v.device)))
     return out
@@ -393,15 +420,15 @@ def incremental_fused(q: Tensor, k: Tensor, v: Tensor, w: Tensor, scale: float, 
     """q, k, v fp16 [steps, B, H, d]; w fp16 [H, D, d]; s fp32 [B,H,2D,d], z fp32 [B,H,2D] updated in place."""
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_half_cuda(name, t, 4)
-    _require(q.shape == k.shape == v.shape, ValueError, "q, k, v must have one shape [steps, bsz, heads, head_dim]")
+    _require(q.shape == k.shape == v.shape, ValueError, lambda: "q, k, v must have one shape [steps, bsz, heads, head_dim]")
     _check_half_cuda("random_matrices", w, 3)
     steps, B, H, d = q.shape
     D = w.shape[1]
-    _require(w.shape[0] == H and w.shape[2] == d, ValueError, "random_matrices must be [heads, proj_dim, head_dim]")
+    _require(w.shape[0] == H and w.shape[2] == d, ValueError, lambda: "random_matrices must be [heads, proj_dim, head_dim]")
     _check_f32_cuda("s", s, (B, H, 2 * D, d))
     _check_f32_cuda("z", z, (B, H, 2 * D))
     out = torch.empty_like(v)
-    with torch.cuda.device(v.device):
+    with _on_device(v.device):
         _lib.check(_lib.load().rfa_incremental_fused(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), w.data_ptr(), float(scale), s.data_ptr(), z.data_ptr(),
             out.data_ptr(), steps, B, H, D, d, _stream_ptr(v.device)))
@@ -415,7 +442,7 @@ def pack_attn_mask(masked: Tensor):
     """bool [T, S] (True = masked) -> (bytes [T, Sp], bytes of the transpose [S, Tp]), rows padded
     to a multiple of 64 with ones, as rfa_masked_forward / rfa_masked_backward read them."""
     _require(masked.dim() == 2 and masked.shape[0] == masked.shape[1], ValueError,
-             f"attn_mask must be [tgt_len, tgt_len] (got {tuple(masked.shape)})")
+             lambda: f"attn_mask must be [tgt_len, tgt_len] (got {tuple(masked.shape)})")
     T = masked.shape[0]
     Tp = (T + 63) // 64 * 64
     m = torch.ones((T, Tp), dtype=torch.uint8, device=masked.device)
@@ -431,7 +458,7 @@ def masked_forward(phi_q: Tensor, phi_k: Tensor, v: Tensor, H: int, key_padding_
     _check_qkv(phi_q, phi_k, v)
     T, N, K = phi_q.shape
     d = v.shape[2]
-    _require(N % H == 0, ValueError, f"N={N} is not a multiple of heads={H}")
+    _require(N % H == 0, ValueError, lambda: f"N={N} is not a multiple of heads={H}")
     B = N // H
     Tp = (T + 63) // 64 * 64
     out = torch.empty_like(v)
@@ -439,8 +466,8 @@ def masked_forward(phi_q: Tensor, phi_k: Tensor, v: Tensor, H: int, key_padding_
     keep, mptr = _mask_arg(key_padding_mask, B, T, v.device)
     if attn_mask_bytes is not None:
         _require(attn_mask_bytes.is_cuda and attn_mask_bytes.dtype == torch.uint8 and attn_mask_bytes.is_contiguous()
-                 and tuple(attn_mask_bytes.shape) == (T, Tp), ValueError, "attn_mask_bytes must come from pack_attn_mask")
-    with torch.cuda.device(v.device):
+                 and tuple(attn_mask_bytes.shape) == (T, Tp), ValueError, lambda: "attn_mask_bytes must come from pack_attn_mask")
+    with _on_device(v.device):
         _lib.check(_lib.load().rfa_masked_forward(
             phi_q.data_ptr(), phi_k.data_ptr(), v.data_ptr(), mptr,
             attn_mask_bytes.data_ptr() if attn_mask_bytes is not None else None, out.data_ptr(), rsum.data_ptr(),
@@ -458,12 +485,12 @@ def masked_backward(phi_q: Tensor, phi_k: Tensor, v: Tensor, grad_attn: Tensor, 
     d = v.shape[2]
     B = N // H
     Tp = (T + 63) // 64 * 64
-    _require(grad_attn.shape == v.shape and out.shape == v.shape, ValueError, "grad_attn and out must match v")
+    _require(grad_attn.shape == v.shape and out.shape == v.shape, ValueError, lambda: "grad_attn and out must match v")
     _check_f32_cuda("rsum", rsum, (T, N))
     dq, dk, dv = torch.empty_like(phi_q), torch.empty_like(phi_k), torch.empty_like(v)
     keep, mptr = _mask_arg(key_padding_mask, B, T, v.device)
     lib = _lib.load()
-    with torch.cuda.device(v.device):
+    with _on_device(v.device):
         nbytes = lib.rfa_masked_backward_workspace_bytes(T, N, d)
         ws = _workspace(nbytes, v.device)
         _lib.check(lib.rfa_masked_backward(
