@@ -361,6 +361,21 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream):
                          "graph_equals_eager": bool(torch.equal(y_graph, y_eager) and torch.equal(mx.grad, gx_eager))}
     del graph, mod
 
+    # ---- matrix-pipe rate of the MFMA instruction the kernels use (register operands, no memory
+    # traffic): the fp16 figure this device delivers, next to the published 2.5 PFLOP/s
+    import ctypes
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    flops = ctypes.c_double(0.0)
+    rates = {}
+    for wps in (1, 2, 4):
+        probe = lambda: _lib.check(lib.rfa_selftest_mfma_rate(wps, 4096, p(sink), ctypes.byref(flops), stream))
+        for _ in range(3):
+            probe()
+        tp = _event_time_ms(torch, probe, 10)
+        rates[f"waves_per_simd_{wps}"] = round(flops.value / (tp * 1e-3) / 1e12, 1)
+    ex["mfma_rate"] = {"instruction": "v_mfma_f32_16x16x32_f16, 8 independent accumulators per wave",
+                       "tflops": rates, "published_dense_fp16_tflops": 2500.0}
+
     # ---- plain device copy of 512 MiB (larger than the 256 MiB last-level cache): the HBM
     # bandwidth a trivial kernel reaches here, and the known-size dispatch against which the
     # rocprofv3 FETCH_SIZE / WRITE_SIZE counters are scaled

@@ -50,6 +50,13 @@ int rfa_shape_supported(int K, int d);
  * kernels assume.  Returns RFA_OK when the layout matches. */
 int rfa_selftest_layout(void* stream);
 
+/* Matrix-pipe rate probe for roofline figures: launches waves_per_simd (1..8) waves on every SIMD
+ * of the device, each issuing iters x 8 independent 16x16x32 fp16 MFMAs on register operands (no
+ * memory traffic), and stores the number of floating-point operations of the launch in *flops
+ * (host memory).  The caller times the launch on its stream; sink is one float of device memory
+ * that is never written in practice.  No counterpart in the reference. */
+int rfa_selftest_mfma_rate(int waves_per_simd, int iters, float* sink, double* flops, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Causal attention (training / prefill).
  *

@@ -34,6 +34,7 @@ SIGNATURES = {
     "rfa_last_error": (c_char_p, []),
     "rfa_shape_supported": (c_int, [c_int, c_int]),
     "rfa_selftest_layout": (c_int, [c_void_p]),
+    "rfa_selftest_mfma_rate": (c_int, [c_int, c_int, c_void_p, ctypes.POINTER(ctypes.c_double), c_void_p]),
     "rfa_causal_num_segments": (c_int, [c_int64, c_int64]),
     "rfa_causal_forward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
     "rfa_causal_forward": (c_int, [c_void_p] * 4 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),

@@ -596,6 +596,31 @@ __global__ void k_selftest(int* bad) {
     if (nbad) atomicAdd(bad, nbad);
 }
 
+// ---- MFMA issue-rate probe ---------------------------------------------------
+// Every wave runs `iters` rounds of 8 independent 16x16x32 fp16 MFMA accumulations on
+// register operands: no memory traffic, so the time measures the matrix pipes alone.
+__global__ __launch_bounds__(256) void k_mfma_rate(int iters, float* sink) {
+    using namespace rfa;
+    const int lane = threadIdx.x & 63;
+    h8 a, b;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        a[e] = (half_t)(float)((lane + e) % 3 - 1);
+        b[e] = (half_t)(float)((lane * 3 + e) % 5 - 2);
+    }
+    f4 acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc[t] = f4_zero();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[t] = mfma32(a, b, acc[t]);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) s += acc[t][0] + acc[t][1] + acc[t][2] + acc[t][3];
+    if (s == 12345.678f) sink[0] = s;      // keeps the loop alive without a store in practice
+}
+
 }  // namespace
 
 extern "C" {
@@ -638,6 +663,20 @@ int rfa_selftest_layout(void* stream) {
     (void)hipFree(dbad);
     if (e != hipSuccess) return fail(RFA_ERR_HIP, "selftest: %s", hipGetErrorString(e));
     if (hbad) return fail(RFA_ERR_HIP, "selftest: %d lane values differ from the assumed MFMA / LDS layout", hbad);
+    return RFA_OK;
+}
+
+int rfa_selftest_mfma_rate(int waves_per_simd, int iters, float* sink, double* flops, void* stream) {
+    if (waves_per_simd < 1 || waves_per_simd > 8 || iters < 1 || !sink || !flops)
+        return fail(RFA_ERR_BAD_SHAPE, "rfa_selftest_mfma_rate: waves_per_simd in 1..8, iters >= 1, non-NULL sink and flops");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int dev = 0, cus = 0;
+    RFA_HIP_TRY(hipGetDevice(&dev));
+    RFA_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int blocks = cus * waves_per_simd;           // 4 waves per workgroup, one per SIMD
+    RFA_LAUNCH(SELFTEST, k_mfma_rate, dim3(blocks), dim3(256), 0, st, iters, sink);
+    RFA_HIP_TRY(hipGetLastError());
+    *flops = (double)blocks * 4 * iters * 8 * (2.0 * 16 * 16 * 32);
     return RFA_OK;
 }
 
