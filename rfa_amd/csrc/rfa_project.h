@@ -35,6 +35,13 @@ __device__ __forceinline__ T pick3(T const (&a)[kMaxProjections], int p) {
     return p == 0 ? a[0] : (p == 1 ? a[1] : a[2]);
 }
 
+// Orders this wave's LDS accesses for the compiler only (the hardware runs one wave's LDS
+// instructions in order); unlike a fence it does not wait for outstanding global loads/stores.
+__device__ __forceinline__ void wave_lds_order() {
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");
+}
+
 template <int D, int DH>
 struct ProjectCfg {
     static_assert(D % 32 == 0 && DH % 64 == 0, "D multiple of 32, DH multiple of 64");
@@ -176,9 +183,9 @@ __global__ __launch_bounds__(kThreads) void k_project_phi(
             }
             *reinterpret_cast<h4*>(Ps + i * LDP + 16 * ct + 4 * G) = yh;
         }
-        wave_lds_fence();
+        wave_lds_order();
         wave_rows_s2g<DH>(Ps, LDP, y, r0, R, H, h, lane);
-        wave_lds_fence();
+        wave_lds_order();
         if (phi) {
             ss = sum_over_groups(ss);
             const float inv = 1.0f / (sqrtf(ss) + 1e-3f);
@@ -200,9 +207,9 @@ __global__ __launch_bounds__(kThreads) void k_project_phi(
                 *reinterpret_cast<h4*>(Ps + i * LDP + 16 * jt + 4 * G) = sv;
                 *reinterpret_cast<h4*>(Ps + i * LDP + D + 16 * jt + 4 * G) = cv;
             }
-            wave_lds_fence();
+            wave_lds_order();
             wave_rows_s2g<2 * D>(Ps, LDP, phi, r0, R, H, h, lane);
-            wave_lds_fence();
+            wave_lds_order();
         }
     }
 }
@@ -221,13 +228,6 @@ __global__ __launch_bounds__(kThreads) void k_project_phi(
 // is copied with memcpy, which keeps registers that stay in flight across loop iterations in
 // private memory)
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-// Orders this wave's LDS accesses for the compiler only (the hardware runs one wave's LDS
-// instructions in order); unlike a fence it does not wait for outstanding global loads/stores.
-__device__ __forceinline__ void wave_lds_order() {
-    __builtin_amdgcn_wave_barrier();
-    asm volatile("" ::: "memory");
-}
 
 template <int D, int DH, int NKS>
 struct ProjectRowCfg {
