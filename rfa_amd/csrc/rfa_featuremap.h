@@ -27,12 +27,13 @@ struct FeatureCfg {
     static constexpr size_t kBwdLds = (size_t)(D * LDW + 64 * LDW + 64 * LDU + 64 * LDG) * 2;
 };
 
-// Orders this wave's earlier LDS writes before its later LDS reads of other lanes' data
-// (one wave executes its LDS instructions in order; this only stops the compiler).
-__device__ __forceinline__ void wave_lds_fence() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+// Orders this wave's earlier LDS writes before its later LDS reads of other lanes' data.  One
+// wave executes its LDS instructions in order, so only the compiler has to be stopped from
+// moving them; a memory fence here would also wait for every global load and store in flight
+// (the next block's prefetch, the previous rows' stores).
+__device__ __forceinline__ void wave_lds_order() {
     __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    asm volatile("" ::: "memory");
 }
 
 // Copy this wave's 16 staged rows (F halves each, row stride ld in LDS) to global rows
@@ -69,8 +70,10 @@ __device__ __forceinline__ void wave_rows_g2r(WaveRows<F>& rr, const half_t* __r
 #pragma unroll
     for (int k = 0; k < 16 / RPI; ++k) {
         const int lr = k * RPI + lane / PPR, pc = lane % PPR;
-        rr.v[k] = make_uint4(0, 0, 0, 0);
-        if (r0 + lr < R) rr.v[k] = *reinterpret_cast<const uint4*>(src + ((int64_t)(r0 + lr) * H + h) * F + pc * 8);
+        // no branch around the load: a row past the end reads the last row and is zeroed afterwards
+        const int rc = min(r0 + lr, R - 1);
+        rr.v[k] = *reinterpret_cast<const uint4*>(src + ((int64_t)rc * H + h) * F + pc * 8);
+        if (r0 + lr >= R) rr.v[k] = make_uint4(0, 0, 0, 0);
     }
 }
 
@@ -147,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_fwd(
     }
     // the fragment layout holds 8 bytes per lane and row: stage through LDS so that the
     // stores to HBM cover whole 4D-byte rows
-    wave_lds_fence();
+    wave_lds_order();
     wave_rows_s2g<2 * D>(Ps, LDP, phi, blockIdx.x * 64 + 16 * wv, R, H, h, lane);
 }
 
@@ -191,9 +194,11 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
         const int r = rb * 64 + lr;
 #pragma unroll
         for (int cs = 0; cs < DH / 32; ++cs) {
+            xn[cs] = *reinterpret_cast<const h8*>(x + ((int64_t)min(r, R - 1) * H + h) * DH + cs * 32 + 8 * G);
+            if (r >= R) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) xn[cs][e] = (half_t)0.f;
-            if (r < R) xn[cs] = *reinterpret_cast<const h8*>(x + ((int64_t)r * H + h) * DH + cs * 32 + 8 * G);
+                for (int e = 0; e < 8; ++e) xn[cs][e] = (half_t)0.f;
+            }
         }
         wave_rows_g2r<2 * D>(gn, gphi, rb * 64 + 16 * wv, R, H, h, lane);
     };
@@ -261,7 +266,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
             for (int e = 0; e < 4; ++e) o[e] = (half_t)(y[ct][e] - (float)xv[e] * xdot);
             *reinterpret_cast<h4*>(Gs + i * LDG + 16 * ct + 4 * G) = o;
         }
-        wave_lds_fence();
+        wave_lds_order();
         wave_rows_s2g<DH>(Gs, LDG, dx, r0, R, H, h, lane);
 
         // dW (m = c, n = j) += X^T Us over the 64 rows of the block

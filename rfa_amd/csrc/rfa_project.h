@@ -35,13 +35,6 @@ __device__ __forceinline__ T pick3(T const (&a)[kMaxProjections], int p) {
     return p == 0 ? a[0] : (p == 1 ? a[1] : a[2]);
 }
 
-// Orders this wave's LDS accesses for the compiler only (the hardware runs one wave's LDS
-// instructions in order); unlike a fence it does not wait for outstanding global loads/stores.
-__device__ __forceinline__ void wave_lds_order() {
-    __builtin_amdgcn_wave_barrier();
-    asm volatile("" ::: "memory");
-}
-
 template <int D, int DH>
 struct ProjectCfg {
     static_assert(D % 32 == 0 && DH % 64 == 0, "D multiple of 32, DH multiple of 64");
