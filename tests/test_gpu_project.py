@@ -278,3 +278,16 @@ def test_module_step_replays_from_a_hip_graph():
         step()
         torch.cuda.synchronize()
         captured = grads_before
+
+
+def test_empty_input():
+    """No rows: the projections come back empty, the weight and bias gradients as zeros."""
+    from rfa_amd import rfa_hip
+    H, d, D, E = 2, 64, 64, 128
+    x = torch.empty(0, 3, E, dtype=torch.float16).cuda()
+    ws = [torch.randn(H * d, E).half().cuda() for _ in range(2)]
+    wf = torch.randn(H, D, d).half().cuda()
+    ys, phis = rfa_hip.project_feature_map(x, ws, [None, None], [True, False], wf, H, O.SCALE)
+    assert ys[0].shape == (0, 3, H, d) and phis[0].shape == (0, 3, H, 2 * D) and phis[1] is None
+    dws, dbs = rfa_hip.linear_weight_grad(x.view(0, E), [torch.empty(0, H * d, dtype=torch.float16).cuda()], [True])
+    assert dws[0].shape == (H * d, E) and (dws[0] == 0).all() and (dbs[0] == 0).all()
