@@ -164,7 +164,7 @@ def test_causal_module_fused_projections_match_unfused_chain(with_pad):
         assert rel(g_f[name].double(), ref[name]) <= 2e-2, (name, rel(g_f[name].double(), ref[name]))
 
 
-@pytest.mark.parametrize("R,Eo,Ei,n", [(8192, 512, 512, 3), (200, 128, 256, 1), (1, 128, 128, 2), (4097, 256, 128, 3),
+@pytest.mark.parametrize("R,Eo,Ei,n", [(8192, 512, 512, 3), (300, 256, 512, 2), (70, 768, 256, 1), (200, 128, 256, 1), (1, 128, 128, 2), (4097, 256, 128, 3),
                                        (64, 384, 128, 1)])
 def test_linear_weight_and_bias_gradients(R, Eo, Ei, n):
     """dW = dy^T x and db = column sums against fp64; fp16 outputs of fp32 sums: <= 1.5e-3 relative
