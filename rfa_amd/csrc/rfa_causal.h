@@ -1411,17 +1411,42 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     // later segments' totals, or the one exclusive suffix k_totals_scan left
     const int s_first = CAUSAL ? (prefixed ? seg : seg + 1) : 0, s_last = CAUSAL ? (prefixed ? seg + 1 : nseg) : 1;
     const int state_stride = CAUSAL ? nseg : 1;
-    for (int s = s_first; s < s_last; ++s) {
-        const float* ri = wsR + ((int64_t)(n * state_stride + s) * KD) * DH;
+    {
+        // The carried state at the segment's last step, R = sum of the slots [s_first, s_last): all
+        // threads add the slots up with coalesced 16-byte loads and pass the sum through LDS (which
+        // the first chunk does not need yet); each wave then takes its fragments from there.  Reading
+        // the fragments straight from HBM costs the dV waves 32 scalar loads per lane and slot.
+        constexpr int LDR = DH + 4;                          // floats; spreads the rows over the banks
+        constexpr bool kStaged = (size_t)KD * LDR * 4 <= Cfg::kBwdDkLds;   // the sum fits the chunk buffers
+        if constexpr (kStaged) {
+        constexpr int PER = KD * DH / 4 / NT;
+        static_assert((KD * DH / 4) % NT == 0, "state does not divide over the threads");
+        float* Rs = reinterpret_cast<float*>(smem_raw);
+        f4 sum[PER];
+#pragma unroll
+        for (int it = 0; it < PER; ++it) sum[it] = f4_zero();
+        for (int s = s_first; s < s_last; ++s) {
+            const float* ri = wsR + ((int64_t)(n * state_stride + s) * KD) * DH;
+#pragma unroll
+            for (int it = 0; it < PER; ++it) sum[it] += *reinterpret_cast<const f4*>(ri + (int64_t)(tid + NT * it) * 4);
+            if (do_dk) {
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt)
+                    racc[kt] += *reinterpret_cast<const f4*>(wsr + (int64_t)(n * state_stride + s) * KD + ws * KS + 16 * kt + 4 * G);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < PER; ++it) {
+            const int e0 = (tid + NT * it) * 4;
+            *reinterpret_cast<f4*>(Rs + (e0 / DH) * LDR + e0 % DH) = sum[it];
+        }
+        __syncthreads();
         if (do_dk) {
 #pragma unroll
             for (int ct = 0; ct < NCT; ++ct)
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt)
-                    RT[ct][kt] += *reinterpret_cast<const f4*>(ri + (ws * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
-#pragma unroll
-            for (int kt = 0; kt < NKT; ++kt)
-                racc[kt] += *reinterpret_cast<const f4*>(wsr + (int64_t)(n * state_stride + s) * KD + ws * KS + 16 * kt + 4 * G);
+                    RT[ct][kt] = *reinterpret_cast<const f4*>(Rs + (ws * KS + 16 * kt + row) * LDR + 16 * ct + 4 * G);
         }
         if (do_dv) {
 #pragma unroll
@@ -1429,8 +1454,32 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
 #pragma unroll
                 for (int ct = 0; ct < NCT2; ++ct)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        RR[kt][ct][e] += ri[(16 * kt + 4 * G + e) * DH + ws * DS + 16 * ct + row];
+                    for (int e = 0; e < 4; ++e) RR[kt][ct][e] = Rs[(16 * kt + 4 * G + e) * LDR + ws * DS + 16 * ct + row];
+        }
+        __syncthreads();                                     // before the first chunk overwrites the staged state
+        } else {
+            for (int s = s_first; s < s_last; ++s) {
+                const float* ri = wsR + ((int64_t)(n * state_stride + s) * KD) * DH;
+                if (do_dk) {
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                        for (int kt = 0; kt < NKT; ++kt)
+                            RT[ct][kt] += *reinterpret_cast<const f4*>(ri + (ws * KS + 16 * kt + row) * DH + 16 * ct + 4 * G);
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt)
+                        racc[kt] += *reinterpret_cast<const f4*>(wsr + (int64_t)(n * state_stride + s) * KD + ws * KS + 16 * kt + 4 * G);
+                }
+                if (do_dv) {
+#pragma unroll
+                    for (int kt = 0; kt < NKT2; ++kt)
+#pragma unroll
+                        for (int ct = 0; ct < NCT2; ++ct)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                RR[kt][ct][e] += ri[(16 * kt + 4 * G + e) * DH + ws * DS + 16 * ct + row];
+                }
+            }
         }
     }
 
