@@ -183,3 +183,34 @@ def test_wide_state_backward_on_half_as_many_segments(nseg, same, monkeypatch):
     for pair in (rfa_hip.backward_saved(pq, pk, v, g, out, saved), rfa_hip.backward(pq, pk, v, g)):
         for name, a, b in zip(("dq", "dk", "dv"), pair, want):
             assert _rel(a.float().cpu(), b) <= GRAD_RTOL, (nseg, name)
+
+
+def _random_cases(count, seed):
+    g = torch.Generator().manual_seed(seed)
+    dims = [(64, 32), (64, 64), (64, 128), (128, 32), (128, 64), (128, 128)]       # (d, D): K = 2D in {64, 128, 256}
+    cases = []
+    for i in range(count):
+        T = int(torch.randint(1, 700, (1,), generator=g))
+        B = int(torch.randint(1, 4, (1,), generator=g))
+        H = int(torch.randint(1, 4, (1,), generator=g))
+        d, D = dims[int(torch.randint(0, len(dims), (1,), generator=g))]
+        cases.append((T, B, H, d, D, 7000 + i))
+    return cases
+
+
+@pytest.mark.parametrize("T,B,H,d,D,seed", _random_cases(16, 424242))
+def test_seeded_random_shapes(T, B, H, d, D, seed):
+    """Sixteen shapes drawn once from a fixed seed (lengths 1..699, 1..3 batch entries and heads, every
+    supported width pair): output, saved-pair and plain-pair gradients against the oracle."""
+    from rfa_amd import rfa_hip
+    cpu = _features(T, B, H, d, D, seed)
+    pq, pk, v, g = (t.cuda() for t in cpu)
+    print(f"causal random T={T} B={B} H={H} d={d} D={D}", flush=True)
+    ref = _oracle_fwd(*cpu[:3])
+    want = _oracle_bwd(*cpu)
+    out, saved = rfa_hip.forward_save(pq, pk, v)
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_ATOL
+    for pair in (rfa_hip.backward_saved(pq, pk, v, g, out, saved), rfa_hip.backward(pq, pk, v, g)):
+        for name, a, b in zip(("dq", "dk", "dv"), pair, want):
+            assert torch.isfinite(a).all(), name
+            assert _rel(a.float().cpu(), b) <= GRAD_RTOL, (name, _rel(a.float().cpu(), b))
