@@ -402,7 +402,7 @@ int launch_masked_fwd(const rfa::half_t* q, const rfa::half_t* k, const rfa::hal
     auto kern = rfa::k_masked_fwd<KD, DH>;
     if (int rc = set_lds(kern, Cfg::kLds)) return rc;
     const int nblk = (T + rfa::kChunk - 1) / rfa::kChunk;
-    RFA_LAUNCH(MASKED_FWD, kern, dim3(N * nblk), dim3(256), Cfg::kLds, st, q, k, v, pad, amask, out, rsum, T, Tp, N, H);
+    RFA_LAUNCH(MASKED_FWD, kern, dim3(N * (amask ? (nblk + 1) / 2 : nblk)), dim3(256), Cfg::kLds, st, q, k, v, pad, amask, out, rsum, T, Tp, N, H);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -420,11 +420,11 @@ int launch_masked_bwd(const rfa::half_t* q, const rfa::half_t* k, const rfa::hal
                rsum, ghat, gz, rows);
     auto kq = rfa::k_masked_dq<KD, DH>;
     if (int rc = set_lds(kq, Cfg::kLds)) return rc;
-    RFA_LAUNCH(MASKED_DQ, kq, dim3(N * nblk), dim3(256), Cfg::kLds, st, (const rfa::half_t*)ghat, (const float*)gz, k,
+    RFA_LAUNCH(MASKED_DQ, kq, dim3(N * (amask ? (nblk + 1) / 2 : nblk)), dim3(256), Cfg::kLds, st, (const rfa::half_t*)ghat, (const float*)gz, k,
                v, pad, amask, dq, T, Tp, N, H);
     auto kk = rfa::k_masked_dkdv<KD, DH>;
     if (int rc = set_lds(kk, Cfg::kLds)) return rc;
-    RFA_LAUNCH(MASKED_DKDV, kk, dim3(N * nblk), dim3(256), Cfg::kLds, st, q, k, v, (const rfa::half_t*)ghat,
+    RFA_LAUNCH(MASKED_DKDV, kk, dim3(N * (amask_t ? (nblk + 1) / 2 : nblk)), dim3(256), Cfg::kLds, st, q, k, v, (const rfa::half_t*)ghat,
                (const float*)gz, pad, amask_t, dk, dv, T, Tp, N, H);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -953,6 +953,9 @@ int rfa_cross_state_backward(const void* phi_k, const void* v, const uint8_t* ke
 // ---- quadratic form with explicit masks ---------------------------------------------------
 static int check_masked(const char* fn, int64_t T, int64_t Tp, int64_t B, int H, int K, int d, const void* amask) {
     if (int rc = check_cross_dims(fn, T, B, H, K, d)) return rc;
+    if (T > (int64_t)64 * rfa::kMaxMaskBlocks)
+        return fail(RFA_ERR_UNSUPPORTED, "%s: at most %d steps in the quadratic form (got %lld)", fn, 64 * rfa::kMaxMaskBlocks,
+                    (long long)T);
     if (amask && (Tp < T || Tp % 64 != 0))
         return fail(RFA_ERR_BAD_SHAPE, "%s: the attn_mask row stride must be T rounded up to a multiple of 64 (got %lld for T=%lld)",
                     fn, (long long)Tp, (long long)T);

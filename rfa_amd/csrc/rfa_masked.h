@@ -63,11 +63,50 @@ __device__ __forceinline__ uint32_t mask_word(const uint8_t* __restrict__ m, int
 }
 
 // ---------------------------------------------------------------------------
-// forward.  grid = N * nblk (nblk = ceil(T / 64)); wave w owns queries [i0 + 16w, i0 + 16w + 16).
+// forward, one block of 64 queries (nblk = ceil(T / 64) blocks per sequence); wave w owns queries [i0 + 16w, i0 + 16w + 16).
 // rsum (may be NULL) receives r_t, fp32 [T][N], for the backward pass.
 // ---------------------------------------------------------------------------
+// Blocks of 64 mask columns that a workgroup can skip: skip[b] != 0 when every entry of the
+// 64 x 64 tile (rows r0 .. r0 + 63, columns 64 b ..) of the byte mask m ([T][Tp]) is set.  Rows past
+// T count as set.  For the causal mask this is every block above the diagonal, half of the work.
+// All 256 threads take part (one 16-byte piece of a tile each, eight tiles in flight); ends with a
+// workgroup barrier.  m == NULL: nothing is skipped.
+constexpr int kMaxMaskBlocks = 1024;
+
+__device__ __forceinline__ void masked_tile_skip(const uint8_t* __restrict__ m, int r0, int T, int Tp, int nblk,
+                                                 unsigned char* skip, int tid) {
+    if (!m) {
+        for (int b = tid; b < nblk; b += 256) skip[b] = 0;
+        __syncthreads();
+        return;
+    }
+    const int r = r0 + (tid >> 2);
+    const uint8_t* mrow = m + (int64_t)min(r, T - 1) * Tp + 16 * (tid & 3);
+    for (int b0 = 0; b0 < nblk; b0 += 8) {
+        uint4 x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = *reinterpret_cast<const uint4*>(mrow + 64 * min(b0 + u, nblk - 1));
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            // no zero byte in any of the four words <=> all 16 entries set
+            auto full = [](uint32_t v) { return ((v - 0x01010101u) & ~v & 0x80808080u) == 0u; };
+            const bool set = r >= T || (full(x[u].x) && full(x[u].y) && full(x[u].z) && full(x[u].w));
+            const int all = __syncthreads_and(set ? 1 : 0);
+            if (tid == 0 && b0 + u < nblk) skip[b0 + u] = all ? 1 : 0;
+        }
+    }
+    __syncthreads();
+}
+
+// first block at or after b that is not skipped (nblk if none); uniform over the workgroup
+__device__ __forceinline__ int next_live_block(const unsigned char* skip, int b, int nblk) {
+    while (b < nblk && skip[b]) ++b;
+    return b;
+}
+
 template <int KD, int DH>
-__global__ __launch_bounds__(256) void k_masked_fwd(
+__device__ __forceinline__ void masked_fwd_block(const int n, const int i0,
+    
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const uint8_t* __restrict__ pad_mask, const uint8_t* __restrict__ attn_mask, half_t* __restrict__ out,
     float* __restrict__ rsum, int T, int Tp, int N, int H) {
@@ -82,7 +121,6 @@ __global__ __launch_bounds__(256) void k_masked_fwd(
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
     const int nblk = (T + C - 1) / C;
-    const int n = blockIdx.x / nblk, i0 = (int)(blockIdx.x % nblk) * C;
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
     const half_t* kb = k + (int64_t)n * KD;
     const half_t* vb = v + (int64_t)n * DH;
@@ -96,27 +134,30 @@ __global__ __launch_bounds__(256) void k_masked_fwd(
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) bq[ks] = *reinterpret_cast<const h8*>(qrow + 32 * ks + 8 * G);
     }
+    __shared__ unsigned char skip[kMaxMaskBlocks];
+    masked_tile_skip(attn_mask, i0, T, Tp, nblk, skip, tid);
     ChunkRegs<KD> rk;
     ChunkRegs<DH> rv;
-    chunk_g2r<KD>(rk, kb, k_stride, T, tid);
-    chunk_g2r<DH>(rv, vb, v_stride, T, tid);
-    if (prow) chunk_mask_rows<KD>(rk, prow, tid);
+    auto prefetch = [&](int jb) {
+        const int t0 = jb * C;
+        chunk_g2r<KD>(rk, kb + (int64_t)t0 * k_stride, k_stride, T - t0, tid);
+        chunk_g2r<DH>(rv, vb + (int64_t)t0 * v_stride, v_stride, T - t0, tid);
+        if (prow) chunk_mask_rows<KD>(rk, prow + t0, tid);
+    };
+    int jb = next_live_block(skip, 0, nblk);
+    if (jb < nblk) prefetch(jb);
 
     f4 acc[NCT];
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) acc[ct] = f4_zero();
     float rpart = 0.f;
 
-    for (int jb = 0; jb < nblk; ++jb) {
+    while (jb < nblk) {
         chunk_r2s<KD>(rk, Ks, LDQ, tid);
         chunk_r2s<DH>(rv, Vs, LDV, tid);
         __syncthreads();
-        if (jb + 1 < nblk) {
-            const int t0 = (jb + 1) * C;
-            chunk_g2r<KD>(rk, kb + (int64_t)t0 * k_stride, k_stride, T - t0, tid);
-            chunk_g2r<DH>(rv, vb + (int64_t)t0 * v_stride, v_stride, T - t0, tid);
-            if (prow) chunk_mask_rows<KD>(rk, prow + t0, tid);
-        }
+        const int jb_next = next_live_block(skip, jb + 1, nblk);
+        if (jb_next < nblk) prefetch(jb_next);
         f4 at[4];   // A^T tiles (m = j, n = i)
 #pragma unroll
         for (int jt = 0; jt < 4; ++jt) {
@@ -137,6 +178,7 @@ __global__ __launch_bounds__(256) void k_masked_fwd(
                 acc[ct] = mfma32(col_split8(Vs, LDV, 32 * jp, 16 * ct, lane), ba, acc[ct]);
         }
         __syncthreads();
+        jb = jb_next;
     }
 
     const float r = sum_over_groups(rpart);
@@ -190,7 +232,8 @@ __global__ __launch_bounds__(256) void k_masked_bwd_prep(const half_t* __restric
 // keys need no mask here: their phi_k rows are read as zero, so they add nothing to dphi_q.
 // ---------------------------------------------------------------------------
 template <int KD, int DH>
-__global__ __launch_bounds__(256) void k_masked_dq(
+__device__ __forceinline__ void masked_dq_block(const int n, const int i0,
+    
     const half_t* __restrict__ ghat, const float* __restrict__ gz, const half_t* __restrict__ k,
     const half_t* __restrict__ v, const uint8_t* __restrict__ pad_mask, const uint8_t* __restrict__ attn_mask,
     half_t* __restrict__ dq, int T, int Tp, int N, int H) {
@@ -205,7 +248,6 @@ __global__ __launch_bounds__(256) void k_masked_dq(
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
     const int nblk = (T + C - 1) / C;
-    const int n = blockIdx.x / nblk, i0 = (int)(blockIdx.x % nblk) * C;
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
     const half_t* kb = k + (int64_t)n * KD;
     const half_t* vb = v + (int64_t)n * DH;
@@ -221,26 +263,29 @@ __global__ __launch_bounds__(256) void k_masked_dq(
         for (int cs = 0; cs < NCS; ++cs) bg[cs] = *reinterpret_cast<const h8*>(ghat + tn * DH + 32 * cs + 8 * G);
         gzi = gz[tn];
     }
+    __shared__ unsigned char skip[kMaxMaskBlocks];
+    masked_tile_skip(attn_mask, i0, T, Tp, nblk, skip, tid);
     ChunkRegs<KD> rk;
     ChunkRegs<DH> rv;
-    chunk_g2r<KD>(rk, kb, k_stride, T, tid);
-    chunk_g2r<DH>(rv, vb, v_stride, T, tid);
-    if (prow) chunk_mask_rows<KD>(rk, prow, tid);
+    auto prefetch = [&](int jb) {
+        const int t0 = jb * C;
+        chunk_g2r<KD>(rk, kb + (int64_t)t0 * k_stride, k_stride, T - t0, tid);
+        chunk_g2r<DH>(rv, vb + (int64_t)t0 * v_stride, v_stride, T - t0, tid);
+        if (prow) chunk_mask_rows<KD>(rk, prow + t0, tid);
+    };
+    int jb = next_live_block(skip, 0, nblk);
+    if (jb < nblk) prefetch(jb);
 
     f4 acc[NKT];   // dQ^T tiles (m = k, n = i)
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt) acc[kt] = f4_zero();
 
-    for (int jb = 0; jb < nblk; ++jb) {
+    while (jb < nblk) {
         chunk_r2s<KD>(rk, Ks, LDQ, tid);
         chunk_r2s<DH>(rv, Vs, LDV, tid);
         __syncthreads();
-        if (jb + 1 < nblk) {
-            const int t0 = (jb + 1) * C;
-            chunk_g2r<KD>(rk, kb + (int64_t)t0 * k_stride, k_stride, T - t0, tid);
-            chunk_g2r<DH>(rv, vb + (int64_t)t0 * v_stride, v_stride, T - t0, tid);
-            if (prow) chunk_mask_rows<KD>(rk, prow + t0, tid);
-        }
+        const int jb_next = next_live_block(skip, jb + 1, nblk);
+        if (jb_next < nblk) prefetch(jb_next);
         f4 pt[4];   // P^T tiles (m = j, n = i)
 #pragma unroll
         for (int jt = 0; jt < 4; ++jt) {
@@ -260,6 +305,7 @@ __global__ __launch_bounds__(256) void k_masked_dq(
                 acc[kt] = mfma32(col_split8(Ks, LDQ, 32 * jp, 16 * kt, lane), bp, acc[kt]);
         }
         __syncthreads();
+        jb = jb_next;
     }
     if (ti < T) {
         half_t* drow = dq + ((int64_t)ti * N + n) * KD;
@@ -274,7 +320,8 @@ __global__ __launch_bounds__(256) void k_masked_dq(
 // dphi_k = 0 (the gradient of masked_fill) and dv = 0 (its weights are zero).
 // ---------------------------------------------------------------------------
 template <int KD, int DH>
-__global__ __launch_bounds__(256) void k_masked_dkdv(
+__device__ __forceinline__ void masked_dkdv_block(const int n, const int j0,
+    
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ ghat, const float* __restrict__ gz, const uint8_t* __restrict__ pad_mask,
     const uint8_t* __restrict__ attn_mask_t, half_t* __restrict__ dk, half_t* __restrict__ dv, int T, int Tp,
@@ -291,7 +338,6 @@ __global__ __launch_bounds__(256) void k_masked_dkdv(
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
     const int nblk = (T + C - 1) / C;
-    const int n = blockIdx.x / nblk, j0 = (int)(blockIdx.x % nblk) * C;
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
     const half_t* qb = q + (int64_t)n * KD;
     const half_t* gb = ghat + (int64_t)n * DH;
@@ -315,7 +361,10 @@ __global__ __launch_bounds__(256) void k_masked_dkdv(
         chunk_g2r<DH>(rg, gb + (int64_t)t0 * v_stride, v_stride, T - t0, tid);
         gz_next = gz[(int64_t)(t0 + min(tid & (C - 1), rg.rows - 1)) * N + n];
     };
-    prefetch(0);
+    __shared__ unsigned char skip[kMaxMaskBlocks];
+    masked_tile_skip(attn_mask_t, j0, T, Tp, nblk, skip, tid);
+    int ib = next_live_block(skip, 0, nblk);
+    if (ib < nblk) prefetch(ib * C);
 
     f4 acck[NKT], accv[NCT];   // dK^T (m = k, n = s), dV^T (m = c, n = s)
 #pragma unroll
@@ -323,12 +372,13 @@ __global__ __launch_bounds__(256) void k_masked_dkdv(
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) accv[ct] = f4_zero();
 
-    for (int ib = 0; ib < nblk; ++ib) {
+    while (ib < nblk) {
         chunk_r2s<KD>(rq, Qs, LDQ, tid);
         chunk_r2s<DH>(rg, Gs, LDV, tid);
         if (tid < C) gzs[tid] = tid < rg.rows ? gz_next : 0.f;
         __syncthreads();
-        if (ib + 1 < nblk) prefetch((ib + 1) * C);
+        const int ib_next = next_live_block(skip, ib + 1, nblk);
+        if (ib_next < nblk) prefetch(ib_next * C);
         f4 a_[4], p_[4];   // tiles (m = t, n = s)
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
@@ -361,6 +411,7 @@ __global__ __launch_bounds__(256) void k_masked_dkdv(
                 acck[kt] = mfma32(col_split8(Qs, LDQ, 32 * ip, 16 * kt, lane), bp, acck[kt]);
         }
         __syncthreads();
+        ib = ib_next;
     }
     if (tj < T) {
         half_t* krow = dk + ((int64_t)tj * N + n) * KD;
@@ -371,5 +422,54 @@ __global__ __launch_bounds__(256) void k_masked_dkdv(
         for (int ct = 0; ct < NCT; ++ct) *reinterpret_cast<h4*>(vrow + 16 * ct + 4 * G) = to_h4(accv[ct]);
     }
 }
+
+// ---------------------------------------------------------------------------
+// Kernels.  With an attention mask, grid = N * ceil(nblk / 2): a workgroup takes row blocks p and
+// nblk - 1 - p of one sequence, one after the other.  With a causal mask block p has p + 1 live
+// column blocks, so every workgroup does the same work (nblk + 1 tiles); without that pairing the
+// last row blocks set the kernel time and skipping the masked tiles would not shorten it.
+// Without a mask nothing is skipped and grid = N * nblk, one row block per workgroup.
+// ---------------------------------------------------------------------------
+#define RFA_MASKED_PAIR(CALL, PAIRED)                                          \
+    const int nblk = (T + kChunk - 1) / kChunk;                                \
+    const int per_seq = (PAIRED) ? (nblk + 1) / 2 : nblk;                      \
+    const int n = blockIdx.x / per_seq, p = blockIdx.x % per_seq;              \
+    CALL(p * kChunk);                                                          \
+    if ((PAIRED) && nblk - 1 - p != p) {                                       \
+        __syncthreads();                                                       \
+        CALL((nblk - 1 - p) * kChunk);                                         \
+    }
+
+template <int KD, int DH>
+__global__ __launch_bounds__(256) void k_masked_fwd(
+    const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    const uint8_t* __restrict__ pad_mask, const uint8_t* __restrict__ attn_mask, half_t* __restrict__ out,
+    float* __restrict__ rsum, int T, int Tp, int N, int H) {
+#define RFA_CALL_BLOCK(R0) masked_fwd_block<KD, DH>(n, R0, q, k, v, pad_mask, attn_mask, out, rsum, T, Tp, N, H)
+    RFA_MASKED_PAIR(RFA_CALL_BLOCK, attn_mask != nullptr)
+#undef RFA_CALL_BLOCK
+}
+
+template <int KD, int DH>
+__global__ __launch_bounds__(256) void k_masked_dq(
+    const half_t* __restrict__ ghat, const float* __restrict__ gz, const half_t* __restrict__ k,
+    const half_t* __restrict__ v, const uint8_t* __restrict__ pad_mask, const uint8_t* __restrict__ attn_mask,
+    half_t* __restrict__ dq, int T, int Tp, int N, int H) {
+#define RFA_CALL_BLOCK(R0) masked_dq_block<KD, DH>(n, R0, ghat, gz, k, v, pad_mask, attn_mask, dq, T, Tp, N, H)
+    RFA_MASKED_PAIR(RFA_CALL_BLOCK, attn_mask != nullptr)
+#undef RFA_CALL_BLOCK
+}
+
+template <int KD, int DH>
+__global__ __launch_bounds__(256) void k_masked_dkdv(
+    const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    const half_t* __restrict__ ghat, const float* __restrict__ gz, const uint8_t* __restrict__ pad_mask,
+    const uint8_t* __restrict__ attn_mask_t, half_t* __restrict__ dk, half_t* __restrict__ dv, int T, int Tp,
+    int N, int H) {
+#define RFA_CALL_BLOCK(R0) masked_dkdv_block<KD, DH>(n, R0, q, k, v, ghat, gz, pad_mask, attn_mask_t, dk, dv, T, Tp, N, H)
+    RFA_MASKED_PAIR(RFA_CALL_BLOCK, attn_mask_t != nullptr)
+#undef RFA_CALL_BLOCK
+}
+#undef RFA_MASKED_PAIR
 
 }  // namespace rfa

@@ -233,6 +233,11 @@ def _masked_case(T, B, H, d, D, seed, with_pad, mask_kind):
         am = torch.zeros(T, T)
         am[(i[None, :] > i[:, None]) | (i[:, None] - i[None, :] >= 40)] = -1.0
         am[i % 7 == 3, 0] = -1.0
+    elif mask_kind == "stripes":    # whole 64 x 64 tiles masked, a fully masked row block, and a ragged edge
+        am = torch.zeros(T, T)
+        am[:64, :] = -1.0                       # queries 0..63 see nothing: zero output rows
+        am[:, 128:192] = -1.0                   # keys 128..191 hidden from everybody
+        am[200:, :70] = -1.0                    # a masked region that ends inside a tile
     else:
         am = None
     return pq, pk, v, g, pad, am
@@ -245,6 +250,8 @@ def _masked_case(T, B, H, d, D, seed, with_pad, mask_kind):
     (200, 1, 2, 64, 64, True, "band"),
     (96, 2, 1, 128, 64, False, None),
     (70, 1, 1, 128, 128, True, "causal"),
+    (600, 1, 1, 64, 64, False, "causal"),      # ten blocks: more than one batch of tile flags
+    (330, 1, 2, 64, 64, True, "stripes"),
 ])
 def test_masked_rfa_matches_oracle_forward_and_backward(T, B, H, d, D, with_pad, mask_kind):
     """masked_rfa on the quadratic-form kernels against the oracle (causal_attention.py:57-109) and
