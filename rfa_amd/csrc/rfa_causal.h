@@ -1603,16 +1603,20 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
             }
 #pragma unroll
             for (int cs = 0; cs < DH / 32; ++cs) {
+                // the four row operands first: their LDS latency runs behind the conversion of the state
+                h8 bvv[4];
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) bvv[jt] = row_split8(Vs, LDV, 16 * jt + row, cs * 32, G);
+                __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
                 h8 hi[NKT], lo[NKT];
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt) acc_to_operand(RT[2 * cs][kt], RT[2 * cs + 1][kt], hi[kt], lo[kt]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
-                    h8 bvv = row_split8(Vs, LDV, 16 * jt + row, cs * 32, G);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(hi[kt], bvv, dkacc[kt][jt]);
+                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(hi[kt], bvv[jt], dkacc[kt][jt]);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(lo[kt], bvv, dkacc[kt][jt]);
+                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(lo[kt], bvv[jt], dkacc[kt][jt]);
                 }
             }
 #pragma unroll
@@ -1644,16 +1648,19 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
                 }
 #pragma unroll
             for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 bkk[4];
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) bkk[jt] = row_split8(Ks, LDQ, 16 * jt + row, ks * 32, G);
+                __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
                 h8 hi[NCT2], lo[NCT2];
 #pragma unroll
                 for (int ct = 0; ct < NCT2; ++ct) acc_to_operand(RR[2 * ks][ct], RR[2 * ks + 1][ct], hi[ct], lo[ct]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
-                    h8 bkk = row_split8(Ks, LDQ, 16 * jt + row, ks * 32, G);
 #pragma unroll
-                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(hi[ct], bkk, dvacc[ct][jt]);
+                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(hi[ct], bkk[jt], dvacc[ct][jt]);
 #pragma unroll
-                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(lo[ct], bkk, dvacc[ct][jt]);
+                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(lo[ct], bkk[jt], dvacc[ct][jt]);
                 }
             }
 #pragma unroll
