@@ -675,16 +675,20 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
             if (live) {
 #pragma unroll
                 for (int ks = 0; ks < KD / 32; ++ks) {
+                    // the four row operands first: their LDS latency runs behind the conversion of the state
+                    h8 bq[4];
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) bq[i4] = row_split8(Qs, LDQ, 16 * i4 + row, ks * 32, G);
+                    __builtin_amdgcn_sched_barrier(0);
                     h8 hi[NCT], lo[NCT];
 #pragma unroll
                     for (int ct = 0; ct < NCT; ++ct) acc_to_operand(S[2 * ks][ct], S[2 * ks + 1][ct], hi[ct], lo[ct]);
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) {
-                        h8 bq = row_split8(Qs, LDQ, 16 * i4 + row, ks * 32, G);
 #pragma unroll
-                        for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(hi[ct], bq, acc[i4][ct]);
+                        for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(hi[ct], bq[i4], acc[i4][ct]);
 #pragma unroll
-                        for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(lo[ct], bq, acc[i4][ct]);
+                        for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(lo[ct], bq[i4], acc[i4][ct]);
                     }
                 }
                 RFA_TICK_AT(11, 256);
@@ -1246,16 +1250,20 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
                 for (int it = 0; it < 4; ++it) yt[kt][it] = f4_zero();
 #pragma unroll
             for (int cs = 0; cs < DH / 32; ++cs) {
+                // the four row operands first: their LDS latency runs behind the conversion of the state
+                h8 bg[4];
+#pragma unroll
+                for (int it = 0; it < 4; ++it) bg[it] = row_split8(Gs, LDV, 16 * it + row, cs * 32, G);
+                __builtin_amdgcn_sched_barrier(0);
                 h8 hi[NKT], lo[NKT];
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt) acc_to_operand(ST[2 * cs][kt], ST[2 * cs + 1][kt], hi[kt], lo[kt]);
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
-                    h8 bg = row_split8(Gs, LDV, 16 * it + row, cs * 32, G);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(hi[kt], bg, yt[kt][it]);
+                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(hi[kt], bg[it], yt[kt][it]);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(lo[kt], bg, yt[kt][it]);
+                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(lo[kt], bg[it], yt[kt][it]);
                 }
             }
         }
