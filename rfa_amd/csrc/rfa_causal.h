@@ -392,16 +392,20 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
             }
 #pragma unroll
             for (int ks = 0; ks < KD / 32; ++ks) {
+                // the four row operands first: their LDS latency runs behind the conversion of the state
+                h8 bq[4];
+#pragma unroll
+                for (int it = 0; it < 4; ++it) bq[it] = row_split8(Qs, LDQ, 16 * it + row, ks * 32, G);
+                __builtin_amdgcn_sched_barrier(0);
                 h8 hi[NCT], lo[NCT];
 #pragma unroll
                 for (int ct = 0; ct < NCT; ++ct) acc_to_operand(S[2 * ks][ct], S[2 * ks + 1][ct], hi[ct], lo[ct]);
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
-                    h8 bq = row_split8(Qs, LDQ, 16 * it + row, ks * 32, G);
 #pragma unroll
-                    for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = mfma32(hi[ct], bq, acc[it][ct]);
+                    for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = mfma32(hi[ct], bq[it], acc[it][ct]);
 #pragma unroll
-                    for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = mfma32(lo[ct], bq, acc[it][ct]);
+                    for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = mfma32(lo[ct], bq[it], acc[it][ct]);
                 }
             }
             RFA_TICK(7);
@@ -904,16 +908,19 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
                 for (int it = 0; it < 4; ++it) yt[kt][it] = f4_zero();
 #pragma unroll
             for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 bg[4];
+#pragma unroll
+                for (int it = 0; it < 4; ++it) bg[it] = row_split8(Gs, LDV, 16 * it + row, cs * 32, G);
+                __builtin_amdgcn_sched_barrier(0);
                 h8 hi[NKT], lo[NKT];
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt) acc_to_operand(ST[2 * cs][kt], ST[2 * cs + 1][kt], hi[kt], lo[kt]);
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
-                    h8 bg = row_split8(Gs, LDV, 16 * it + row, cs * 32, G);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(hi[kt], bg, yt[kt][it]);
+                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(hi[kt], bg[it], yt[kt][it]);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(lo[kt], bg, yt[kt][it]);
+                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(lo[kt], bg[it], yt[kt][it]);
                 }
             }
             float e2[4] = {0.f, 0.f, 0.f, 0.f};
@@ -1868,16 +1875,19 @@ __device__ __forceinline__ void dkdv_role_dk(
             }
 #pragma unroll
             for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 bvv[4];
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) bvv[jt] = row_split8(Vs, LDV, 16 * jt + row, cs * 32, G);
+                __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
                 h8 hi[NKT], lo[NKT];
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt) acc_to_operand(RT[2 * cs][kt], RT[2 * cs + 1][kt], hi[kt], lo[kt]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
-                    h8 bvv = row_split8(Vs, LDV, 16 * jt + row, cs * 32, G);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(hi[kt], bvv, dkacc[kt][jt]);
+                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(hi[kt], bvv[jt], dkacc[kt][jt]);
 #pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(lo[kt], bvv, dkacc[kt][jt]);
+                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(lo[kt], bvv[jt], dkacc[kt][jt]);
                 }
             }
 #pragma unroll
@@ -2027,16 +2037,19 @@ __device__ __forceinline__ void dkdv_role_dv(
                 }
 #pragma unroll
             for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 bkk[4];
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) bkk[jt] = row_split8(Ks, LDQ, 16 * jt + row, ks * 32, G);
+                __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
                 h8 hi[NCT2], lo[NCT2];
 #pragma unroll
                 for (int ct = 0; ct < NCT2; ++ct) acc_to_operand(RR[2 * ks][ct], RR[2 * ks + 1][ct], hi[ct], lo[ct]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
-                    h8 bkk = row_split8(Ks, LDQ, 16 * jt + row, ks * 32, G);
 #pragma unroll
-                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(hi[ct], bkk, dvacc[ct][jt]);
+                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(hi[ct], bkk[jt], dvacc[ct][jt]);
 #pragma unroll
-                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(lo[ct], bkk, dvacc[ct][jt]);
+                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(lo[ct], bkk[jt], dvacc[ct][jt]);
                 }
             }
 #pragma unroll
