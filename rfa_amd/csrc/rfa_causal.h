@@ -1625,7 +1625,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
                 __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
                 h8 hi[NKT], lo[NKT];
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt) acc_to_operand(RT[2 * cs][kt], RT[2 * cs + 1][kt], hi[kt], lo[kt]);
+                for (int kt = 0; kt < NKT; ++kt) acc_to_operand<CAUSAL>(RT[2 * cs][kt], RT[2 * cs + 1][kt], hi[kt], lo[kt]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
 #pragma unroll
@@ -1669,7 +1669,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
                 __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
                 h8 hi[NCT2], lo[NCT2];
 #pragma unroll
-                for (int ct = 0; ct < NCT2; ++ct) acc_to_operand(RR[2 * ks][ct], RR[2 * ks + 1][ct], hi[ct], lo[ct]);
+                for (int ct = 0; ct < NCT2; ++ct) acc_to_operand<CAUSAL>(RR[2 * ks][ct], RR[2 * ks + 1][ct], hi[ct], lo[ct]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
 #pragma unroll
