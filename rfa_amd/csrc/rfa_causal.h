@@ -96,7 +96,8 @@ __global__ __launch_bounds__(64 * NW) void k_segment_state(
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
-    const int n = blockIdx.x / nseg_out, seg = blockIdx.x % nseg_out;
+    int n, seg;
+    seq_seg_of_block(blockIdx.x, N, nseg_out, n, seg);
     // MASKED is a compile-time switch: a run-time test around the mask loads would be a branch
     // between the chunk loads, and the compiler drains all outstanding loads at its join
     const uint8_t* mrow = MASKED ? pad_mask + (int64_t)(n / H) * T : nullptr;
@@ -233,7 +234,8 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
     const int row = lane & 15, G = lane >> 4;
     const int rb = w & 3, half = w >> 2;   // tile-phase role: 16-row block and which of its tiles
     constexpr int JPW = Cfg::JPW, NH = Cfg::NH;
-    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    int n, seg;
+    seq_seg_of_block(blockIdx.x, N, nseg, n, seg);
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
@@ -511,7 +513,8 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
     const int w = wave & 3;                    // wave inside its group
     const int tid = threadIdx.x & (NT - 1);    // thread inside its group
     const int row = lane & 15, G = lane >> 4;
-    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    int n, seg;
+    seq_seg_of_block(blockIdx.x, N, nseg, n, seg);
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
     const int n_chunks = t_end > t_begin ? (t_end - t_begin + C - 1) / C : 0;
@@ -776,7 +779,8 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
     const int row = lane & 15, G = lane >> 4;
     const int rb = w & 3, half = w >> 2;   // tile-phase role: 16-row block and which of its tiles
     constexpr int JPW = Cfg::JPW, NH = Cfg::NH;
-    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    int n, seg;
+    seq_seg_of_block(blockIdx.x, N, nseg, n, seg);
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
@@ -1119,7 +1123,8 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     const int nsq = N * nseg;
     const int koff = (int)(blockIdx.x / nsq) * KD;
     const int bid = blockIdx.x % nsq;
-    const int n = bid / nseg, seg = bid % nseg;
+    int n, seg;
+    seq_seg_of_block(bid, N, nseg, n, seg);
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
     const int64_t k_stride = (int64_t)N * KDG, v_stride = (int64_t)N * DH;
@@ -1399,7 +1404,8 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     const int ws = SPLIT ? (w & 3) : w;    // state-phase slice
     const bool do_dk = !SPLIT || w < 4, do_dv = !SPLIT || w >= 4;
     constexpr int JPW = Cfg::JPW, NH = Cfg::NH;
-    const int n = blockIdx.x / nseg, seg = blockIdx.x % nseg;
+    int n, seg;
+    seq_seg_of_block(blockIdx.x, N, nseg, n, seg);
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
@@ -1764,7 +1770,8 @@ __device__ __forceinline__ void dkdv_role_dk(
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
     const int rb = w & 3, half = w >> 2;
-    const int n = bid / nseg, seg = bid % nseg;
+    int n, seg;
+    seq_seg_of_block(bid, N, nseg, n, seg);
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
@@ -1940,7 +1947,8 @@ __device__ __forceinline__ void dkdv_role_dv(
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = lane & 15, G = lane >> 4;
     const int rb = w & 3, half = w >> 2;
-    const int n = bid / nseg, seg = bid % nseg;
+    int n, seg;
+    seq_seg_of_block(bid, N, nseg, n, seg);
     const int t_begin = seg * seg_len;
     const int t_end = min(T, t_begin + seg_len);
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;

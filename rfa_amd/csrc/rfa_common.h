@@ -181,6 +181,28 @@ __device__ __forceinline__ void fast_sincos(float x, float& s, float& c) {
 }
 
 // sum over the four 16-lane groups (lanes i, i+16, i+32, i+48)
+// Workgroup index -> (sequence, segment) of the scan kernels.  Workgroups are dealt to the 8 XCDs
+// round-robin by index, and the work of a workgroup grows with its segment number (it reads one
+// fp32 state total per earlier -- or, in the reverse sweep, later -- segment).  With the segments
+// of a sequence on consecutive indices and a segment count of 2, 4 or 8, every workgroup of the
+// heaviest kind lands on the same one, two or four XCDs, whose share of the memory fabric then
+// sets the kernel time.  Here the 8 sequences of a group go to the 8 XCDs and the segments of a
+// sequence stay on one XCD: every XCD gets the same mix, and the totals that several segments
+// of a sequence read are fetched into that XCD's L2 once.
+__device__ __forceinline__ void seq_seg_of_block(int b, int N, int nseg, int& n, int& seg) {
+    const int per_group = 8 * nseg, full = N / 8;
+    const int g = b / per_group;
+    if (g < full) {
+        const int r = b - g * per_group;
+        n = 8 * g + (r & 7);
+        seg = r >> 3;
+    } else {                       // the last N % 8 sequences
+        const int m = N - 8 * full, r = b - full * per_group;
+        n = 8 * full + r % m;
+        seg = r / m;
+    }
+}
+
 __device__ __forceinline__ float sum_over_groups(float x) {
     x += __shfl_xor(x, 16, 64);
     x += __shfl_xor(x, 32, 64);
