@@ -536,10 +536,18 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
         f4 zacc[NKTW];      // z for feature tiles kt = w*NKTW + a, element k = 16kt + 4G + e
 #pragma unroll
         for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
-        for (int s = prefixed ? seg : 0; s < (prefixed ? seg + 1 : seg); ++s) {
+        {
+            struct ZSlot { f4 z[NKTW]; };
+            sum_slots<4, ZSlot>(prefixed ? seg : 0, prefixed ? seg + 1 : seg,
+                [&](int s, ZSlot& t) {
 #pragma unroll
-            for (int a = 0; a < NKTW; ++a)
-                zacc[a] += *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * nseg + s) * KD + 16 * (w * NKTW + a) + 4 * G);
+                    for (int a = 0; a < NKTW; ++a)
+                        t.z[a] = *reinterpret_cast<const f4*>(wsZ + (int64_t)(n * nseg + s) * KD + 16 * (w * NKTW + a) + 4 * G);
+                },
+                [&](const ZSlot& t, float keep) {
+#pragma unroll
+                    for (int a = 0; a < NKTW; ++a) zacc[a] += keep * t.z[a];
+                });
         }
         const h8 ones = h8_ones();
         RFA_TICK_AT(0, 0);
@@ -638,12 +646,23 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
         for (int a = 0; a < NKT; ++a)
 #pragma unroll
             for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
-        for (int s = prefixed ? seg : 0; s < (prefixed ? seg + 1 : seg); ++s) {
-            const f4* sf = reinterpret_cast<const f4*>(wsS + ((int64_t)(n * nseg + s) * KD) * DH) + (int64_t)w * NKT * NCT * 64;
+        {
+            struct SSlot { f4 s[NKT][NCT]; };
+            constexpr int GRP = (NKT * NCT <= 8) ? 3 : 1;     // 32 registers per slot at K = 128, d = 64
+            sum_slots<GRP, SSlot>(prefixed ? seg : 0, prefixed ? seg + 1 : seg,
+                [&](int s, SSlot& t) {
+                    const f4* sf = reinterpret_cast<const f4*>(wsS + ((int64_t)(n * nseg + s) * KD) * DH) + (int64_t)w * NKT * NCT * 64;
 #pragma unroll
-            for (int kt = 0; kt < NKT; ++kt)
+                    for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-                for (int ct = 0; ct < NCT; ++ct) S[kt][ct] += sf[(kt * NCT + ct) * 64 + lane];
+                        for (int ct = 0; ct < NCT; ++ct) t.s[kt][ct] = sf[(kt * NCT + ct) * 64 + lane];
+                },
+                [&](const SSlot& t, float keep) {
+#pragma unroll
+                    for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                        for (int ct = 0; ct < NCT; ++ct) S[kt][ct] += keep * t.s[kt][ct];
+                });
         }
         RFA_TICK_AT(8, 256);
         for (int it = 0; it <= n_chunks; ++it) {
@@ -1446,15 +1465,26 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
         f4 sum[PER];
 #pragma unroll
         for (int it = 0; it < PER; ++it) sum[it] = f4_zero();
-        for (int s = s_first; s < s_last; ++s) {
-            const float* ri = wsR + ((int64_t)(n * state_stride + s) * KD) * DH;
+        {
+            struct RSlot { f4 s[PER]; f4 r[NKT]; };
+            constexpr int GRP = (PER + NKT <= 8) ? 3 : 1;
+            sum_slots<GRP, RSlot>(s_first, s_last,
+                [&](int s, RSlot& t) {
+                    const float* ri = wsR + ((int64_t)(n * state_stride + s) * KD) * DH;
 #pragma unroll
-            for (int it = 0; it < PER; ++it) sum[it] += *reinterpret_cast<const f4*>(ri + (int64_t)(tid + NT * it) * 4);
-            if (do_dk) {
+                    for (int it = 0; it < PER; ++it) t.s[it] = *reinterpret_cast<const f4*>(ri + (int64_t)(tid + NT * it) * 4);
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt)
-                    racc[kt] += *reinterpret_cast<const f4*>(wsr + (int64_t)(n * state_stride + s) * KD + ws * KS + 16 * kt + 4 * G);
-            }
+                    for (int kt = 0; kt < NKT; ++kt)
+                        t.r[kt] = *reinterpret_cast<const f4*>(wsr + (int64_t)(n * state_stride + s) * KD + ws * KS + 16 * kt + 4 * G);
+                },
+                [&](const RSlot& t, float keep) {
+#pragma unroll
+                    for (int it = 0; it < PER; ++it) sum[it] += keep * t.s[it];
+                    if (do_dk) {
+#pragma unroll
+                        for (int kt = 0; kt < NKT; ++kt) racc[kt] += keep * t.r[kt];
+                    }
+                });
         }
 #pragma unroll
         for (int it = 0; it < PER; ++it) {

@@ -181,6 +181,30 @@ __device__ __forceinline__ void fast_sincos(float x, float& s, float& c) {
 }
 
 // sum over the four 16-lane groups (lanes i, i+16, i+32, i+48)
+// Sum of the per-segment slots [s_first, s_last) of a carried state.  A loop that loads and adds one
+// slot per iteration pays one full memory latency per slot (the slots were written by other
+// workgroups of the previous kernel: they come from memory, about 1 us each).  Here GRP slots
+// are requested before the first one is added, branch-free: a slot index past the end is clamped
+// to the last slot and its values are multiplied by 0 (a load under a branch would make the
+// compiler wait for everything outstanding at the join).  The additions keep the slot order of
+// the plain loop.  load(s, slot) fills a Slot; add(slot, keep) accumulates keep * slot, keep = 1 or 0.
+template <int GRP, typename Slot, typename Load, typename Add>
+__device__ __forceinline__ void sum_slots(int s_first, int s_last, Load load, Add add) {
+    if (s_last - s_first == 1) {      // one slot (scanned totals, or the segment next to the end): no spare loads
+        Slot t;
+        load(s_first, t);
+        add(t, 1.0f);
+        return;
+    }
+    for (int s0 = s_first; s0 < s_last; s0 += GRP) {
+        Slot t[GRP];
+#pragma unroll
+        for (int u = 0; u < GRP; ++u) load(min(s0 + u, s_last - 1), t[u]);
+#pragma unroll
+        for (int u = 0; u < GRP; ++u) add(t[u], (s0 + u < s_last) ? 1.0f : 0.0f);
+    }
+}
+
 // Workgroup index -> (sequence, segment) of the scan kernels.  Workgroups are dealt to the 8 XCDs
 // round-robin by index, and the work of a workgroup grows with its segment number (it reads one
 // fp32 state total per earlier -- or, in the reverse sweep, later -- segment).  With the segments

@@ -57,6 +57,7 @@ SHAPES = [
     (130, 1, 1, 64, 128),    # K = 256
     (70, 65, 8, 64, 64),     # many sequences (N = 520), two chunks each
     (3000, 1, 2, 64, 64),    # long ragged sequence: 16 segments, last one short
+    (640, 1, 11, 64, 64),    # 11 sequences x 5 segments: one full group of 8 sequences and a rest of 3
     (1100, 1, 2, 128, 128),  # K = 256, d = 128: split dQ sweep, dK / dV in separate workgroups
 ]
 
