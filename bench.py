@@ -28,11 +28,11 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the bench configuration, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
 # passes summarised in profiles/bench_cfg2_hbm_traffic.md (counters scaled on the 512 MiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "k_segment_state": 25416351,
-    "k_causal_fwd": 63768431,
-    "k_causal_bwd_dq": 95826699,
-    "k_causal_bwd_dkdv": 89474273,
-    "k_decode_step": 68884880,
+    "k_segment_state": 25418517,
+    "k_causal_fwd": 59084176,
+    "k_causal_bwd_dq": 92570941,
+    "k_causal_bwd_dkdv": 86254696,
+    "k_decode_step": 68873673,
 }
 
 
