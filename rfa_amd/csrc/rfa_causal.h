@@ -576,8 +576,6 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
                 if (it + 1 < n_chunks) {
                     const int rows = t_end - t0 - C;
                     chunk_g2r<KD, NT>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-                    chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-                    chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
                 }
                 RFA_TICK_AT(3, 0);
                 // rows i in [16w, 16w+16) of A as A^T tiles (m=j, n=i), all four j tiles
@@ -589,6 +587,11 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
                     h8 bq = row8(Qs, LDQ, 16 * w + row, ks * 32, G);
 #pragma unroll
                     for (int a = 0; a < 4; ++a) at[a] = mfma32(row8(Ks, LDQ, 16 * a + row, ks * 32, G), bq, at[a]);
+                }
+                if (it + 1 < n_chunks) {      // second part of the next chunk's rows
+                    const int rows = t_end - t0 - C;
+                    chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+                    chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
                 }
                 float part = 0.f;
 #pragma unroll
@@ -1193,20 +1196,24 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     ChunkRegs<KD, NT> rq, rk;
     ChunkRegs<DH, NT> rv, rg, ro;
     float dn[VP];
-    auto prefetch = [&](int t0) {
+    auto prefetch_a = [&](int t0) {
         const int rows = t_end - t0;
         chunk_g2r<KD, NT>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
         chunk_g2r<DH, NT>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
         chunk_g2r<DH, NT>(ro, ob + (int64_t)t0 * v_stride, v_stride, rows, tid);
+    };
+    auto prefetch_b = [&](int t0) {
+        const int rows = t_end - t0;
         chunk_g2r<KD, NT>(rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
         chunk_g2r<DH, NT>(rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
 #pragma unroll
         for (int it = 0; it < VP; ++it) {
-            const int r_ = min((tid + NT * it) / PPR, rg.rows - 1);
+            const int r_ = min((tid + NT * it) / PPR, rv.rows - 1);
             dn[it] = den_raw[(int64_t)(t0 + r_) * N + n];
         }
     };
-    prefetch(t_begin);
+    prefetch_a(t_begin);
+    prefetch_b(t_begin);
     RFA_TICK(0);
 
     for (int t0 = t_begin; t0 < t_end; t0 += C) {
@@ -1245,7 +1252,15 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
         RFA_TICK(1);
         __syncthreads();
         RFA_TICK(2);
-        if (t0 + C < t_end) prefetch(t0 + C);
+        // The next chunk is requested in two parts, q, g, out here and k, v, den after the second
+        // barrier (0.8 us per config-2 sweep: the requests of the 256 workgroups, which run in step,
+        // are spread over the chunk).  The feature-half form keeps them together (1 % faster at
+        // T = 16384, K = 256, d = 128); in the dK/dV sweep the split changed nothing.
+        constexpr bool kSplitPrefetch = (KDG == KD);
+        if (t0 + C < t_end) {
+            prefetch_a(t0 + C);
+            if (!kSplitPrefetch) prefetch_b(t0 + C);
+        }
         RFA_TICK(3);
 
         // ---- phase A: P rows of this wave's row block (tiles jt = half*JPW + a); Y^T for the wave's feature slice
@@ -1301,6 +1316,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
         RFA_TICK(5);
         __syncthreads();
         RFA_TICK(6);
+        if (kSplitPrefetch && t0 + C < t_end) prefetch_b(t0 + C);
 
         // ---- phase D: dQ^T tiles (m=k, n=i), then the carried sums
         {
