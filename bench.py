@@ -28,11 +28,11 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the bench configuration, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
 # passes summarised in profiles/bench_cfg2_hbm_traffic.md (counters scaled on the 512 MiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "k_segment_state": 25418517,
-    "k_causal_fwd": 59084176,
-    "k_causal_bwd_dq": 92570941,
-    "k_causal_bwd_dkdv": 86254696,
-    "k_decode_step": 68873673,
+    "k_segment_state": 25430707,
+    "k_causal_fwd": 59032842,
+    "k_causal_bwd_dq": 92586190,
+    "k_causal_bwd_dkdv": 86253955,
+    "k_decode_step": 68884952,
 }
 
 
@@ -212,6 +212,22 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream):
                     "algorithmic_bytes_per_step": step_bytes,
                     "hbm_gbs": round(step_bytes * steps / (ms * 1e-3) / 1e9, 1),
                     "hbm_frac": round(step_bytes * steps / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    # The same 2048 steps as 32 calls of 64 steps, each preceded by an (untimed) elementwise pass that
+    # rewrites that call's q, k, v rows: in a decoder the rows of a step are written by the projection
+    # GEMMs just before the step, not read for the first time from HBM as in the loop above.
+    s.copy_(s0); z.copy_(z0)
+    row_bytes, call_steps, call_ms = N * d * 2, 64, 0.0
+    for c in range(steps // call_steps):
+        sl = slice(c * call_steps, (c + 1) * call_steps)
+        qs[sl].mul_(1.0); ks[sl].mul_(1.0); vs[sl].mul_(1.0)
+        off = c * call_steps * row_bytes
+        call_ms += _event_time_ms(torch, lambda: _lib.check(lib.rfa_incremental_fused(
+            p(qs) + off, p(ks) + off, p(vs) + off, p(W), O.SCALE, p(s), p(z), p(outs) + off, call_steps, B, H, D, d,
+            stream)), 1)
+    ex["decode"]["rows_written_just_before"] = {
+        "us_per_step": round(1e3 * call_ms / steps, 3),
+        "hbm_frac": round(step_bytes * steps / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "note": "64-step calls, q/k/v rows of each call rewritten on the device just before it (untimed)"}
     # parity of the first steps against the oracle on 2 heads
     s.copy_(s0); z.copy_(z0)
     _lib.check(lib.rfa_incremental_fused(p(qs), p(ks), p(vs), p(W), O.SCALE, p(s), p(z), p(outs), 8, B, H, D, d, stream))
