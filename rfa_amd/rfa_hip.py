@@ -331,7 +331,14 @@ def _mask_arg(mask, B: int, S: int, device):
         return None, None
     _require(tuple(mask.shape) == (B, S), ValueError, lambda: f"key_padding_mask must be [{B}, {S}] (got {tuple(mask.shape)})")
     _require(mask.device == device, RuntimeError, lambda: "key_padding_mask must be on the tensors' device")
-    m = (mask != 0).to(torch.uint8).contiguous()
+    # the kernels test the bytes for non-zero: a contiguous one-byte mask goes in as it is (no
+    # conversion kernels in front of the launch), anything else is reduced to 0/1 bytes first
+    if mask.dtype == torch.bool and mask.is_contiguous():
+        m = mask.view(torch.uint8)
+    elif mask.dtype == torch.uint8 and mask.is_contiguous():
+        m = mask
+    else:
+        m = (mask != 0).to(torch.uint8).contiguous()
     return m, m.data_ptr()
 
 

@@ -99,6 +99,38 @@ def test_cross_forward(S, T, B, H, d, D, lengths):
     assert (out - want).abs().max().item() <= OUT_ATOL
 
 
+def test_cross_mask_dtypes_agree():
+    """The padding mask may come as bool, as bytes (any non-zero value marks a padded key), as int64 or
+    as float, contiguous or not: one-byte contiguous masks reach the kernels as they are, the
+    others are reduced to 0/1 bytes first.  All of them must give the same bits."""
+    from rfa_amd import rfa_hip
+    pq, pk, v, g, mask = _cross_inputs(130, 70, 3, 2, 64, 64, 777, [130, 64, 7])
+    pk_c, v_c = pk.cuda(), v.cuda()
+    base_s, base_z = rfa_hip.cross_state(pk_c, v_c, mask.cuda())
+    ds = torch.randn_like(base_s)
+    dz = torch.randn_like(base_z)
+    base_dk, base_dv = rfa_hip.cross_state_backward(pk_c, v_c, ds, dz, mask.cuda())
+    wide = torch.zeros(3, 260, dtype=torch.bool)
+    wide[:, ::2] = mask
+    variants = {
+        "uint8 ones": mask.to(torch.uint8),
+        "uint8 sevens": mask.to(torch.uint8) * 7,
+        "int64": mask.to(torch.int64),
+        "float": mask.to(torch.float32),
+        "strided bool": wide[:, ::2],
+    }
+    for name, m in variants.items():
+        print(f"cross mask variant {name}", flush=True)
+        m = m.cuda()
+        if name == "strided bool":
+            m = wide.cuda()[:, ::2]
+            assert not m.is_contiguous()
+        s, z = rfa_hip.cross_state(pk_c, v_c, m)
+        assert torch.equal(s, base_s) and torch.equal(z, base_z), name
+        dk, dv = rfa_hip.cross_state_backward(pk_c, v_c, ds, dz, m)
+        assert torch.equal(dk, base_dk) and torch.equal(dv, base_dv), name
+
+
 def test_cross_readout_negative_denominator():
     """abs() in the denominator: flip the sign of z so that q.z < -1."""
     from rfa_amd import rfa_hip
