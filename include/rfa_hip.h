@@ -127,6 +127,19 @@ int rfa_causal_num_segments(int64_t T, int64_t N);
  * Supported: D in {32, 64, 128}, d in {64, 128} (rfa_feature_map_supported).
  * ------------------------------------------------------------------------- */
 int rfa_feature_map_supported(int D, int d);
+
+/* The matrix the feature map is taken with: W' = (sigma * W if sigma) / tau
+ *   (build_random_matrices, random_feature_attention/utils.py:90-97; two elementwise ATen
+ *   launches per call there, three more in the backward pass).  Same fp16 arithmetic: the
+ *   product is rounded to fp16 before the division.
+ *   w, out : fp16 [H, D, d];  sigma : fp16 [H, d] (the module's [H, 1, d] parameter,
+ *   causal_attention.py:165) or NULL;  tau != 0.
+ * rfa_build_random_matrices_backward: grad_out fp16 [H, D, d] -> dsigma fp16 [H, d] and/or
+ *   dw fp16 [H, D, d] (either may be NULL), as autograd derives them from those launches. */
+int rfa_build_random_matrices(const void* w, const void* sigma, float tau, void* out, int H, int D, int d,
+                              void* stream);
+int rfa_build_random_matrices_backward(const void* w, const void* sigma, const void* grad_out, float tau,
+                                       void* dsigma, void* dw, int H, int D, int d, void* stream);
 int rfa_feature_map_forward(const void* x, const void* w, void* phi, int64_t R, int H, int D, int d,
                             float scale, void* stream);
 size_t rfa_feature_map_backward_workspace_bytes(int64_t R, int H, int D, int d);

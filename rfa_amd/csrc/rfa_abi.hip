@@ -42,13 +42,13 @@ int fail(int code, const char* fmt, ...) {
 namespace prof {
 enum Id { SEG_STATE, CAUSAL_FWD, CAUSAL_BWD_DQ, CAUSAL_BWD_DKDV, CROSS_READOUT, CROSS_READOUT_BWD,
           CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, MASKED_FWD, MASKED_PREP, MASKED_DQ, MASKED_DKDV, PROJECT_PHI, WGRAD_PARTIAL, WGRAD_REDUCE, TOTALS_SCAN, ZERO_FILL,
-          SELFTEST, COUNT };
+          SELFTEST, BUILD_W, COUNT };
 const char* const kNames[COUNT] = {"k_segment_state", "k_causal_fwd", "k_causal_bwd_dq", "k_causal_bwd_dkdv",
                                    "k_cross_readout", "k_cross_readout_bwd", "k_cross_state_bwd", "k_decode_step",
                                    "k_feature_map_fwd", "k_feature_map_bwd", "k_feature_map_dw_reduce",
                                    "k_masked_fwd", "k_masked_bwd_prep", "k_masked_dq", "k_masked_dkdv", "k_project_phi",
                                    "k_weight_grad_partial", "k_weight_grad_reduce", "k_totals_scan",
-                                   "k_zero_f32", "k_selftest"};
+                                   "k_zero_f32", "k_selftest", "k_build_random_matrices"};
 struct Rec { int id; hipEvent_t a, b; };
 std::mutex mu;
 bool enabled = false;
@@ -1061,6 +1061,49 @@ int rfa_incremental_fused(const void* q, const void* k, const void* v, const voi
     RFA_DISPATCH_KD(K, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+// ---- random matrices ----------------------------------------------------------------
+static int check_matrix_dims(const char* fn, int H, int D, int d, float tau) {
+    if (H < 0 || D <= 0 || d <= 0 || H > (1 << 20) || D > (1 << 14) || d > (1 << 14))
+        return fail(RFA_ERR_BAD_SHAPE, "%s: bad sizes H=%d D=%d d=%d", fn, H, D, d);
+    if (!(tau != 0.f)) return fail(RFA_ERR_BAD_SHAPE, "%s: tau must be non-zero", fn);
+    return RFA_OK;
+}
+
+int rfa_build_random_matrices(const void* w, const void* sigma, float tau, void* out, int H, int D, int d,
+                              void* stream) {
+    if (int rc = check_matrix_dims("rfa_build_random_matrices", H, D, d, tau)) return rc;
+    if (H == 0) return RFA_OK;
+    if (!w || !out) return fail(RFA_ERR_NULL_POINTER, "rfa_build_random_matrices: NULL tensor pointer");
+    const int64_t total = (int64_t)H * D * d;
+    RFA_LAUNCH(BUILD_W, rfa::k_build_random_matrices, dim3((unsigned)((total + rfa::kThreads - 1) / rfa::kThreads)),
+               dim3(rfa::kThreads), 0, static_cast<hipStream_t>(stream), static_cast<const rfa::half_t*>(w),
+               static_cast<const rfa::half_t*>(sigma), static_cast<rfa::half_t*>(out), tau, D, d, total);
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
+}
+
+int rfa_build_random_matrices_backward(const void* w, const void* sigma, const void* grad_out, float tau,
+                                       void* dsigma, void* dw, int H, int D, int d, void* stream) {
+    if (int rc = check_matrix_dims("rfa_build_random_matrices_backward", H, D, d, tau)) return rc;
+    if (H == 0 || (!dsigma && !dw)) return RFA_OK;
+    if (!w || !grad_out) return fail(RFA_ERR_NULL_POINTER, "rfa_build_random_matrices_backward: NULL tensor pointer");
+    if (dsigma && !sigma)
+        return fail(RFA_ERR_NULL_POINTER, "rfa_build_random_matrices_backward: dsigma asked for without sigma");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* gh = static_cast<const rfa::half_t*>(grad_out);
+    if (dsigma)
+        RFA_LAUNCH(BUILD_W, rfa::k_build_random_matrices_dsigma, dim3((unsigned)H), dim3(rfa::kThreads), 0, st,
+                   static_cast<const rfa::half_t*>(w), gh, static_cast<rfa::half_t*>(dsigma), tau, D, d);
+    if (dw) {
+        const int64_t total = (int64_t)H * D * d;
+        RFA_LAUNCH(BUILD_W, rfa::k_build_random_matrices_dw, dim3((unsigned)((total + rfa::kThreads - 1) / rfa::kThreads)),
+                   dim3(rfa::kThreads), 0, st, static_cast<const rfa::half_t*>(sigma), gh,
+                   static_cast<rfa::half_t*>(dw), tau, D, d, total);
+    }
+    RFA_HIP_TRY(hipGetLastError());
+    return RFA_OK;
 }
 
 // ---- feature map --------------------------------------------------------------------

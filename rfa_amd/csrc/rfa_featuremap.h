@@ -322,4 +322,58 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_dw_reduce(const float*
     }
 }
 
+// W' = (sigma * W if sigma) / tau, one element per thread, in the reference's own arithmetic
+// (utils.py:90-97 on fp16 tensors: the product is rounded to fp16, then divided by tau in
+// fp32 and rounded again).  w, out: [H, D, d]; sigma: [H, d] (broadcast over D) or NULL.
+__global__ __launch_bounds__(kThreads) void k_build_random_matrices(const half_t* __restrict__ w,
+                                                                    const half_t* __restrict__ sigma,
+                                                                    half_t* __restrict__ out, float tau, int D,
+                                                                    int d, int64_t total) {
+    const int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= total) return;
+    half_t t = w[e];
+    if (sigma) t = (half_t)((float)sigma[(e / ((int64_t)D * d)) * d + e % d] * (float)t);
+    out[e] = (half_t)((float)t / tau);
+}
+
+// Gradient of k_build_random_matrices as autograd forms it from the same fp16 operations, with
+// t = fp16(g / tau):  dw = fp16(t * sigma) (t itself without sigma), one element per thread.
+__global__ __launch_bounds__(kThreads) void k_build_random_matrices_dw(const half_t* __restrict__ sigma,
+                                                                       const half_t* __restrict__ g,
+                                                                       half_t* __restrict__ dw, float tau, int D,
+                                                                       int d, int64_t total) {
+    const int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= total) return;
+    const half_t t = (half_t)((float)g[e] / tau);
+    dw[e] = sigma ? (half_t)((float)t * (float)sigma[(e / ((int64_t)D * d)) * d + e % d]) : t;
+}
+
+// dsigma[h][c] = fp16(sum_j fp16(t[h][j][c] * w[h][j][c])), fp32 sum.  One workgroup per head:
+// 64 columns at a time, the D rows dealt to the 4 waves, the 4 partial sums added in wave order.
+__global__ __launch_bounds__(kThreads) void k_build_random_matrices_dsigma(const half_t* __restrict__ w,
+                                                                           const half_t* __restrict__ g,
+                                                                           half_t* __restrict__ dsigma, float tau,
+                                                                           int D, int d) {
+    __shared__ float red[4][64];
+    const int h = blockIdx.x, lane = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const half_t* wh = w + (int64_t)h * D * d;
+    const half_t* gh = g + (int64_t)h * D * d;
+    for (int c0 = 0; c0 < d; c0 += 64) {
+        const int c = c0 + lane;
+        float acc = 0.f;
+        if (c < d) {
+#pragma unroll 8
+            for (int j = slice; j < D; j += 4) {     // unrolled: the loads of eight rows are in flight together
+                const half_t t = (half_t)((float)gh[j * d + c] / tau);
+                acc += (float)(half_t)((float)t * (float)wh[j * d + c]);
+            }
+        }
+        red[slice][lane] = acc;
+        __syncthreads();
+        if (slice == 0 && c < d)
+            dsigma[(int64_t)h * d + c] = (half_t)(((red[0][lane] + red[1][lane]) + red[2][lane]) + red[3][lane]);
+        __syncthreads();
+    }
+}
+
 }  // namespace rfa

@@ -203,6 +203,39 @@ def _check_feature_args(x: Tensor, w: Tensor):
     _require(x.device == w.device, RuntimeError, lambda: "x and random_matrices must be on one device")
 
 
+def build_random_matrices(w: Tensor, sigma: Optional[Tensor], tau: float) -> Tensor:
+    """W' = (sigma * w if sigma is not None) / tau in one launch; w fp16 [H, D, d], sigma fp16 [H, 1, d]."""
+    _check_half_cuda("random_matrices", w, 3)
+    H, D, d = w.shape
+    if sigma is not None:
+        _check_half_cuda("sigma", sigma, 3)
+        _require(tuple(sigma.shape) == (H, 1, d), ValueError, lambda: f"sigma must be [{H}, 1, {d}] (got {tuple(sigma.shape)})")
+    out = torch.empty_like(w)
+    with _on_device(w.device):
+        _lib.check(_lib.load().rfa_build_random_matrices(
+            w.data_ptr(), None if sigma is None else sigma.data_ptr(), float(tau), out.data_ptr(), H, D, d,
+            _stream_ptr(w.device)))
+    return out
+
+
+def build_random_matrices_backward(w: Tensor, sigma: Optional[Tensor], grad_out: Tensor, tau: float,
+                                   want_dsigma: bool, want_dw: bool):
+    """(dsigma fp16 [H, 1, d] or None, dw fp16 [H, D, d] or None) for grad_out fp16 [H, D, d]."""
+    _check_half_cuda("random_matrices", w, 3)
+    _check_half_cuda("grad_out", grad_out, 3)
+    _require(grad_out.shape == w.shape, ValueError, lambda: "grad_out must have the shape of random_matrices")
+    H, D, d = w.shape
+    want_dsigma = bool(want_dsigma and sigma is not None)
+    dsigma = torch.empty((H, 1, d), dtype=torch.float16, device=w.device) if want_dsigma else None
+    dw = torch.empty_like(w) if want_dw else None
+    with _on_device(w.device):
+        _lib.check(_lib.load().rfa_build_random_matrices_backward(
+            w.data_ptr(), None if sigma is None else sigma.data_ptr(), grad_out.data_ptr(), float(tau),
+            None if dsigma is None else dsigma.data_ptr(), None if dw is None else dw.data_ptr(), H, D, d,
+            _stream_ptr(w.device)))
+    return dsigma, dw
+
+
 def feature_map_forward(x: Tensor, w: Tensor, scale: float) -> Tensor:
     """phi [L, B, H, 2D] for x fp16 [L, B, H, d] and w fp16 [H, D, d]."""
     _check_feature_args(x, w)

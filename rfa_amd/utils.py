@@ -89,9 +89,40 @@ def sample_random_matrices(*, num_layers: int, num_heads: int, random_matrices: 
     return random_matrices[list(range(num_heads))]
 
 
+class _BuildRandomMatrices(torch.autograd.Function):
+    """W' = (sigma * W if sigma) / tau and its gradient, one launch each."""
+
+    @staticmethod
+    def forward(ctx, random_matrices: Tensor, sigma: Optional[Tensor], tau: float) -> Tensor:
+        w = random_matrices.contiguous()
+        sg = None if sigma is None else sigma.contiguous()
+        ctx.tau = tau
+        ctx.has_sigma = sg is not None
+        ctx.save_for_backward(w, *([sg] if sg is not None else []))
+        return rfa_hip.build_random_matrices(w, sg, tau)
+
+    @staticmethod
+    def backward(ctx, grad_out: Tensor):
+        w = ctx.saved_tensors[0]
+        sg = ctx.saved_tensors[1] if ctx.has_sigma else None
+        dsigma, dw = rfa_hip.build_random_matrices_backward(
+            w, sg, grad_out.contiguous(), ctx.tau, ctx.has_sigma and ctx.needs_input_grad[1], ctx.needs_input_grad[0])
+        return dw, dsigma, None
+
+
 def build_random_matrices(random_matrices: Tensor, tau: float, sigma: Optional[Tensor] = None,
                           reparam_proj: bool = False) -> Tensor:
-    """W' = (sigma * W if reparam_proj) / tau (reference utils.py:90-97)."""
+    """W' = (sigma * W if reparam_proj) / tau (reference utils.py:90-97).
+
+    fp16 tensors on a HIP device ([H, D, d] matrices, [H, 1, d] sigma) take one kernel launch
+    forward and one backward, in the arithmetic of the reference's two ATen launches; anything
+    else takes those ATen launches."""
+    sg = sigma if reparam_proj else None
+    if (random_matrices.is_cuda and random_matrices.dtype == torch.float16 and random_matrices.dim() == 3
+            and isinstance(tau, (int, float)) and tau != 0
+            and (sg is None or (sg.is_cuda and sg.dtype == torch.float16 and sg.dim() == 3
+                                and tuple(sg.shape) == (random_matrices.shape[0], 1, random_matrices.shape[2])))):
+        return _BuildRandomMatrices.apply(random_matrices, sg, float(tau))
     if reparam_proj:
         random_matrices = sigma * random_matrices
     return random_matrices / tau

@@ -59,6 +59,42 @@ def test_feature_map_backward(L, B, H, d, D):
     assert _rel(dw, rw) <= GRAD_RTOL, _rel(dw, rw)
 
 
+@pytest.mark.parametrize("H,D,d,tau,with_sigma", [(8, 64, 64, 1.0, True), (3, 32, 128, 0.7, True),
+                                                   (2, 128, 64, 2.0, False), (1, 5, 24, 1.3, True)])
+def test_build_random_matrices_matches_the_aten_chain(H, D, d, tau, with_sigma):
+    """W' = (sigma * W) / tau (reference utils.py:90-97): the one-launch form must give the bits of
+    the two ATen launches on the same fp16 tensors, and gradients that agree with autograd through
+    them (the column sums of dsigma are taken in another order, hence a tolerance there)."""
+    from rfa_amd.utils import build_random_matrices
+    print(f"build_random_matrices H={H} D={D} d={d} tau={tau} sigma={with_sigma}", flush=True)
+    W = _randn(H, D, d, seed=900 + D).half().cuda()
+    sigma = (1.0 + 0.3 * _randn(H, 1, d, seed=901 + d)).half().cuda() if with_sigma else None
+    g = _randn(H, D, d, seed=902).half().cuda()
+    # reference chain with autograd
+    Wr = W.clone().requires_grad_(True)
+    sr = sigma.clone().requires_grad_(True) if with_sigma else None
+    ref = (sr * Wr if with_sigma else Wr) / tau
+    ref.backward(g)
+    # fused
+    Wf = W.clone().requires_grad_(True)
+    sf = sigma.clone().requires_grad_(True) if with_sigma else None
+    got = build_random_matrices(random_matrices=Wf, tau=tau, sigma=sf, reparam_proj=with_sigma)
+    assert type(got.grad_fn).__name__.startswith("_BuildRandomMatrices")
+    assert torch.equal(got, ref)
+    got.backward(g)
+    assert torch.equal(Wf.grad, Wr.grad)
+    if with_sigma:
+        assert sf.grad.shape == sr.grad.shape
+        assert _rel(sf.grad.float().cpu(), sr.grad.float().cpu()) <= 2e-3
+    # without gradients asked for sigma only the matrix gradient is formed, and vice versa
+    sf2 = sigma.clone().requires_grad_(True) if with_sigma else None
+    out2 = build_random_matrices(random_matrices=W, tau=tau, sigma=sf2, reparam_proj=with_sigma)
+    assert torch.equal(out2, ref)
+    if with_sigma:
+        out2.backward(g)
+        assert torch.equal(sf2.grad, sf.grad)
+
+
 # ------------------------------------------------------------------------ cross
 def _cross_inputs(S, T, B, H, d, D, seed, lengths=None):
     W = O.make_w(d, D, H)
