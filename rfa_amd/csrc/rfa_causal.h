@@ -304,13 +304,9 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
         RFA_TICK(1);
         __syncthreads();
         RFA_TICK(2);
-        if (t0 + C < t_end) {
+        if (t0 + C < t_end) {      // the next chunk in two parts: q here, k and v after the tile phase
             const int rows = t_end - t0 - C;
             chunk_g2r<KD, NT>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-            if (CAUSAL) {
-                chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-                chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
-            }
         }
 
         RFA_TICK(3);
@@ -362,6 +358,11 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
                 for (int a = 0; a < JPW; ++a)
                     *reinterpret_cast<h4*>(As + (16 * rb + row) * LDA + 16 * (half * JPW + a) + 4 * G) = to_h4(at[a]);
             }
+        }
+        if (CAUSAL && t0 + C < t_end) {
+            const int rows = t_end - t0 - C;
+            chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
+            chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
         }
         RFA_TICK(4);
         __syncthreads();
@@ -2022,9 +2023,12 @@ __device__ __forceinline__ void dkdv_role_dv(
     ChunkRegs<KD, NT> rq, rk;
     ChunkRegs<DH, NT> rg;
     float inv_den[VP];
-    auto prefetch = [&](int t0) {
+    // the next chunk is requested in two parts, k after the first barrier, q, g, den after the second
+    auto prefetch_a = [&](int t0) {
+        chunk_g2r<KD, NT>(rk, kb + (int64_t)t0 * k_stride, k_stride, t_end - t0, tid);
+    };
+    auto prefetch_b = [&](int t0) {
         const int rows = t_end - t0;
-        chunk_g2r<KD, NT>(rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
         chunk_g2r<KD, NT>(rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
         chunk_g2r<DH, NT>(rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
 #pragma unroll
@@ -2034,7 +2038,8 @@ __device__ __forceinline__ void dkdv_role_dv(
         }
     };
     const int n_chunks = (t_end - t_begin + C - 1) / C;
-    prefetch(t_begin + (n_chunks - 1) * C);
+    prefetch_a(t_begin + (n_chunks - 1) * C);
+    prefetch_b(t_begin + (n_chunks - 1) * C);
     for (int ci = n_chunks - 1; ci >= 0; --ci) {
         const int t0 = t_begin + ci * C;
         chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
@@ -2043,7 +2048,7 @@ __device__ __forceinline__ void dkdv_role_dv(
         for (int it = 0; it < VP; ++it) inv_den[it] = 1.0f / fmaxf(inv_den[it], 1.0f);
         chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
         __syncthreads();
-        if (ci > 0) prefetch(t0 - C);
+        if (ci > 0) prefetch_a(t0 - C);
 
         // ---- A tiles (m=i, n=j) for column block rb, rows 16*(half*JPW + a)
         {
@@ -2071,6 +2076,7 @@ __device__ __forceinline__ void dkdv_role_dv(
             }
         }
         __syncthreads();
+        if (ci > 0) prefetch_b(t0 - C);
 
         // ---- dV^T tiles (m=c, n=j) and the carried sum
         {
