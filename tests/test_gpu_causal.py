@@ -215,3 +215,45 @@ def test_seeded_random_shapes(T, B, H, d, D, seed):
         for name, a, b in zip(("dq", "dk", "dv"), pair, want):
             assert torch.isfinite(a).all(), name
             assert _rel(a.float().cpu(), b) <= GRAD_RTOL, (name, _rel(a.float().cpu(), b))
+
+
+def test_two_threads_on_two_streams_agree_with_one():
+    """The library keeps no state between calls and launches on the caller's stream (the reference
+    launches on the legacy default stream, forward.cu:155): two host threads, each with its own
+    non-default stream, tensors and workspace, run the training pair at the same time and must get
+    the bits of the same calls made one after the other on the default stream."""
+    import threading
+    from rfa_amd import rfa_hip
+    cases = [_features(700, 1, 5, 64, 64, seed=8100), _features(450, 2, 3, 64, 32, seed=8101)]
+    gpu = [tuple(t.cuda() for t in c) for c in cases]
+    want = []
+    for pq, pk, v, g in gpu:
+        out, saved = rfa_hip.forward_save(pq, pk, v)
+        want.append((out, *rfa_hip.backward_saved(pq, pk, v, g, out, saved)))
+    torch.cuda.synchronize()
+    got = [None, None]
+    errors = []
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            pq, pk, v, g = gpu[i]
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    out, saved = rfa_hip.forward_save(pq, pk, v)
+                    grads = rfa_hip.backward_saved(pq, pk, v, g, out, saved)
+                got[i] = (out, *grads)
+            stream.synchronize()
+        except Exception as exc:      # surfaced in the main thread below
+            errors.append(exc)
+
+    print("causal two threads, two streams", flush=True)
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(2):
+        for a, b in zip(got[i], want[i]):
+            assert torch.equal(a, b)
