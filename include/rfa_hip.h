@@ -146,6 +146,14 @@ size_t rfa_feature_map_backward_workspace_bytes(int64_t R, int H, int D, int d);
 int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi, void* dx, float* dw,
                              int64_t R, int H, int D, int d, float scale, void* workspace,
                              size_t workspace_bytes, void* stream);
+/* Two tensors that went through the same w (phi(q) and phi(k) of a module, causal_attention.py:246-247)
+ *   differentiated in one launch: dx0, dx1 as above, dw = the sum of both contributions (what
+ *   autograd accumulates into w there). */
+size_t rfa_feature_map_backward_pair_workspace_bytes(int64_t R, int H, int D, int d);
+int rfa_feature_map_backward_pair(const void* x0, const void* x1, const void* w, const void* grad_phi0,
+                                  const void* grad_phi1, void* dx0, void* dx1, float* dw, int64_t R, int H,
+                                  int D, int d, float scale, void* workspace, size_t workspace_bytes,
+                                  void* stream);
 
 /* ---------------------------------------------------------------------------
  * Linear projections to heads with the feature map in the epilogue.

@@ -531,16 +531,19 @@ int launch_feature_fwd(const rfa::half_t* x, const rfa::half_t* w, rfa::half_t* 
 
 template <int D, int DH>
 int launch_feature_bwd(const rfa::half_t* x, const rfa::half_t* w, const rfa::half_t* gphi, rfa::half_t* dx,
+                       const rfa::half_t* x1, const rfa::half_t* gphi1, rfa::half_t* dx1,
                        float* dw, float* part, int R, int H, float scale, hipStream_t st) {
     using Cfg = rfa::FeatureCfg<D, DH>;
     const int nblk = feature_bwd_blocks(R, H);
+    const int ntens = x1 ? 2 : 1;       // two tensors through the same w: one launch, one reduction
     auto kern = rfa::k_feature_map_bwd<D, DH>;
     if (int rc = set_lds(kern, Cfg::kBwdLds)) return rc;
-    RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, part, R, H, scale);
+    RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H, ntens), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, x1, gphi1,
+               dx1, part, R, H, scale);
     const int64_t elems = (int64_t)H * D * DH;
     static_assert((D * DH) % 256 == 0, "dw reduce works on blocks of 256 elements");
     RFA_LAUNCH(FEATURE_DW_REDUCE, rfa::k_feature_map_dw_reduce, dim3((unsigned)(elems / 256)), dim3(rfa::kThreads), 0, st,
-                       part, dw, nblk, elems);
+                       part, dw, ntens * nblk, elems);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -1171,7 +1174,41 @@ int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi,
     auto* gh = static_cast<const rfa::half_t*>(grad_phi);
     auto* dxh = static_cast<rfa::half_t*>(dx);
     float* part = static_cast<float*>(workspace);
-#define RFA_CALL(DD, DH) launch_feature_bwd<DD, DH>(xh, wh, gh, dxh, dw, part, (int)R, H, scale, st)
+#define RFA_CALL(DD, DH) launch_feature_bwd<DD, DH>(xh, wh, gh, dxh, nullptr, nullptr, nullptr, dw, part, (int)R, H, scale, st)
+    RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+size_t rfa_feature_map_backward_pair_workspace_bytes(int64_t R, int H, int D, int d) {
+    return 2 * rfa_feature_map_backward_workspace_bytes(R, H, D, d);
+}
+
+int rfa_feature_map_backward_pair(const void* x0, const void* x1, const void* w, const void* grad_phi0,
+                                  const void* grad_phi1, void* dx0, void* dx1, float* dw, int64_t R, int H, int D,
+                                  int d, float scale, void* workspace, size_t workspace_bytes, void* stream) {
+    if (int rc = check_feature_dims("rfa_feature_map_backward_pair", R, H, D, d)) return rc;
+    if (!dw) return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward_pair: NULL dw");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (R == 0) {
+        zero_f32(dw, (int64_t)H * D * d, st);
+        return RFA_OK;
+    }
+    if (!x0 || !x1 || !w || !grad_phi0 || !grad_phi1 || !dx0 || !dx1)
+        return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward_pair: NULL tensor pointer");
+    if (!aligned16(x0) || !aligned16(x1) || !aligned16(w) || !aligned16(grad_phi0) || !aligned16(grad_phi1) ||
+        !aligned16(dx0) || !aligned16(dx1) || !aligned16(dw))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_feature_map_backward_pair: tensors must be 16-byte aligned");
+    const size_t need = rfa_feature_map_backward_pair_workspace_bytes(R, H, D, d);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+        return fail(RFA_ERR_WORKSPACE, "rfa_feature_map_backward_pair: workspace of %zu bytes required, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    float* part = static_cast<float*>(workspace);
+#define RFA_CALL(DD, DH)                                                                                         \
+    launch_feature_bwd<DD, DH>(static_cast<const rfa::half_t*>(x0), static_cast<const rfa::half_t*>(w),           \
+                               static_cast<const rfa::half_t*>(grad_phi0), static_cast<rfa::half_t*>(dx0),        \
+                               static_cast<const rfa::half_t*>(x1), static_cast<const rfa::half_t*>(grad_phi1),   \
+                               static_cast<rfa::half_t*>(dx1), dw, part, (int)R, H, scale, st)
     RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");

@@ -160,10 +160,18 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_fwd(
 // into dw_part[b][h][j][c] (fp32); k_feature_map_dw_reduce sums the nblk shares.
 // With n = ||x||, inv = 1/(n + 1e-3), dus = du * inv, y = dus W':
 //     dx = y - x * (x . y) / (n * (n + 1e-3))          (0 where n = 0)
+// gridDim.z = 2 differentiates two tensors that went through the same W' in one launch (phi(q) and
+// phi(k) of a module): workgroups with blockIdx.z = 1 take x1 / gphi1 / dx1 and the partial
+// sums nblk .. 2 nblk - 1, so that the reduction over 2 nblk shares yields the sum of both dW'.
 template <int D, int DH>
 __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
-    const half_t* __restrict__ x, const half_t* __restrict__ w, const half_t* __restrict__ gphi,
-    half_t* __restrict__ dx, float* __restrict__ dw_part, int R, int H, float scale) {
+    const half_t* __restrict__ x0, const half_t* __restrict__ w, const half_t* __restrict__ gphi0,
+    half_t* __restrict__ dx0, const half_t* __restrict__ x1, const half_t* __restrict__ gphi1,
+    half_t* __restrict__ dx1, float* __restrict__ dw_part, int R, int H, float scale) {
+    const bool second = blockIdx.z != 0;
+    const half_t* __restrict__ x = second ? x1 : x0;
+    const half_t* __restrict__ gphi = second ? gphi1 : gphi0;
+    half_t* __restrict__ dx = second ? dx1 : dx0;
     using Cfg = FeatureCfg<D, DH>;
     constexpr int LDW = Cfg::LDW, LDU = Cfg::LDU, LDG = Cfg::LDG;
     constexpr int NCTW = DH / 64;   // c-tiles of dW owned by one wave
@@ -285,7 +293,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
         __syncthreads();   // all reads of Xs / Us / Gs done before the next block overwrites them
     }
 
-    float* po = dw_part + ((int64_t)blockIdx.x * H + h) * D * DH;
+    float* po = dw_part + ((int64_t)(blockIdx.z * gridDim.x + blockIdx.x) * H + h) * D * DH;
 #pragma unroll
     for (int a = 0; a < NCTW; ++a)
 #pragma unroll

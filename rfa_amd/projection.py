@@ -54,9 +54,18 @@ class _ProjectHeads(torch.autograd.Function):
         dwf = None
         dys = []
         yi = 0
+        phi_idx = [p for p in range(n) if ctx.want_phi[p]]
+        pair = {}
+        if len(phi_idx) == 2:       # phi(q) and phi(k): both through the same w, one launch for the two
+            p0, p1 = phi_idx
+            dy0, dy1, dwf = rfa_hip.feature_map_backward_pair(ys[0], ys[1], wf, grads[p0].contiguous(),
+                                                              grads[p1].contiguous(), ctx.scale)
+            pair = {p0: dy0, p1: dy1}
         for p in range(n):
             g = grads[p].contiguous()
-            if ctx.want_phi[p]:
+            if p in pair:
+                dy = pair[p]
+            elif ctx.want_phi[p]:
                 dy, dw = rfa_hip.feature_map_backward(ys[yi], wf, g, ctx.scale)
                 yi += 1
                 dwf = dw if dwf is None else dwf + dw

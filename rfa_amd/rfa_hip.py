@@ -348,6 +348,29 @@ def feature_map_backward(x: Tensor, w: Tensor, grad_phi: Tensor, scale: float):
     return dx, dw
 
 
+def feature_map_backward_pair(x0: Tensor, x1: Tensor, w: Tensor, grad_phi0: Tensor, grad_phi1: Tensor, scale: float):
+    """Two tensors that went through the same w in one launch: (dx0, dx1 fp16 [L,B,H,d], dw fp32 [H,D,d]
+    = the sum of both contributions)."""
+    _check_feature_args(x0, w)
+    _check_feature_args(x1, w)
+    _require(x0.shape == x1.shape, ValueError, lambda: "the two tensors must have one shape")
+    L, B, H, d = x0.shape
+    D = w.shape[1]
+    for name, g in (("grad_phi0", grad_phi0), ("grad_phi1", grad_phi1)):
+        _check_half_cuda(name, g, 4)
+        _require(tuple(g.shape) == (L, B, H, 2 * D), ValueError, lambda: f"{name} {tuple(g.shape)} must be {(L, B, H, 2 * D)}")
+    lib = _lib.load()
+    dx0, dx1 = torch.empty_like(x0), torch.empty_like(x1)
+    dw = torch.empty((H, D, d), dtype=torch.float32, device=x0.device)
+    with _on_device(x0.device):
+        nbytes = lib.rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d)
+        ws = _workspace(nbytes, x0.device)
+        _lib.check(lib.rfa_feature_map_backward_pair(
+            x0.data_ptr(), x1.data_ptr(), w.data_ptr(), grad_phi0.data_ptr(), grad_phi1.data_ptr(), dx0.data_ptr(),
+            dx1.data_ptr(), dw.data_ptr(), L * B, H, D, d, float(scale), ws.data_ptr(), nbytes, _stream_ptr(x0.device)))
+    return dx0, dx1, dw
+
+
 # ---------------------------------------------------------------------------
 # cross attention
 # ---------------------------------------------------------------------------

@@ -59,6 +59,27 @@ def test_feature_map_backward(L, B, H, d, D):
     assert _rel(dw, rw) <= GRAD_RTOL, _rel(dw, rw)
 
 
+@pytest.mark.parametrize("L,B,H,d,D", FEATURE_SHAPES)
+def test_feature_map_backward_pair(L, B, H, d, D):
+    """Two tensors through the same W' in one launch: dx of each as from its own call (same bits),
+    dW' the sum of both (summed in another order, and checked against the oracle)."""
+    from rfa_amd import rfa_hip
+    x0 = (_randn(L, B, H, d, seed=30 + L) * 1.3).half().cuda()
+    x1 = (_randn(L, B, H, d, seed=31 + L) * 0.7).half().cuda()
+    w = (_randn(H, D, d, seed=32) * 0.9).half().cuda()
+    g0 = _randn(L, B, H, 2 * D, seed=33).half().cuda()
+    g1 = _randn(L, B, H, 2 * D, seed=34).half().cuda()
+    print(f"phi bwd pair L={L} B={B} H={H} d={d} D={D}", flush=True)
+    dx0, dx1, dw = rfa_hip.feature_map_backward_pair(x0, x1, w, g0, g1, O.SCALE)
+    sx0, sw0 = rfa_hip.feature_map_backward(x0, w, g0, O.SCALE)
+    sx1, sw1 = rfa_hip.feature_map_backward(x1, w, g1, O.SCALE)
+    assert torch.equal(dx0, sx0) and torch.equal(dx1, sx1)
+    assert _rel(dw.cpu(), (sw0 + sw1).cpu()) <= 1e-5
+    _, rw0 = O.random_project_backward(x0.float().cpu(), w.float().cpu(), g0.float().cpu())
+    _, rw1 = O.random_project_backward(x1.float().cpu(), w.float().cpu(), g1.float().cpu())
+    assert _rel(dw.cpu(), rw0 + rw1) <= GRAD_RTOL
+
+
 @pytest.mark.parametrize("H,D,d,tau,with_sigma", [(8, 64, 64, 1.0, True), (3, 32, 128, 0.7, True),
                                                    (2, 128, 64, 2.0, False), (1, 5, 24, 1.3, True)])
 def test_build_random_matrices_matches_the_aten_chain(H, D, d, tau, with_sigma):
