@@ -150,3 +150,15 @@ def test_random_matrix_generators():
     assert np.allclose(unit @ unit.T, np.eye(16), atol=1e-10)      # orthogonal directions
     np.random.seed(2)
     assert softmax_kernel_error(16, 2048, rrf(head_dim=16, proj_dim=2048), iters=5) < 0.15
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """No fallback of any kind: without the built library the first call raises ImportError that
+    says how to build it, and the ctypes table binds every declared entry point (a signature
+    missing there would only show up when that entry point is first called)."""
+    from rfa_amd import _lib
+    assert sorted(_lib.SIGNATURES) == sorted(s for s in _lib.declared_symbols() if s != "rfa_debug_phase_ticks")
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "librfa_hip.so"))
+    with pytest.raises(ImportError, match="rfa_amd.build"):
+        _lib.load()
