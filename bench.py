@@ -28,11 +28,11 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the bench configuration, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
 # passes summarised in profiles/bench_cfg2_hbm_traffic.md (counters scaled on the 512 MiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "k_segment_state": 25430780,
-    "k_causal_fwd": 58998267,
-    "k_causal_bwd_dq": 92586349,
-    "k_causal_bwd_dkdv": 86253209,
-    "k_decode_step": 68877775,
+    "k_segment_state": 25430824,
+    "k_causal_fwd": 59003656,
+    "k_causal_bwd_dq": 92586196,
+    "k_causal_bwd_dkdv": 86253280,
+    "k_decode_step": 68884953,
 }
 
 
