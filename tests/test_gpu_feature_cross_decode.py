@@ -188,6 +188,47 @@ def test_cross_mask_dtypes_agree():
         assert torch.equal(dk, base_dk) and torch.equal(dv, base_dv), name
 
 
+@pytest.mark.parametrize("pattern", ["left padded", "holes", "all but one", "everything"])
+def test_cross_arbitrary_padding_patterns(pattern):
+    """The source mask need not be a suffix: left-padded batches (fairseq's default for sources),
+    masked keys in the middle, a single live key, and a fully masked sequence (zero state, zero
+    gradients) against the oracle."""
+    from rfa_amd import rfa_hip
+    S, T, B, H, d, D = 200, 70, 3, 2, 64, 64
+    pq, pk, v, g, _ = _cross_inputs(S, T, B, H, d, D, 880)
+    gen = torch.Generator().manual_seed(881)
+    mask = torch.zeros(B, S, dtype=torch.bool)
+    if pattern == "left padded":
+        for b, L in enumerate([0, 37, 150]):
+            mask[b, :L] = True
+    elif pattern == "holes":
+        mask = torch.rand(B, S, generator=gen) < 0.4
+    elif pattern == "all but one":
+        mask[:] = True
+        mask[0, 199] = mask[1, 0] = mask[2, 64] = False
+    else:
+        mask[1] = True
+    print(f"cross mask pattern {pattern}", flush=True)
+    omask = mask.t()
+    rs, rz = O.cross_state(pk.float(), v.float(), omask)
+    s, z = rfa_hip.cross_state(pk.cuda(), v.cuda(), mask.cuda())
+    assert (s.cpu() - rs).abs().max().item() <= 1e-3 * max(1.0, rs.abs().max().item())
+    assert (z.cpu() - rz).abs().max().item() <= 1e-3 * max(1.0, rz.abs().max().item())
+    if pattern == "everything":
+        assert (s[1] == 0).all() and (z[1] == 0).all()
+    out = rfa_hip.cross_readout(pq.cuda(), s, z).float().cpu()
+    assert (out - O.cross_readout(pq.float(), rs, rz)).abs().max().item() <= OUT_ATOL
+    wq, wds, wdz = O.cross_readout_backward(pq.float(), rs, rz, g.float())
+    wk, wv = O.cross_state_backward(pk.float(), v.float(), wds, wdz, omask)
+    dq, ds, dz = rfa_hip.cross_readout_backward(pq.cuda(), s, z, g.cuda())
+    dk, dv = rfa_hip.cross_state_backward(pk.cuda(), v.cuda(), ds, dz, mask.cuda())
+    for name, got, want in (("dq", dq, wq), ("dk", dk, wk), ("dv", dv, wv)):
+        got = got.float().cpu()
+        assert torch.isfinite(got).all(), name
+        assert _rel(got, want) <= GRAD_RTOL, (name, _rel(got, want))
+    assert (dk.float().cpu()[omask] == 0).all()
+
+
 def test_cross_readout_negative_denominator():
     """abs() in the denominator: flip the sign of z so that q.z < -1."""
     from rfa_amd import rfa_hip
