@@ -139,4 +139,17 @@ __global__ __launch_bounds__(kThreads) void k_decode_step(
     }
 }
 
+// Reads n16 16-byte pieces and throws them away: brings rows that a later kernel reads with a
+// dependent, latency-bound access into the cache hierarchy at streaming speed.
+__global__ __launch_bounds__(kThreads) void k_touch_rows(const uint4* __restrict__ a, const uint4* __restrict__ b,
+                                                         const uint4* __restrict__ c, int64_t na, int64_t nb,
+                                                         int64_t nc) {
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    unsigned int acc = 0u;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < na; i += stride) acc ^= a[i].x;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nb; i += stride) acc ^= b[i].x;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nc; i += stride) acc ^= c[i].x;
+    asm volatile("" ::"v"(acc));
+}
+
 }  // namespace rfa
