@@ -23,7 +23,16 @@ def _require(cond: bool, exc, msg):
         raise exc(msg())
 
 
+_HALF = torch.float16
+
+
 def _check_half_cuda(name: str, t: Tensor, ndim: int):
+    # one cheap test for the common case; the individual checks below only name what is wrong
+    try:
+        if t.is_cuda and t.dtype is _HALF and t.dim() == ndim and t.is_contiguous():
+            return
+    except AttributeError:
+        pass
     _require(isinstance(t, Tensor), TypeError, lambda: f"{name} must be a torch.Tensor")
     _require(t.is_cuda, RuntimeError,
              lambda: f"{name} must live on a HIP device (got {t.device}); the kernels have no CPU path")
