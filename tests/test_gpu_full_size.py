@@ -131,3 +131,68 @@ def test_decode_full_size_config4():
                                          v.view(T, N, d)[:, sl].float().cpu())
     assert (dec.view(steps, N, d)[:, sl].float().cpu() - want[prefill:]).abs().max().item() <= 2e-3
     assert _rel(s.view(N, K, d)[sl].cpu(), ws) <= 1e-3
+
+
+@pytest.mark.parametrize("nseg", [None, 2])
+def test_element_offsets_beyond_32_bits(nseg, monkeypatch):
+    """phi tensors of 2.28e9 elements (4.6 GB each): every kernel forms offsets past 2**31 elements
+    and 2**32 bytes.  Sequences are independent, so a handful of them run as a small problem of
+    their own (same cut into segments) must reproduce their slices of the large run bit for bit;
+    the last sequence is also checked against the oracle."""
+    from rfa_amd import rfa_hip
+    T, B, H, d, D = 1088, 2050, 8, 64, 64          # 17 chunks of 64 steps, 16400 sequences
+    N, K = B * H, 2 * D
+    assert T * N * K > 2 ** 31
+    if nseg is not None:
+        monkeypatch.setenv("RFA_HIP_NSEG", str(nseg))
+    else:
+        monkeypatch.setenv("RFA_HIP_NSEG", "1")
+    print(f"offsets beyond 32 bits: T={T} N={N} K={K} d={d} segments={nseg or 1}", flush=True)
+    torch.manual_seed(77)
+    unit = lambda t: t / t.norm(dim=-1, keepdim=True)
+    W = O.make_w(d, D, H).half().cuda()
+    q = unit(torch.randn(T, B, H, d, device="cuda")).half()
+    k = unit(torch.randn(T, B, H, d, device="cuda")).half()
+    v = torch.randn(T, N, d, device="cuda").half()
+    g = torch.randn(T, N, d, device="cuda").half()
+    pq = rfa_hip.feature_map_forward(q, W, O.SCALE).view(T, N, K)
+    pk = rfa_hip.feature_map_forward(k, W, O.SCALE).view(T, N, K)
+    idx = torch.tensor([0, 1, N // 2 + 3, N - 2, N - 1], device="cuda")
+    # rows of phi at the far end of the tensor against a small call on those rows alone
+    far = rfa_hip.feature_map_forward(q[T - 3:].contiguous(), W, O.SCALE).view(3, N, K)
+    assert torch.equal(far, pq[T - 3:])
+    small = lambda t: t[:, idx].contiguous()
+    sq, sk, sv, sg = small(pq), small(pk), small(v), small(g)
+
+    out = rfa_hip.forward(pq, pk, v)
+    assert torch.equal(out[:, idx], rfa_hip.forward(sq, sk, sv))
+    grads = rfa_hip.backward(pq, pk, v, g)
+    for nm, big, ref in zip(("dq", "dk", "dv"), grads, rfa_hip.backward(sq, sk, sv, sg)):
+        assert torch.equal(big[:, idx], ref), nm
+    # the saving pair (what RFA.apply runs)
+    from rfa_amd.rfa import RFA
+    lq, lk, lv = (t.detach().requires_grad_(True) for t in (pq, pk, v))
+    o2 = RFA.apply(lq, lk, lv)
+    o2.backward(g)
+    mq, mk, mv = (t.detach().requires_grad_(True) for t in (sq, sk, sv))
+    o3 = RFA.apply(mq, mk, mv)
+    o3.backward(sg)
+    assert torch.equal(o2.detach()[:, idx], o3.detach())
+    for nm, big, ref in (("dq", lq.grad, mq.grad), ("dk", lk.grad, mk.grad), ("dv", lv.grad, mv.grad)):
+        assert torch.equal(big[:, idx], ref), nm
+    # oracle on the last sequence
+    cq, ck, cv, cg = (t[:, N - 1:].float().cpu() for t in (pq, pk, v, g))
+    assert (out[:, N - 1:].float().cpu() - O.causal_forward_chunked(cq, ck, cv)).abs().max().item() <= 2e-3
+    for nm, got, want in zip(("dq", "dk", "dv"), grads, O.causal_backward_chunked(cq, ck, cv, cg)):
+        assert _rel(got[:, N - 1:].float().cpu(), want) <= 1e-2, nm
+    del grads, o2, o3, lq, lk, lv
+
+    # cross attention over the same tensors (source = target length here)
+    s, z = rfa_hip.cross_state(pk.view(T, B, H, K), v.view(T, B, H, d))
+    bsel = torch.tensor([0, B // 2, B - 1], device="cuda")
+    bsmall = lambda t, w: t.view(T, B, H, w)[:, bsel].contiguous()
+    s1, z1 = rfa_hip.cross_state(bsmall(pk, K), bsmall(v, d))
+    assert torch.equal(s[bsel], s1) and torch.equal(z[bsel], z1)
+    co = rfa_hip.cross_readout(pq.view(T, B, H, K), s, z)
+    co1 = rfa_hip.cross_readout(bsmall(pq, K), s1, z1)
+    assert torch.equal(co.view(T, B, H, d)[:, bsel].reshape(co1.shape), co1)
