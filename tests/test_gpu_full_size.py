@@ -237,3 +237,39 @@ def test_element_offsets_beyond_32_bits_feature_backward_and_quadratic_form():
     g1 = rfa_hip.masked_backward(sm(pq), sm(pk), sm(v), sm(g), o1, r1, H, key_padding_mask=spad)
     for nm, big, ref in zip(("dq", "dk", "dv"), grads, g1):
         assert torch.equal(sm(big), ref), nm
+
+
+def test_element_offsets_beyond_32_bits_projections():
+    """Module projections at the same size class: rows are independent in the forward launch; the
+    weight gradient is a sum over all rows and is compared with a library GEMM in fp32."""
+    from rfa_amd import rfa_hip
+    L, B, E, H, d, D = 1088, 2050, 512, 8, 64, 64
+    print(f"offsets beyond 32 bits: projections L*B={L*B} E={E}", flush=True)
+    torch.manual_seed(79)
+    W = O.make_w(d, D, H).half().cuda()
+    x = torch.randn(L, B, E, device="cuda").half()
+    ws = [(torch.randn(E, E, device="cuda") * E ** -0.5).half() for _ in range(3)]
+    bs = [torch.randn(E, device="cuda").half().mul_(0.1), None, torch.randn(E, device="cuda").half().mul_(0.1)]
+    ys, phis = rfa_hip.project_feature_map(x, ws, bs, [True, True, False], W, H, O.SCALE)
+    assert phis[0].numel() > 2 ** 31 and phis[2] is None
+    ys1, phis1 = rfa_hip.project_feature_map(x[L - 2:].contiguous(), ws, bs, [True, True, False], W, H, O.SCALE)
+    for p in range(3):
+        assert torch.equal(ys[p][L - 2:], ys1[p]), p
+    for p in range(2):
+        assert torch.equal(phis[p][L - 2:], phis1[p]), p
+    del ys, phis
+
+    R, e_in, e_out = L * B, 1024, 128
+    xr = torch.randn(R, e_in, device="cuda").half()
+    assert xr.numel() > 2 ** 31
+    dy = torch.randn(R, e_out, device="cuda").half()
+    (dw,), (db,) = rfa_hip.linear_weight_grad(xr, [dy], [True])
+    want_w = torch.zeros(e_out, e_in, device="cuda")
+    step = 1 << 18
+    for r in range(0, R, step):
+        want_w += dy[r:r + step].float().t() @ xr[r:r + step].float()
+    assert _rel(dw.float(), want_w) <= 2e-3
+    assert _rel(db.float(), dy.float().sum(0)) <= 2e-3
+    # the rows past 2**31 elements count: without them the result differs
+    far = (2 ** 31) // e_in
+    assert _rel(dw.float(), want_w - dy[far:].float().t() @ xr[far:].float()) > 1e-2
