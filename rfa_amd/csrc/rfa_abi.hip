@@ -316,7 +316,12 @@ ScanPlan make_free_plan(int64_t T, int64_t N) {
     ScanPlan p{1, rfa::kChunk};
     if (T <= 0 || N <= 0) return p;
     const int64_t nchunks = (T + rfa::kChunk - 1) / rfa::kChunk;
-    int64_t want = (512 + N - 1) / N;
+    int64_t target = 512;      // workgroups to aim for; RFA_HIP_FREE_WG overrides (tuning sweeps)
+    if (const char* env = getenv("RFA_HIP_FREE_WG")) {
+        const long v = strtol(env, nullptr, 10);
+        if (v >= 1) target = v;
+    }
+    int64_t want = (target + N - 1) / N;
     if (want > nchunks) want = nchunks;
     if (want < 1) want = 1;
     const int64_t cps = (nchunks + want - 1) / want;
