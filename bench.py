@@ -354,6 +354,9 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream):
     mod.fuse_projections = True
     y_eager = mstep().detach().clone()
     gx_eager = mx.grad.detach().clone()
+    import warnings
+    # the warm-up below runs the step on a side stream on purpose (graph capture needs one)
+    warnings.filterwarnings("ignore", message="The AccumulateGrad node's stream does not match")
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
