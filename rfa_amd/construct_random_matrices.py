@@ -27,10 +27,17 @@ def orf(*, head_dim: int, proj_dim: int, rng=np.random) -> np.ndarray:
 
 
 def construct_random_matrices(feature_func, num_random_matrices: int, *, head_dim: int, proj_dim: int,
-                              seed=None) -> np.ndarray:
-    if seed is not None:
-        np.random.seed(seed)
-    return np.stack([feature_func(head_dim=head_dim, proj_dim=proj_dim) for _ in range(num_random_matrices)], axis=0)
+                              seed=None, rng=None) -> np.ndarray:
+    """Stack of num_random_matrices draws.  ``rng`` (a numpy RandomState) keeps the draws off the
+    global numpy generator; RandomState(s) yields the stream that np.random.seed(s) followed by the
+    module-level functions yields.  ``seed`` without ``rng`` seeds the global generator, which is
+    what the reference script does (construct_random_matrices.py:77)."""
+    if rng is None:
+        if seed is not None:
+            np.random.seed(seed)
+        rng = np.random
+    return np.stack([feature_func(head_dim=head_dim, proj_dim=proj_dim, rng=rng) for _ in range(num_random_matrices)],
+                    axis=0)
 
 
 def softmax_kernel_error(head_dim: int, proj_dim: int, random_matrix: np.ndarray, tau: float = 0.7,

@@ -36,31 +36,6 @@ def upgrade_state_dict_named(state_dict, name):
     return state_dict
 
 
-def get_rfa_attr(args):
-    """Defaults of the model flags (reference utils.py:20-28)."""
-    args.use_rfa = getattr(args, "use_rfa", False)
-    args.use_linfa = args.use_rfa      # attribute name the reference sets (utils.py:21)
-    args.cross_proj_dim = getattr(args, "cross_proj_dim", 64)
-    args.causal_proj_dim = getattr(args, "causal_proj_dim", 64)
-    args.cross_tau = getattr(args, "cross_tau", 1.0)
-    args.causal_tau = getattr(args, "causal_tau", 1.0)
-    args.reparam_proj = getattr(args, "reparam_proj", True)
-    args.cuda_causal_rfa = getattr(args, "cuda_causal_rfa", True)
-    return args
-
-
-def add_rfa_args(parser):
-    """Model flags (reference utils.py:31-46)."""
-    parser.add_argument("--use-rfa", action="store_true", help="use random feature attention")
-    parser.add_argument("--cross-proj-dim", type=int, metavar="N", help="projection size for cross rfa")
-    parser.add_argument("--causal-proj-dim", type=int, metavar="N", help="projection size for causal rfa")
-    parser.add_argument("--cross-tau", type=float, metavar="D", help="tau for cross rfa")
-    parser.add_argument("--causal-tau", type=float, metavar="D", help="tau for causal rfa")
-    parser.add_argument("--reparam-proj", action="store_true", help="reparameterize the random matrices")
-    parser.add_argument("--cuda-causal-rfa", action="store_true", help="use the fused kernel for causal rfa")
-    return parser
-
-
 def load_random_matrices(*, head_dim: int, proj_dim: int, dtype: torch.dtype = torch.half) -> Tensor:
     """[num_random_matrices, proj_dim, head_dim] as a frozen Parameter (reference utils.py:49-59).
 
@@ -73,7 +48,9 @@ def load_random_matrices(*, head_dim: int, proj_dim: int, dtype: torch.dtype = t
         mats = np.load(path)
     else:
         from .construct_random_matrices import construct_random_matrices, rrf
-        mats = construct_random_matrices(rrf, 500, head_dim=head_dim, proj_dim=proj_dim, seed=31415)
+        # a generator of its own: the caller's global numpy seed is left as it is
+        mats = construct_random_matrices(rrf, 500, head_dim=head_dim, proj_dim=proj_dim,
+                                         rng=np.random.RandomState(31415))
     return torch.nn.Parameter(torch.tensor(mats, dtype=dtype), requires_grad=False)
 
 

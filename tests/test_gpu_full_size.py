@@ -34,6 +34,7 @@ def _features_gpu(T, B, H, d, D, seed):
 ])
 def test_causal_full_size(name, T, B, H, d, D, n_check):
     from rfa_amd import rfa_hip
+    from rfa_amd.rfa import RFA
     print(f"{name}: causal fwd+bwd T={T} N={B*H} K={2*D} d={d}", flush=True)
     pq, pk, v, g = _features_gpu(T, B, H, d, D, seed=1234 + T)
     N = B * H
@@ -48,6 +49,27 @@ def test_causal_full_size(name, T, B, H, d, D, n_check):
         rq, rk, rv = O.causal_backward_chunked(cq, ck, cv, cg)
         for nm, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
             assert _rel(got[:, sl].float().cpu(), want) <= 1e-2, (nm, _rel(got[:, sl].float().cpu(), want))
+    # the training pair (forward_save / backward_saved: other kernels than the plain pair, and the
+    # ones RFA.apply and the benchmark run) and RFA.apply itself, on the same sequences
+    out_s, saved = rfa_hip.forward_save(pq, pk, v)
+    assert torch.equal(out_s, out)
+    sq, sk, sv = rfa_hip.backward_saved(pq, pk, v, g, out_s, saved)
+    lq, lk, lv = (t.detach().clone().requires_grad_(True) for t in (pq, pk, v))
+    out_a = RFA.apply(lq, lk, lv)
+    out_a.backward(g)
+    assert torch.equal(out_a.detach(), out)
+    assert torch.equal(lq.grad, sq) and torch.equal(lk.grad, sk) and torch.equal(lv.grad, sv)
+    assert all(torch.isfinite(t.float()).all() for t in (sq, sk, sv))
+    for sl in (slice(0, n_check), slice(N - n_check, N)):
+        cq, ck, cv, cg = (t[:, sl].float().cpu() for t in (pq, pk, v, g))
+        rq, rk, rv = O.causal_backward_chunked(cq, ck, cv, cg)
+        for nm, got, want in (("dq", sq, rq), ("dk", sk, rk), ("dv", sv, rv)):
+            assert _rel(got[:, sl].float().cpu(), want) <= 1e-2, ("saved pair", nm, _rel(got[:, sl].float().cpu(), want))
+    assert all(torch.equal(a, b) for a, b in zip(rfa_hip.backward_saved(pq, pk, v, g, out_s, saved), (sq, sk, sv)))
+    fo, fsaved = rfa_hip.forward_save(*(t.flip(1).contiguous() for t in (pq, pk, v)))
+    for a, b in zip(rfa_hip.backward_saved(*(t.flip(1).contiguous() for t in (pq, pk, v, g)), fo, fsaved), (sq, sk, sv)):
+        assert torch.equal(a, b.flip(1))
+    del lq, lk, lv, out_a, fo, fsaved
     # determinism: a second run is bit-identical
     assert torch.equal(rfa_hip.forward(pq, pk, v), out)
     assert all(torch.equal(a, b) for a, b in zip(rfa_hip.backward(pq, pk, v, g), (dq, dk, dv)))

@@ -1,7 +1,6 @@
 """CPU-only tests: the C-ABI library loads and exports every declared symbol,
 argument validation happens before any GPU work, and the host-side mirror of the
 reference API has the reference's names, defaults and parameter layout."""
-import argparse
 import ctypes
 
 import numpy as np
@@ -88,7 +87,7 @@ def test_formula_statements_match_oracle_on_cpu():
 
 def test_module_parameter_names_and_defaults():
     from rfa_amd import CausalAttention, CrossAttention, CrossAttentionProject, CrossAttentionState
-    from rfa_amd.utils import EPS, SCALE, add_rfa_args, get_rfa_attr
+    from rfa_amd.utils import EPS, SCALE
     assert EPS == 1.0 and SCALE == 0.1
     m = CausalAttention(embed_dim=128, num_heads=2, head_dim=64, proj_dim=64)
     assert sorted(m.state_dict()) == sorted(
@@ -107,11 +106,6 @@ def test_module_parameter_names_and_defaults():
     assert tuple(p.random_matrices.shape) == (500, 32, 64) and p.random_matrices.dtype == torch.float16
     assert tuple(p.random_matrices_eval.shape) == (2, 32, 64) and not p.random_matrices_eval.requires_grad
     assert CrossAttentionState._fields == ("s", "z", "random_matrices", "tau")
-    args = get_rfa_attr(argparse.Namespace())
-    assert (args.cross_proj_dim, args.causal_proj_dim, args.cross_tau, args.causal_tau) == (64, 64, 1.0, 1.0)
-    assert args.reparam_proj and args.cuda_causal_rfa and not args.use_rfa
-    ns = add_rfa_args(argparse.ArgumentParser()).parse_args(["--use-rfa", "--causal-proj-dim", "128"])
-    assert ns.use_rfa and ns.causal_proj_dim == 128
 
 
 def test_sample_and_build_random_matrices():
@@ -130,6 +124,24 @@ def test_sample_and_build_random_matrices():
     assert torch.equal(build_random_matrices(W, 4.0), W / 4.0)
 
 
+def test_load_random_matrices_leaves_the_global_numpy_generator_alone():
+    """The matrix file does not ship, so every CrossAttentionProject generates the matrices in
+    memory; that must not reseed numpy for the caller (sample_random_matrices and any numpy-based
+    shuffling draw from the global generator afterwards)."""
+    from rfa_amd.construct_random_matrices import construct_random_matrices, rrf
+    from rfa_amd.utils import load_random_matrices
+    draws = []
+    for seed in (7, 99):
+        np.random.seed(seed)
+        mats = load_random_matrices(head_dim=64, proj_dim=32)
+        draws.append(np.random.rand())
+    assert draws[0] != draws[1]
+    np.random.seed(7)
+    assert draws[0] == np.random.rand()
+    want = construct_random_matrices(rrf, 500, head_dim=64, proj_dim=32, seed=31415)   # the reference script's recipe
+    assert torch.equal(mats, torch.tensor(want, dtype=torch.half))
+
+
 def test_masked_rfa_has_no_cpu_path():
     """masked_rfa runs on the quadratic-form HIP kernels only: CPU tensors raise."""
     from rfa_amd.causal_attention import masked_rfa
@@ -144,6 +156,11 @@ def test_random_matrix_generators():
     a = construct_random_matrices(rrf, 3, head_dim=8, proj_dim=16, seed=31415)
     b = construct_random_matrices(rrf, 3, head_dim=8, proj_dim=16, seed=31415)
     assert a.shape == (3, 16, 8) and np.array_equal(a, b)
+    # a generator handed in: same stream as the seeded global one, global state untouched
+    np.random.seed(7)
+    before = np.random.get_state()[1].copy()
+    c = construct_random_matrices(rrf, 3, head_dim=8, proj_dim=16, rng=np.random.RandomState(31415))
+    assert np.array_equal(a, c) and np.array_equal(np.random.get_state()[1], before)
     np.random.seed(1)
     o = orf(head_dim=16, proj_dim=16)
     unit = o / np.linalg.norm(o, axis=1, keepdims=True)
