@@ -127,7 +127,7 @@ def main():
         "k_causal_bwd_dq": (2 * K + 3 * d) * 2 + K * 2 + 8,       # q, k, v, g, out in; dq out; den in, gz out
         "k_causal_bwd_dkdv": (2 * K + 2 * d) * 2 + 8 + (K + d) * 2,
     }
-    nseg = lib.rfa_causal_num_segments(T, N)
+    nseg = lib.rfa_causal_num_segments(T, N, K, d)
     units = {n_: N * T for n_ in per_tok}
     units["k_segment_state"] = N * T * (nseg - 1) // max(nseg, 1)
     dominant = max((n_ for n_ in kern_us if n_ in per_tok), key=lambda n_: totals[n_][0])

@@ -12,6 +12,7 @@
  *   - nothing is allocated by the library: kernels that need scratch memory
  *     take a caller-owned workspace whose size the matching *_workspace_bytes
  *     function reports (0 is a valid answer; then workspace may be NULL);
+ *     rfa_selftest_layout keeps its one result word in a static device variable;
  *   - K = 2 * proj_dim is the width of the feature vectors phi(q), phi(k);
  *     d = head_dim; N = bsz * num_heads.
  *
@@ -109,9 +110,35 @@ int rfa_causal_backward_saved(const void* q, const void* k, const void* v, const
                               void* dv, int64_t T, int64_t N, int K, int d, void* workspace,
                               size_t workspace_bytes, void* stream);
 
+/* A saved buffer describes itself: its first 256 bytes hold the plan of the forward call that
+ * wrote it (16 ints: magic, version, layout, K, d, segments, steps per segment, scanned-totals
+ * flag, T and N as two ints each, zeros), written on the device by that call.
+ * rfa_causal_backward_saved runs with the plan recorded on the host when a forward call of this
+ * process last wrote the buffer (whatever the tuning knobs say by then) and returns
+ * RFA_ERR_WORKSPACE if that call had another T, N, K or d.  For a buffer this process has no
+ * record of, it assumes the current plan and its kernels compare the header with it on the
+ * device: on a mismatch dq, dk, dv are filled with NaN rather than computed from totals laid out
+ * for another plan.  rfa_causal_backward_saved_workspace_bytes is the workspace that call needs
+ * for a given saved buffer (= rfa_causal_backward_workspace_bytes unless the knobs changed since
+ * the forward).  rfa_causal_saved_describe copies the 16 header ints to host memory and waits
+ * for the stream (a debugging aid).  No counterpart in the reference. */
+size_t rfa_causal_backward_saved_workspace_bytes(const void* saved, int64_t T, int64_t N, int K, int d);
+int rfa_causal_saved_describe(const void* saved, int32_t* words16, void* stream);
+
 /* Number of time segments the causal kernels cut a sequence into for the given
- * shape (>= 1).  Environment variable RFA_HIP_NSEG overrides the heuristic. */
-int rfa_causal_num_segments(int64_t T, int64_t N);
+ * shape on the current device (>= 1). */
+int rfa_causal_num_segments(int64_t T, int64_t N, int K, int d);
+
+/* Launch-heuristic overrides for sweeps and tests (process-wide; -1 restores the heuristic):
+ *   "nseg"  segments per sequence of the causal kernels (1..16)
+ *   "prefix"  1/0: consumers read pre-scanned segment totals / add the totals up themselves
+ *   "nseg_same"  1: the K = 256, d = 128 backward keeps the forward's segment length
+ *   "free_wg"  workgroups the cross-attention readout and state backward aim for
+ *   "project_streaming"  1: rfa_project_feature_map uses its streaming kernel for every shape
+ * Initial values come from the environment variables RFA_HIP_<NAME>, read once per process and
+ * never on the launch path.  No counterpart in the reference. */
+int rfa_tuning_set(const char* name, int value);
+int rfa_tuning_get(const char* name, int* value);
 
 /* ---------------------------------------------------------------------------
  * Feature map  phi(x) = scale * [sin(W x^), cos(W x^)],  x^ = x / (||x|| + 1e-3).
@@ -264,6 +291,16 @@ int rfa_incremental(const void* phi_q, const void* phi_k, const void* v, float* 
                     int64_t steps, int64_t N, int K, int d, void* stream);
 int rfa_incremental_fused(const void* q, const void* k, const void* v, const void* w, float scale, float* s,
                           float* z, void* out, int64_t steps, int64_t B, int H, int D, int d, void* stream);
+/* The same steps with the state read from s_in, z_in and the advanced state written to s_out,
+ * z_out (the first step reads the inputs, later steps advance the outputs in place), as the
+ * reference's `s = s + ...` leaves the caller's tensors alone (causal_attention.py:42-43).
+ * Same traffic as the in-place form; s_out, z_out may alias s_in, z_in. */
+int rfa_incremental_out(const void* phi_q, const void* phi_k, const void* v, const float* s_in, const float* z_in,
+                        float* s_out, float* z_out, void* out, int64_t steps, int64_t N, int K, int d,
+                        void* stream);
+int rfa_incremental_fused_out(const void* q, const void* k, const void* v, const void* w, float scale,
+                              const float* s_in, const float* z_in, float* s_out, float* z_out, void* out,
+                              int64_t steps, int64_t B, int H, int D, int d, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Per-kernel timing (no counterpart in the reference; used by bench.py).

@@ -35,7 +35,11 @@ SIGNATURES = {
     "rfa_shape_supported": (c_int, [c_int, c_int]),
     "rfa_selftest_layout": (c_int, [c_void_p]),
     "rfa_selftest_mfma_rate": (c_int, [c_int, c_int, c_void_p, ctypes.POINTER(ctypes.c_double), c_void_p]),
-    "rfa_causal_num_segments": (c_int, [c_int64, c_int64]),
+    "rfa_causal_num_segments": (c_int, [c_int64, c_int64, c_int, c_int]),
+    "rfa_tuning_set": (c_int, [c_char_p, c_int]),
+    "rfa_tuning_get": (c_int, [c_char_p, POINTER(c_int)]),
+    "rfa_causal_backward_saved_workspace_bytes": (c_size_t, [c_void_p, c_int64, c_int64, c_int, c_int]),
+    "rfa_causal_saved_describe": (c_int, [c_void_p, POINTER(ctypes.c_int32), c_void_p]),
     "rfa_causal_forward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
     "rfa_causal_forward": (c_int, [c_void_p] * 4 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "rfa_causal_prefill": (c_int, [c_void_p] * 6 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
@@ -69,6 +73,8 @@ SIGNATURES = {
     "rfa_profile_kernel_count": (c_int, []),
     "rfa_profile_get": (c_int, [c_int, POINTER(c_char_p), POINTER(c_double), POINTER(c_int64)]),
     "rfa_incremental_fused": (c_int, [c_void_p] * 4 + [c_float] + [c_void_p] * 3 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
+    "rfa_incremental_out": (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int, c_int, c_void_p]),
+    "rfa_incremental_fused_out": (c_int, [c_void_p] * 4 + [c_float] + [c_void_p] * 5 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
 }
 
 _lib = None
@@ -101,6 +107,36 @@ def declared_symbols() -> list:
     with open(HEADER_PATH) as f:
         text = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
     return sorted(set(re.findall(r"\b(rfa_[a-z0-9_]+)\s*\(", text)))
+
+
+def tuning_set(name: str, value: int) -> None:
+    """Override a launch heuristic of the library (-1 restores it); see rfa_tuning_set in the header."""
+    check(load().rfa_tuning_set(name.encode(), int(value)))
+
+
+def tuning_get(name: str) -> int:
+    v = c_int(0)
+    check(load().rfa_tuning_get(name.encode(), ctypes.byref(v)))
+    return v.value
+
+
+class tuning:
+    """``with tuning(nseg=2, prefix=1): ...`` sets knobs for the block and puts the old values back."""
+
+    def __init__(self, **knobs):
+        self.knobs = knobs
+        self.old = {}
+
+    def __enter__(self):
+        for name, value in self.knobs.items():
+            self.old[name] = tuning_get(name)
+            tuning_set(name, value)
+        return self
+
+    def __exit__(self, *exc):
+        for name, value in self.old.items():
+            tuning_set(name, value)
+        return False
 
 
 def profile_totals() -> dict:

@@ -47,19 +47,24 @@ def incremental_rfa(*, phi_q: Tensor, phi_k: Tensor, v: Tensor, s: Optional[Tens
         assert z is None
         s = torch.zeros((bsz, num_heads, feat, head_dim), device=v.device, dtype=torch.float32)
         z = torch.zeros((bsz, num_heads, feat), device=v.device, dtype=torch.float32)
+        s_new, z_new = s, z
     else:
         assert z is not None
-        if s.dtype != torch.float32 or z.dtype != torch.float32 or not inplace:
-            s = s.to(torch.float32, copy=True)
-            z = z.to(torch.float32, copy=True)
-        s, z = s.contiguous(), z.contiguous()
+        s_in, z_in = s, z
+        s, z = s.to(torch.float32).contiguous(), z.to(torch.float32).contiguous()
+        if inplace or (s is not s_in and z is not z_in):
+            s_new, z_new = s, z          # the caller's own tensors, or private fp32 copies: advance where they are
+        else:
+            # the kernel reads the caller's state and writes the advanced one elsewhere: no copy pass
+            s_new, z_new = torch.empty_like(s), torch.empty_like(z)
     n = bsz * num_heads
     attn = rfa_hip.incremental(
         phi_q.detach().to(torch.float16).contiguous().view(tgt_len, n, feat),
         phi_k.detach().to(torch.float16).contiguous().view(tgt_len, n, feat),
         v.detach().to(torch.float16).contiguous().view(tgt_len, n, head_dim),
-        s.view(n, feat, head_dim), z.view(n, feat))
-    return attn.to(v.dtype).view(tgt_len, bsz, num_heads * head_dim), s, z
+        s.view(n, feat, head_dim), z.view(n, feat),
+        None if s_new is s else s_new.view(n, feat, head_dim), None if z_new is z else z_new.view(n, feat))
+    return attn.to(v.dtype).view(tgt_len, bsz, num_heads * head_dim), s_new, z_new
 
 
 class _MaskedRFA(torch.autograd.Function):
@@ -167,6 +172,12 @@ class CausalAttention(nn.Module):
         self.upgrade_state_dict_named = upgrade_state_dict_named
         # q/k/v projections + view to heads + phi(q), phi(k) as one launch when the tensors allow it
         self.fuse_projections = True
+        # Decoding: the reference builds a new state tensor every step (causal_attention.py:42-43), so
+        # a caller may keep the tensors of an earlier step (a prefix shared between hypotheses, a
+        # roll-back).  False keeps that: each step writes its state into fresh tensors (the kernel
+        # reads one buffer and writes the other, no extra pass).  True advances the tensors under
+        # "prev_s" / "prev_z" where they are -- what a captured HIP graph of the step needs.
+        self.decode_inplace = False
 
     def reset_parameters(self):
         for proj in (self.q_proj, self.k_proj, self.v_proj, self.out_proj):
@@ -227,17 +238,24 @@ class CausalAttention(nn.Module):
                 s = s.view(bsz, self.num_heads, feat, self.head_dim)
                 z = z.view(bsz, self.num_heads, feat)
             else:
+                s_out = z_out = None
                 if s is None:
                     s = torch.zeros((bsz, self.num_heads, feat, self.head_dim), device=x.device, dtype=torch.float32)
                     z = torch.zeros((bsz, self.num_heads, feat), device=x.device, dtype=torch.float32)
                 else:
                     assert z is not None
+                    s_in, z_in = s, z
                     s = s.to(torch.float32).contiguous()
                     z = z.to(torch.float32).contiguous()
-                # feature map + state update + readout in one kernel per step; state advanced in place
+                    if not self.decode_inplace and (s is s_in or z is z_in):
+                        s_out, z_out = torch.empty_like(s), torch.empty_like(z)
+                # feature map + state update + readout in one kernel per step
                 attn = rfa_hip.incremental_fused(
                     q.detach().to(torch.float16).contiguous(), k.detach().to(torch.float16).contiguous(),
-                    v.detach().to(torch.float16).contiguous(), w.detach().to(torch.float16).contiguous(), SCALE, s, z)
+                    v.detach().to(torch.float16).contiguous(), w.detach().to(torch.float16).contiguous(), SCALE, s, z,
+                    s_out, z_out)
+                if s_out is not None:
+                    s, z = s_out, z_out
             attn = attn.to(x.dtype).view(tgt_len, bsz, embed_dim)
             saved_state["prev_s"], saved_state["prev_z"] = s, z
         else:

@@ -5,11 +5,13 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <unordered_map>
 #include <vector>
 
 #include "rfa_causal.h"
@@ -88,33 +90,149 @@ void launch(int id, F kern, dim3 grid, dim3 block, size_t lds, hipStream_t st, A
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// ---- tuning knobs --------------------------------------------------------------------
+// Process-wide overrides of the launch heuristics, for sweeps and for tests that must reach
+// every code path at small sizes.  -1 = the heuristic.  The environment is read once, when the
+// first knob is looked up, never on the launch path; rfa_tuning_set changes a knob afterwards.
+namespace tune {
+enum Key { NSEG, PREFIX, NSEG_SAME, FREE_WG, PROJECT_STREAMING, SLICED, COUNT };
+const char* const kNames[COUNT] = {"nseg", "prefix", "nseg_same", "free_wg", "project_streaming", "sliced"};
+const char* const kEnv[COUNT] = {"RFA_HIP_NSEG", "RFA_HIP_PREFIX", "RFA_HIP_NSEG_SAME", "RFA_HIP_FREE_WG",
+                                 "RFA_HIP_PROJECT_STREAMING", "RFA_HIP_SLICED"};
+std::atomic<int> value[COUNT];
+std::once_flag once;
+
+void init() {
+    for (int i = 0; i < COUNT; ++i) {
+        int v = -1;
+        if (const char* env = getenv(kEnv[i])) {
+            char* end = nullptr;
+            const long x = strtol(env, &end, 10);
+            if (end != env && x >= 0 && x <= (1 << 20)) v = (int)x;
+        }
+        value[i].store(v, std::memory_order_relaxed);
+    }
+}
+
+int get(Key k) {
+    std::call_once(once, init);
+    return value[k].load(std::memory_order_relaxed);
+}
+
+int find(const char* name) {
+    if (!name) return -1;
+    for (int i = 0; i < COUNT; ++i)
+        if (strcmp(name, kNames[i]) == 0) return i;
+    return -1;
+}
+}  // namespace tune
+
+// Compute units of the current device (256 on an MI355X in its default partition mode);
+// queried once per device.  Without a device (a host that only asks for buffer sizes) the
+// MI355X figure is assumed.
+int device_cus() {
+    constexpr int kMaxDev = 64;
+    static std::atomic<int> cache[kMaxDev];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    int cus = cache[dev].load(std::memory_order_relaxed);
+    if (cus <= 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+            (void)hipGetLastError();
+            cus = 256;
+        }
+        cache[dev].store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
+
 struct ScanPlan {
     int nseg;      // segments per sequence
     int seg_len;   // steps per segment (multiple of 64)
+    int prefixed;  // the consumers read one pre-scanned state (k_totals_scan) instead of adding up the
+                   // segment totals themselves
 };
 
-// Enough (sequence, segment) workgroups to cover the 256 CUs, at least two
+// Whether the consumers read one pre-scanned state instead of adding up the segment totals
+// themselves, (nseg - 1) / 2 states of K * d floats on average per workgroup: worth its pass over
+// the totals from 128 KiB of such reads on.
+bool use_scanned_totals(int nseg, int K, int d) {
+    if (nseg < 2) return false;
+    const int knob = tune::get(tune::PREFIX);
+    if (knob >= 0) return knob != 0;
+    return (int64_t)(nseg - 1) * K * d * 2 >= 128 * 1024;
+}
+
+// Enough (sequence, segment) workgroups to cover the compute units, at least two
 // chunks per segment, at most 16 segments (the consumer sums the totals of all
 // earlier segments).
-ScanPlan make_plan(int64_t T, int64_t N) {
-    ScanPlan p{1, rfa::kChunk};
+ScanPlan make_plan(int64_t T, int64_t N, int K, int d) {
+    ScanPlan p{1, rfa::kChunk, 0};
     if (T <= 0 || N <= 0) return p;
     const int64_t nchunks = (T + rfa::kChunk - 1) / rfa::kChunk;
-    int64_t want = (256 + N - 1) / N;
-    if (const char* env = getenv("RFA_HIP_NSEG")) {
-        const long v = strtol(env, nullptr, 10);
-        if (v >= 1) want = v;
+    int64_t want = (device_cus() + N - 1) / N;
+    const int knob = tune::get(tune::NSEG);
+    if (knob >= 1) {
+        want = knob;
     } else {
         if (want > nchunks / 2) want = nchunks / 2;
     }
-    if (want > 16) want = 16;
+    if (want > rfa::kMaxSegments) want = rfa::kMaxSegments;
     if (want > nchunks) want = nchunks;
     if (want < 1) want = 1;
     const int64_t cps = (nchunks + want - 1) / want;
     p.nseg = (int)((nchunks + cps - 1) / cps);
     p.seg_len = (int)(cps * rfa::kChunk);
+    p.prefixed = use_scanned_totals(p.nseg, K, d) ? 1 : 0;
     return p;
 }
+
+// ---- description of a saved-state buffer ---------------------------------------------
+constexpr size_t kSavedHeaderBytes = 256;
+enum SavedLayout { LAYOUT_SEGMENTS = 0 };
+
+rfa::PlanWords plan_words(int layout, int64_t T, int64_t N, int K, int d, const ScanPlan& p) {
+    rfa::PlanWords w{};
+    w.w[0] = rfa::kPlanMagic;
+    w.w[1] = 1;
+    w.w[2] = layout;
+    w.w[3] = K;
+    w.w[4] = d;
+    w.w[5] = p.nseg;
+    w.w[6] = p.seg_len;
+    w.w[7] = p.prefixed;
+    w.w[8] = (int)(T & 0xffffffff);
+    w.w[9] = (int)(T >> 32);
+    w.w[10] = (int)(N & 0xffffffff);
+    w.w[11] = (int)(N >> 32);
+    return w;
+}
+
+// What the last rfa_causal_forward_save wrote at each saved-buffer address, kept on the host so
+// that the backward call runs with that forward's plan whatever the knobs say by then.  A buffer
+// the table does not know (copied by the caller, written by another process) is taken to follow
+// the current plan; the backward kernels then check the header on the device.
+namespace registry {
+std::mutex mu;
+std::unordered_map<const void*, rfa::PlanWords> table;
+
+void put(const void* saved, const rfa::PlanWords& w) {
+    std::lock_guard<std::mutex> lk(mu);
+    if (table.size() >= 4096) table.clear();
+    table[saved] = w;
+}
+
+bool get(const void* saved, rfa::PlanWords* w) {
+    std::lock_guard<std::mutex> lk(mu);
+    auto it = table.find(saved);
+    if (it == table.end()) return false;
+    *w = it->second;
+    return true;
+}
+}  // namespace registry
 
 size_t align_up(size_t x) { return (x + 255) & ~size_t(255); }
 
@@ -157,16 +275,6 @@ int set_lds(Kern kern, size_t bytes) {
     return RFA_OK;
 }
 
-// Whether the consumers read one pre-scanned state (k_totals_scan) instead of adding up the
-// segment totals themselves, (nseg - 1) / 2 states of K * d floats on average per workgroup:
-// worth its pass over the totals from 128 KiB of such reads on.
-// RFA_HIP_PREFIX=0/1 overrides (the forward and the backward of a saved pair must agree).
-bool use_scanned_totals(int nseg, int K, int d) {
-    if (nseg < 2) return false;
-    if (const char* env = getenv("RFA_HIP_PREFIX")) return env[0] == '1';
-    return (int64_t)(nseg - 1) * K * d * 2 >= 128 * 1024;
-}
-
 template <bool REVERSE>
 void launch_totals_scan(float* a, int64_t Ma, float* b, int64_t Mb, int N, int nseg, hipStream_t st) {
     const int64_t threads = (Ma + Mb) / 4;
@@ -176,8 +284,8 @@ void launch_totals_scan(float* a, int64_t Ma, float* b, int64_t Mb, int N, int n
 
 template <int KD, int DH>
 int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, rfa::half_t* out,
-                   int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, float* savedS, float* savedZ,
-                   float* savedDen, float* final_s, float* final_z, hipStream_t st) {
+                   int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, int* savedHdr, float* savedS,
+                   float* savedZ, float* savedDen, float* final_s, float* final_z, hipStream_t st) {
     // the two-stage pipelined forward needs both chunk buffers in LDS: K <= 128
     constexpr bool PIPE = rfa::FwdPipeCfg<KD, DH>::kLds <= 160 * 1024;
     constexpr int NW = PIPE ? 4 : causal_waves(KD, DH);
@@ -193,42 +301,51 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
         RFA_LAUNCH(SEG_STATE, kern, dim3(N * (p.nseg - 1)), dim3(64 * NW), Cfg::kSegStateLds, st,
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
-    const int prefixed = use_scanned_totals(p.nseg, KD, DH) ? 1 : 0;
-    if (prefixed) launch_totals_scan<false>(wsS, (int64_t)KD * DH, wsZ, KD, N, p.nseg, st);
+    if (p.prefixed) launch_totals_scan<false>(wsS, (int64_t)KD * DH, wsZ, KD, N, p.nseg, st);
+    const rfa::PlanWords pw = plan_words(LAYOUT_SEGMENTS, T, N, KD, DH, p);
     if constexpr (PIPE) {
         auto kern = rfa::k_causal_fwd_pipe<KD, DH>;
         if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(512), rfa::FwdPipeCfg<KD, DH>::kLds, st, q, k, v, out,
-                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, prefixed);
+                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, p.prefixed, savedHdr, pw);
     } else {
         auto kern = rfa::k_causal_fwd<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q, k, v, out,
-                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, prefixed);
+                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, p.prefixed, savedHdr, pw);
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
+}
+
+// The cut into segments the backward sweeps use for a forward plan pf.  Where both sweeps run as two
+// workgroups per (sequence, segment) and the totals are scanned, the backward takes segments twice
+// as long: half as many workgroups already cover the compute units, in one round instead of two.
+ScanPlan backward_plan(const ScanPlan& pf, int K, int d, bool have_saved, int* s_ratio) {
+    ScanPlan p = pf;
+    *s_ratio = 1;
+    if (K >= 256 && d >= 128 && have_saved && pf.prefixed && pf.nseg >= 4 && pf.nseg % 2 == 0 &&
+        tune::get(tune::NSEG_SAME) <= 0) {
+        p.nseg = pf.nseg / 2;
+        p.seg_len = 2 * pf.seg_len;
+        p.prefixed = use_scanned_totals(p.nseg, K, d) ? 1 : 0;      // of dR, dr
+        *s_ratio = 2;
+    }
+    return p;
 }
 
 template <int KD, int DH>
 int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v,
                     const rfa::half_t* g, const rfa::half_t* out, rfa::half_t* dq, rfa::half_t* dk,
                     rfa::half_t* dv, int T, int N, const ScanPlan& pf, char* ws, const Workspace& wl,
-                    const float* savedS, const float* savedZ, const float* savedDen, hipStream_t st) {
-    // pf is the forward's cut into segments (that of the saved totals).  Where both sweeps run as two
-    // workgroups per (sequence, segment) and the totals are scanned, the backward takes segments
-    // twice as long: half as many workgroups already cover the CUs, in one round instead of two.
-    ScanPlan p = pf;
-    const int prefixed_s = use_scanned_totals(pf.nseg, KD, DH) ? 1 : 0;
+                    const int* savedHdr, const float* savedS, const float* savedZ, const float* savedDen,
+                    hipStream_t st) {
+    // pf is the forward's cut into segments (that of the saved totals)
     int s_ratio = 1;
-    if constexpr (KD >= 256 && DH >= 128) {
-        if (savedS && prefixed_s && pf.nseg >= 4 && pf.nseg % 2 == 0 && !getenv("RFA_HIP_NSEG_SAME")) {
-            p.nseg = pf.nseg / 2;
-            p.seg_len = 2 * pf.seg_len;
-            s_ratio = 2;
-        }
-    }
-    const int prefixed = (s_ratio == 1) ? prefixed_s : (use_scanned_totals(p.nseg, KD, DH) ? 1 : 0);   // of dR, dr
+    const ScanPlan p = backward_plan(pf, KD, DH, savedS != nullptr, &s_ratio);
+    const int prefixed_s = pf.prefixed;
+    const int prefixed = p.prefixed;   // of dR, dr
+    const rfa::PlanWords pw = plan_words(LAYOUT_SEGMENTS, T, N, KD, DH, pf);
     constexpr int NW = causal_waves(KD, DH);
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
@@ -261,14 +378,16 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
             auto kern = rfa::k_causal_bwd_dq_saved<KL, DH, NWQ, fwd_state_waves_v<KD, DH>, KD>;
             if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
             RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(2 * N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g,
-                       out, savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len, prefixed_s, pf.nseg, s_ratio);
+                       out, savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len, prefixed_s, pf.nseg, s_ratio,
+                       savedHdr, pw);
         } else {
             constexpr int NWQ = dq_waves(KD, DH);
             using CfgQ = rfa::CausalCfg<KD, DH, NWQ>;
             auto kern = rfa::k_causal_bwd_dq_saved<KD, DH, NWQ, fwd_state_waves_v<KD, DH>>;
             if (int rc = set_lds(kern, CfgQ::kBwdDqSavedLds)) return rc;
             RFA_LAUNCH(CAUSAL_BWD_DQ, kern, dim3(N * p.nseg), dim3(64 * NWQ), CfgQ::kBwdDqSavedLds, st, q, k, v, g, out,
-                       savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len, prefixed_s, pf.nseg, s_ratio);
+                       savedDen, dq, inS, inZ, wsR, wsr, gz, T, N, p.nseg, p.seg_len, prefixed_s, pf.nseg, s_ratio,
+                       savedHdr, pw);
         }
         den_in = savedDen;
     } else {
@@ -290,7 +409,8 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         auto kern = rfa::k_causal_bwd_dkdv_roles<KD, DH, NWR>;
         if (int rc = set_lds(kern, CfgR::kLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(2 * N * p.nseg), dim3(64 * NWR), CfgR::kLds, st, q, k, v, g, dk, dv,
-                   (const float*)wsR, (const float*)wsr, den_in, (const float*)gz, T, N, p.nseg, p.seg_len, prefixed);
+                   (const float*)wsR, (const float*)wsr, den_in, (const float*)gz, T, N, p.nseg, p.seg_len, prefixed,
+                   savedHdr, pw);
     } else
     if constexpr (NW == 4 && KD <= 128) {
         // 8 waves with the state phase split by role (dK waves / dV waves): two waves per SIMD
@@ -299,12 +419,14 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
         auto kern = rfa::k_causal_bwd_dkdv<KD, DH, 8, true, true>;
         if (int rc = set_lds(kern, CfgK::kBwdDkLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(512), CfgK::kBwdDkLds, st, q, k, v, g,
-                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len, prefixed);
+                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len, prefixed,
+                           savedHdr, pw);
     } else {
         auto kern = rfa::k_causal_bwd_dkdv<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
         RFA_LAUNCH(CAUSAL_BWD_DKDV, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDkLds, st, q, k, v, g,
-                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len, prefixed);
+                           dk, dv, wsR, wsr, den_in, gz, (const uint8_t*)nullptr, 1, T, N, p.nseg, p.seg_len, prefixed,
+                           savedHdr, pw);
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -313,14 +435,11 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
 // ---- cross attention launchers ---------------------------------------------------
 // time split for kernels whose workgroups do not depend on each other
 ScanPlan make_free_plan(int64_t T, int64_t N) {
-    ScanPlan p{1, rfa::kChunk};
+    ScanPlan p{1, rfa::kChunk, 0};
     if (T <= 0 || N <= 0) return p;
     const int64_t nchunks = (T + rfa::kChunk - 1) / rfa::kChunk;
-    int64_t target = 512;      // workgroups to aim for; RFA_HIP_FREE_WG overrides (tuning sweeps)
-    if (const char* env = getenv("RFA_HIP_FREE_WG")) {
-        const long v = strtol(env, nullptr, 10);
-        if (v >= 1) target = v;
-    }
+    int64_t target = 2 * device_cus();      // workgroups to aim for: two per compute unit
+    if (tune::get(tune::FREE_WG) >= 1) target = tune::get(tune::FREE_WG);
     int64_t want = (target + N - 1) / N;
     if (want > nchunks) want = nchunks;
     if (want < 1) want = 1;
@@ -361,7 +480,7 @@ int launch_cross_readout(const rfa::half_t* q, const float* s, const float* z, r
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
     RFA_LAUNCH(CROSS_READOUT, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kFwdLds, st, q,
                        (const rfa::half_t*)nullptr, (const rfa::half_t*)nullptr, out, s, z, (float*)nullptr,
-                       (float*)nullptr, (float*)nullptr, T, N, p.nseg, p.seg_len, 0);
+                       (float*)nullptr, (float*)nullptr, T, N, p.nseg, p.seg_len, 0, (int*)nullptr, rfa::PlanWords{});
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -392,7 +511,8 @@ int launch_cross_state_bwd(const rfa::half_t* k, const rfa::half_t* v, const uin
     if (int rc = set_lds(kern, Cfg::kBwdDkLds)) return rc;
     RFA_LAUNCH(CROSS_STATE_BWD, kern, dim3(N * p.nseg), dim3(64 * NW), Cfg::kBwdDkLds, st,
                        (const rfa::half_t*)nullptr, k, v, (const rfa::half_t*)nullptr, dk, dv, ds, dz,
-                       (const float*)nullptr, (const float*)nullptr, mask, H, T, N, p.nseg, p.seg_len, 0);
+                       (const float*)nullptr, (const float*)nullptr, mask, H, T, N, p.nseg, p.seg_len, 0,
+                       (const int*)nullptr, rfa::PlanWords{});
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -438,8 +558,8 @@ int launch_masked_bwd(const rfa::half_t* q, const rfa::half_t* k, const rfa::hal
 // ---- decode launchers --------------------------------------------------------------
 template <int KD, int DH, bool FUSED>
 int launch_decode(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, const rfa::half_t* w,
-                  float scale, int H, float* s, float* z, rfa::half_t* out, int64_t steps, int64_t N,
-                  hipStream_t st) {
+                  float scale, int H, const float* s_in, const float* z_in, float* s, float* z, rfa::half_t* out,
+                  int64_t steps, int64_t N, hipStream_t st) {
     const int64_t qk_step = FUSED ? N * DH : N * KD;
     // A step's q, k, v rows sit between its state loads and its state stores (the feature map
     // needs them first).  In a decoder they were written a moment ago; in a multi-step call they
@@ -455,8 +575,8 @@ int launch_decode(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t*
                        reinterpret_cast<const uint4*>(v + t * N * DH), m * qk_step / 8, m * qk_step / 8, m * N * DH / 8);
         }
         RFA_LAUNCH(DECODE_STEP, (rfa::k_decode_step<KD, DH, FUSED>), dim3((unsigned)N), dim3(rfa::kThreads), 0, st,
-                           q + t * qk_step, k + t * qk_step, v + t * N * DH, w, scale, H, s, z, s, z,
-                           out + t * N * DH);
+                           q + t * qk_step, k + t * qk_step, v + t * N * DH, w, scale, H,
+                           t == 0 ? s_in : (const float*)s, t == 0 ? z_in : (const float*)z, s, z, out + t * N * DH);
     }
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
@@ -472,7 +592,7 @@ int launch_project_rows(const rfa::half_t* x, const rfa::ProjectArgs& pa, const 
     if (int rc = set_lds(kern, Cfg::kLds)) return rc;
     const int nrt = (R + Cfg::BM - 1) / Cfg::BM;
     const int pairs = H * np;
-    int ngroups = (256 + nrt - 1) / nrt;
+    int ngroups = (device_cus() + nrt - 1) / nrt;
     if (ngroups > pairs) ngroups = pairs;
     const int ppg = (pairs + ngroups - 1) / ngroups;
     ngroups = (pairs + ppg - 1) / ppg;
@@ -487,7 +607,7 @@ template <int D, int DH>
 int launch_project_phi(const rfa::half_t* x, const rfa::ProjectArgs& pa, const rfa::half_t* wf, int R, int E, int H,
                        int np, float scale, hipStream_t st) {
     if constexpr (DH == 64 && D <= 64) {
-        if (!getenv("RFA_HIP_PROJECT_STREAMING")) {
+        if (tune::get(tune::PROJECT_STREAMING) <= 0) {
             if (E == 128) return launch_project_rows<D, DH, 4>(x, pa, wf, R, H, np, scale, st);
             if (E == 256) return launch_project_rows<D, DH, 8>(x, pa, wf, R, H, np, scale, st);
             if (E == 384) return launch_project_rows<D, DH, 12>(x, pa, wf, R, H, np, scale, st);
@@ -588,6 +708,38 @@ int check_causal_dims(int64_t T, int64_t N, int K, int d) {
     return RFA_OK;
 }
 
+// ---- static device memory --------------------------------------------------
+// Memory the library owns without allocating: file-scope device variables, one copy per GPU, held
+// until the process ends.  In host code such a name is a stand-in, not a device address: the
+// address on the current device comes from hipGetSymbolAddress, once per device.
+static __device__ int g_selftest_word;        // result word of rfa_selftest_layout
+
+constexpr int kMaxDevices = 64;
+
+// address of a static device variable on the current device, looked up once per device
+int cached_symbol_address(std::atomic<void*>* cache, hipError_t (*lookup)(void**), void** out) {
+    int dev = 0;
+    RFA_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(RFA_ERR_HIP, "device index %d not supported", dev);
+    void* p = cache[dev].load(std::memory_order_acquire);
+    if (!p) {
+        RFA_HIP_TRY(lookup(&p));
+        if (!p) return fail(RFA_ERR_HIP, "hipGetSymbolAddress returned a NULL address");
+        cache[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return RFA_OK;
+}
+
+int selftest_word_address(int** out) {
+    static std::atomic<void*> cache[kMaxDevices];
+    void* p = nullptr;
+    if (int rc = cached_symbol_address(cache, [](void** q) { return hipGetSymbolAddress(q, HIP_SYMBOL(g_selftest_word)); }, &p))
+        return rc;
+    *out = static_cast<int*>(p);
+    return RFA_OK;
+}
+
 // ---- layout self test ------------------------------------------------------
 __global__ void k_selftest(int* bad) {
     using namespace rfa;
@@ -667,21 +819,33 @@ int rfa_shape_supported(int K, int d) {
     return ((K == 64 || K == 128 || K == 256) && (d == 64 || d == 128)) ? 1 : 0;
 }
 
-int rfa_causal_num_segments(int64_t T, int64_t N) { return make_plan(T, N).nseg; }
+int rfa_causal_num_segments(int64_t T, int64_t N, int K, int d) { return make_plan(T, N, K, d).nseg; }
+
+int rfa_tuning_set(const char* name, int value) {
+    const int k = tune::find(name);
+    if (k < 0) return fail(RFA_ERR_BAD_SHAPE, "rfa_tuning_set: no knob named '%s'", name ? name : "(null)");
+    if (value < -1 || value > (1 << 20)) return fail(RFA_ERR_BAD_SHAPE, "rfa_tuning_set: value %d out of range", value);
+    (void)tune::get((tune::Key)k);      // the environment is read before the first store
+    tune::value[k].store(value, std::memory_order_relaxed);
+    return RFA_OK;
+}
+
+int rfa_tuning_get(const char* name, int* value) {
+    const int k = tune::find(name);
+    if (k < 0 || !value) return fail(RFA_ERR_BAD_SHAPE, "rfa_tuning_get: no knob named '%s'", name ? name : "(null)");
+    *value = tune::get((tune::Key)k);
+    return RFA_OK;
+}
 
 int rfa_selftest_layout(void* stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int* dbad = nullptr;
-    RFA_HIP_TRY(hipMalloc(&dbad, sizeof(int)));
+    int* dbad = nullptr;      // a word of the library's static device memory: nothing is allocated
+    if (int rc = selftest_word_address(&dbad)) return rc;
     int hbad = 0;
-    hipError_t e = hipMemcpyAsync(dbad, &hbad, sizeof(int), hipMemcpyHostToDevice, st);
-    if (e == hipSuccess) {
-        RFA_LAUNCH(SELFTEST, k_selftest, dim3(1), dim3(64), 0, st, dbad);
-        e = hipMemcpyAsync(&hbad, dbad, sizeof(int), hipMemcpyDeviceToHost, st);
-    }
-    if (e == hipSuccess) e = hipStreamSynchronize(st);
-    (void)hipFree(dbad);
-    if (e != hipSuccess) return fail(RFA_ERR_HIP, "selftest: %s", hipGetErrorString(e));
+    RFA_HIP_TRY(hipMemcpyAsync(dbad, &hbad, sizeof(int), hipMemcpyHostToDevice, st));
+    RFA_LAUNCH(SELFTEST, k_selftest, dim3(1), dim3(64), 0, st, dbad);
+    RFA_HIP_TRY(hipMemcpyAsync(&hbad, dbad, sizeof(int), hipMemcpyDeviceToHost, st));
+    RFA_HIP_TRY(hipStreamSynchronize(st));
     if (hbad) return fail(RFA_ERR_HIP, "selftest: %d lane values differ from the assumed MFMA / LDS layout", hbad);
     return RFA_OK;
 }
@@ -702,12 +866,12 @@ int rfa_selftest_mfma_rate(int waves_per_simd, int iters, float* sink, double* f
 
 size_t rfa_causal_forward_workspace_bytes(int64_t T, int64_t N, int K, int d) {
     if (T <= 0 || N <= 0 || !rfa_shape_supported(K, d)) return 0;
-    return layout_workspace(T, N, K, d, make_plan(T, N), false).total;
+    return layout_workspace(T, N, K, d, make_plan(T, N, K, d), false).total;
 }
 
 size_t rfa_causal_backward_workspace_bytes(int64_t T, int64_t N, int K, int d) {
     if (T <= 0 || N <= 0 || !rfa_shape_supported(K, d)) return 0;
-    return layout_workspace(T, N, K, d, make_plan(T, N), true).total;
+    return layout_workspace(T, N, K, d, make_plan(T, N, K, d), true).total;
 }
 
 #define RFA_DISPATCH_KD(K, d, CALL)                                   \
@@ -718,19 +882,59 @@ size_t rfa_causal_backward_workspace_bytes(int64_t T, int64_t N, int K, int d) {
     if (K == 128 && d == 128) { return CALL(128, 128); }              \
     if (K == 256 && d == 128) { return CALL(256, 128); }
 
-// bytes of the saved buffer: segment totals (row-major S, then z), then the raw denominators
-static size_t saved_state_bytes(int64_t T, int64_t N, int K, int d, size_t* z_offset, size_t* den_offset) {
-    const ScanPlan p = make_plan(T, N);
-    const size_t s_bytes = align_up((size_t)N * p.nseg * K * d * 4);
-    const size_t z_bytes = align_up((size_t)N * p.nseg * K * 4);
-    if (z_offset) *z_offset = s_bytes;
-    if (den_offset) *den_offset = s_bytes + z_bytes;
-    return s_bytes + z_bytes + align_up((size_t)T * N * 4);
+// The saved buffer: a 256-byte header (rfa::PlanWords: the plan of the forward that wrote the
+// buffer), the segment totals S (fragment order), z, and the raw denominators.
+struct SavedLayoutBytes { size_t S, Z, den, total; };
+
+static SavedLayoutBytes saved_layout(int64_t T, int64_t N, int K, int d, const ScanPlan& p) {
+    SavedLayoutBytes l{};
+    size_t off = kSavedHeaderBytes;
+    l.S = off; off += align_up((size_t)N * p.nseg * K * d * 4);
+    l.Z = off; off += align_up((size_t)N * p.nseg * K * 4);
+    l.den = off; off += align_up((size_t)T * N * 4);
+    l.total = off;
+    return l;
 }
 
 size_t rfa_causal_saved_state_bytes(int64_t T, int64_t N, int K, int d) {
     if (T <= 0 || N <= 0 || !rfa_shape_supported(K, d)) return 0;
-    return saved_state_bytes(T, N, K, d, nullptr, nullptr);
+    return saved_layout(T, N, K, d, make_plan(T, N, K, d)).total;
+}
+
+// The plan a backward call on `saved` runs with: the one recorded when a forward call of this
+// process last wrote that buffer, else the current one.  RFA_ERR_WORKSPACE if the recorded
+// forward had another shape.
+static int saved_plan(const char* fn, const void* saved, int64_t T, int64_t N, int K, int d, ScanPlan* p) {
+    rfa::PlanWords w;
+    if (saved && registry::get(saved, &w)) {
+        const rfa::PlanWords same = plan_words(w.w[2], T, N, K, d, ScanPlan{w.w[5], w.w[6], w.w[7]});
+        if (memcmp(&w, &same, sizeof(w)) != 0)
+            return fail(RFA_ERR_WORKSPACE,
+                        "%s: the saved buffer was written by a forward call of another shape (T=%lld N=%lld K=%d d=%d), "
+                        "this call has T=%lld N=%lld K=%d d=%d", fn,
+                        (long long)(((int64_t)w.w[9] << 32) | (uint32_t)w.w[8]),
+                        (long long)(((int64_t)w.w[11] << 32) | (uint32_t)w.w[10]), w.w[3], w.w[4], (long long)T,
+                        (long long)N, K, d);
+        *p = ScanPlan{w.w[5], w.w[6], w.w[7]};
+        return RFA_OK;
+    }
+    *p = make_plan(T, N, K, d);
+    return RFA_OK;
+}
+
+size_t rfa_causal_backward_saved_workspace_bytes(const void* saved, int64_t T, int64_t N, int K, int d) {
+    if (T <= 0 || N <= 0 || !rfa_shape_supported(K, d)) return 0;
+    ScanPlan p;
+    if (saved_plan("rfa_causal_backward_saved_workspace_bytes", saved, T, N, K, d, &p) != RFA_OK) return 0;
+    return layout_workspace(T, N, K, d, p, true).total;
+}
+
+int rfa_causal_saved_describe(const void* saved, int32_t* words16, void* stream) {
+    if (!saved || !words16) return fail(RFA_ERR_NULL_POINTER, "rfa_causal_saved_describe: NULL pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    RFA_HIP_TRY(hipMemcpyAsync(words16, saved, 16 * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    RFA_HIP_TRY(hipStreamSynchronize(st));
+    return RFA_OK;
 }
 
 static int causal_forward_impl(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
@@ -770,25 +974,28 @@ static int causal_forward_impl(const void* q, const void* k, const void* v, void
                                float* final_z, void* workspace, size_t workspace_bytes, void* stream) {
     if (int rc = check_causal_dims(T, N, K, d)) return rc;
     if (T == 0 || N == 0) return RFA_OK;
+    const ScanPlan p = make_plan(T, N, K, d);
+    int* savedHdr = nullptr;
     float* savedS = nullptr;
     float* savedZ = nullptr;
     float* savedDen = nullptr;
     if (want_saved) {
-        size_t zoff = 0, doff = 0;
-        const size_t need = saved_state_bytes(T, N, K, d, &zoff, &doff);
-        if (!saved || saved_bytes < need || !aligned16(saved))
+        const SavedLayoutBytes sl = saved_layout(T, N, K, d, p);
+        if (!saved || saved_bytes < sl.total || !aligned16(saved))
             return fail(RFA_ERR_WORKSPACE, "rfa_causal_forward_save: saved-state buffer of %zu bytes required, got %zu",
-                        need, saved ? saved_bytes : (size_t)0);
-        savedS = static_cast<float*>(saved);
-        savedZ = reinterpret_cast<float*>(static_cast<char*>(saved) + zoff);
-        savedDen = reinterpret_cast<float*>(static_cast<char*>(saved) + doff);
+                        sl.total, saved ? saved_bytes : (size_t)0);
+        char* sb = static_cast<char*>(saved);
+        savedHdr = reinterpret_cast<int*>(sb);
+        savedS = reinterpret_cast<float*>(sb + sl.S);
+        savedZ = reinterpret_cast<float*>(sb + sl.Z);
+        savedDen = reinterpret_cast<float*>(sb + sl.den);
     }
     if (!q || !k || !v || !out) return fail(RFA_ERR_NULL_POINTER, "rfa_causal_forward: NULL tensor pointer");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
         return fail(RFA_ERR_ALIGNMENT, "rfa_causal_forward: tensors must be 16-byte aligned");
-    const ScanPlan p = make_plan(T, N);
     const Workspace wl = layout_workspace(T, N, K, d, p, false);
-    if (wl.total > 0 && (!workspace || workspace_bytes < wl.total || !aligned16(workspace)))
+    // with a saved buffer the segment totals go there and the workspace is not touched
+    if (!want_saved && wl.total > 0 && (!workspace || workspace_bytes < wl.total || !aligned16(workspace)))
         return fail(RFA_ERR_WORKSPACE, "rfa_causal_forward: workspace of %zu bytes required, got %zu", wl.total,
                     workspace ? workspace_bytes : (size_t)0);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -797,7 +1004,8 @@ static int causal_forward_impl(const void* q, const void* k, const void* v, void
     auto* vh = static_cast<const rfa::half_t*>(v);
     auto* oh = static_cast<rfa::half_t*>(out);
     char* ws = static_cast<char*>(workspace);
-#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedS, savedZ, savedDen, final_s, final_z, st)
+    if (want_saved) registry::put(saved, plan_words(LAYOUT_SEGMENTS, T, N, K, d, p));
+#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedHdr, savedS, savedZ, savedDen, final_s, final_z, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_FWD)
 #undef RFA_CALL_FWD
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
@@ -833,25 +1041,30 @@ static int causal_backward_impl(const void* q, const void* k, const void* v, con
                                 size_t workspace_bytes, void* stream) {
     if (int rc = check_causal_dims(T, N, K, d)) return rc;
     if (T == 0 || N == 0) return RFA_OK;
+    ScanPlan p = make_plan(T, N, K, d);
+    const int* savedHdr = nullptr;
     const float* savedS = nullptr;
     const float* savedZ = nullptr;
     const float* savedDen = nullptr;
     if (have_saved) {
-        size_t zoff = 0, doff = 0;
-        const size_t need = saved_state_bytes(T, N, K, d, &zoff, &doff);
-        if (!saved || saved_bytes < need || !aligned16(saved))
+        if (!saved || !aligned16(saved))
+            return fail(RFA_ERR_WORKSPACE, "rfa_causal_backward_saved: NULL or misaligned saved-state buffer");
+        if (int rc = saved_plan("rfa_causal_backward_saved", saved, T, N, K, d, &p)) return rc;
+        const SavedLayoutBytes sl = saved_layout(T, N, K, d, p);
+        if (saved_bytes < sl.total)
             return fail(RFA_ERR_WORKSPACE, "rfa_causal_backward_saved: saved-state buffer of %zu bytes required, got %zu",
-                        need, saved ? saved_bytes : (size_t)0);
-        savedS = static_cast<const float*>(saved);
-        savedZ = reinterpret_cast<const float*>(static_cast<const char*>(saved) + zoff);
-        savedDen = reinterpret_cast<const float*>(static_cast<const char*>(saved) + doff);
+                        sl.total, saved_bytes);
+        const char* sb = static_cast<const char*>(saved);
+        savedHdr = reinterpret_cast<const int*>(sb);
+        savedS = reinterpret_cast<const float*>(sb + sl.S);
+        savedZ = reinterpret_cast<const float*>(sb + sl.Z);
+        savedDen = reinterpret_cast<const float*>(sb + sl.den);
     }
     if (!q || !k || !v || !grad_attn || !dq || !dk || !dv)
         return fail(RFA_ERR_NULL_POINTER, "rfa_causal_backward: NULL tensor pointer");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(grad_attn) || !aligned16(dq) ||
         !aligned16(dk) || !aligned16(dv))
         return fail(RFA_ERR_ALIGNMENT, "rfa_causal_backward: tensors must be 16-byte aligned");
-    const ScanPlan p = make_plan(T, N);
     const Workspace wl = layout_workspace(T, N, K, d, p, true);
     if (!workspace || workspace_bytes < wl.total || !aligned16(workspace))
         return fail(RFA_ERR_WORKSPACE, "rfa_causal_backward: workspace of %zu bytes required, got %zu", wl.total,
@@ -866,7 +1079,7 @@ static int causal_backward_impl(const void* q, const void* k, const void* v, con
     auto* dkh = static_cast<rfa::half_t*>(dk);
     auto* dvh = static_cast<rfa::half_t*>(dv);
     char* ws = static_cast<char*>(workspace);
-#define RFA_CALL_BWD(KD, DH) launch_backward<KD, DH>(qh, kh, vh, gh, outh, dqh, dkh, dvh, (int)T, (int)N, p, ws, wl, savedS, savedZ, savedDen, st)
+#define RFA_CALL_BWD(KD, DH) launch_backward<KD, DH>(qh, kh, vh, gh, outh, dqh, dkh, dvh, (int)T, (int)N, p, ws, wl, savedHdr, savedS, savedZ, savedDen, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_BWD)
 #undef RFA_CALL_BWD
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
@@ -1043,33 +1256,46 @@ int rfa_masked_backward(const void* phi_q, const void* phi_k, const void* v, con
 }
 
 // ---- incremental decoding -----------------------------------------------------------
-int rfa_incremental(const void* phi_q, const void* phi_k, const void* v, float* s, float* z, void* out,
-                    int64_t steps, int64_t N, int K, int d, void* stream) {
-    if (int rc = check_cross_dims("rfa_incremental", steps, N, 1, K, d)) return rc;
+static int incremental_impl(const char* fn, const void* phi_q, const void* phi_k, const void* v, const float* s_in,
+                            const float* z_in, float* s, float* z, void* out, int64_t steps, int64_t N, int K, int d,
+                            void* stream) {
+    if (int rc = check_cross_dims(fn, steps, N, 1, K, d)) return rc;
     if (steps == 0 || N == 0) return RFA_OK;
-    if (!phi_q || !phi_k || !v || !s || !z || !out) return fail(RFA_ERR_NULL_POINTER, "rfa_incremental: NULL tensor pointer");
-    if (!aligned16(phi_q) || !aligned16(phi_k) || !aligned16(v) || !aligned16(s) || !aligned16(z) || !aligned16(out))
-        return fail(RFA_ERR_ALIGNMENT, "rfa_incremental: tensors must be 16-byte aligned");
+    if (!phi_q || !phi_k || !v || !s_in || !z_in || !s || !z || !out) return fail(RFA_ERR_NULL_POINTER, "%s: NULL tensor pointer", fn);
+    if (!aligned16(phi_q) || !aligned16(phi_k) || !aligned16(v) || !aligned16(s_in) || !aligned16(z_in) || !aligned16(s) ||
+        !aligned16(z) || !aligned16(out))
+        return fail(RFA_ERR_ALIGNMENT, "%s: tensors must be 16-byte aligned", fn);
     hipStream_t st = static_cast<hipStream_t>(stream);
     auto* qh = static_cast<const rfa::half_t*>(phi_q);
     auto* kh = static_cast<const rfa::half_t*>(phi_k);
     auto* vh = static_cast<const rfa::half_t*>(v);
     auto* oh = static_cast<rfa::half_t*>(out);
-#define RFA_CALL(KD, DH) launch_decode<KD, DH, false>(qh, kh, vh, nullptr, 0.f, 1, s, z, oh, steps, N, st)
+#define RFA_CALL(KD, DH) launch_decode<KD, DH, false>(qh, kh, vh, nullptr, 0.f, 1, s_in, z_in, s, z, oh, steps, N, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
 }
 
-int rfa_incremental_fused(const void* q, const void* k, const void* v, const void* w, float scale, float* s,
-                          float* z, void* out, int64_t steps, int64_t B, int H, int D, int d, void* stream) {
-    if (int rc = check_cross_dims("rfa_incremental_fused", steps, B, H, 2 * D, d)) return rc;
+int rfa_incremental(const void* phi_q, const void* phi_k, const void* v, float* s, float* z, void* out,
+                    int64_t steps, int64_t N, int K, int d, void* stream) {
+    return incremental_impl("rfa_incremental", phi_q, phi_k, v, s, z, s, z, out, steps, N, K, d, stream);
+}
+
+int rfa_incremental_out(const void* phi_q, const void* phi_k, const void* v, const float* s_in, const float* z_in,
+                        float* s_out, float* z_out, void* out, int64_t steps, int64_t N, int K, int d, void* stream) {
+    return incremental_impl("rfa_incremental_out", phi_q, phi_k, v, s_in, z_in, s_out, z_out, out, steps, N, K, d, stream);
+}
+
+static int incremental_fused_impl(const char* fn, const void* q, const void* k, const void* v, const void* w, float scale,
+                                  const float* s_in, const float* z_in, float* s, float* z, void* out, int64_t steps,
+                                  int64_t B, int H, int D, int d, void* stream) {
+    if (int rc = check_cross_dims(fn, steps, B, H, 2 * D, d)) return rc;
     const int64_t N = B * H;
     if (steps == 0 || N == 0) return RFA_OK;
-    if (!q || !k || !v || !w || !s || !z || !out)
-        return fail(RFA_ERR_NULL_POINTER, "rfa_incremental_fused: NULL tensor pointer");
-    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(s) || !aligned16(z) || !aligned16(out))
-        return fail(RFA_ERR_ALIGNMENT, "rfa_incremental_fused: tensors must be 16-byte aligned");
+    if (!q || !k || !v || !w || !s_in || !z_in || !s || !z || !out) return fail(RFA_ERR_NULL_POINTER, "%s: NULL tensor pointer", fn);
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(s_in) || !aligned16(z_in) ||
+        !aligned16(s) || !aligned16(z) || !aligned16(out))
+        return fail(RFA_ERR_ALIGNMENT, "%s: tensors must be 16-byte aligned", fn);
     hipStream_t st = static_cast<hipStream_t>(stream);
     auto* qh = static_cast<const rfa::half_t*>(q);
     auto* kh = static_cast<const rfa::half_t*>(k);
@@ -1077,10 +1303,22 @@ int rfa_incremental_fused(const void* q, const void* k, const void* v, const voi
     auto* wh = static_cast<const rfa::half_t*>(w);
     auto* oh = static_cast<rfa::half_t*>(out);
     const int K = 2 * D;
-#define RFA_CALL(KD, DH) launch_decode<KD, DH, true>(qh, kh, vh, wh, scale, H, s, z, oh, steps, N, st)
+#define RFA_CALL(KD, DH) launch_decode<KD, DH, true>(qh, kh, vh, wh, scale, H, s_in, z_in, s, z, oh, steps, N, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+int rfa_incremental_fused(const void* q, const void* k, const void* v, const void* w, float scale, float* s,
+                          float* z, void* out, int64_t steps, int64_t B, int H, int D, int d, void* stream) {
+    return incremental_fused_impl("rfa_incremental_fused", q, k, v, w, scale, s, z, s, z, out, steps, B, H, D, d, stream);
+}
+
+int rfa_incremental_fused_out(const void* q, const void* k, const void* v, const void* w, float scale,
+                              const float* s_in, const float* z_in, float* s_out, float* z_out, void* out,
+                              int64_t steps, int64_t B, int H, int D, int d, void* stream) {
+    return incremental_fused_impl("rfa_incremental_fused_out", q, k, v, w, scale, s_in, z_in, s_out, z_out, out, steps,
+                                  B, H, D, d, stream);
 }
 
 // ---- random matrices ----------------------------------------------------------------

@@ -215,13 +215,14 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
     float* __restrict__ den_out, float* __restrict__ final_s, float* __restrict__ final_z, int T, int N,
-    int nseg, int seg_len, int prefixed) {
+    int nseg, int seg_len, int prefixed, int* __restrict__ hdr_out, PlanWords plan) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = Cfg::DS;
     constexpr int NKT = KD / 16, NCT = DS / 16, NKTW = NKT / NW;
     static_assert(DH % (16 * NW) == 0 && NKT % NW == 0, "shape does not split over the waves");
     extern __shared__ __align__(16) unsigned char smem_raw[];
+    plan_write(hdr_out, plan);
     half_t* Qs = reinterpret_cast<half_t*>(smem_raw);
     half_t* Ks = Qs + C * LDQ;
     half_t* Vs = Ks + C * LDQ;
@@ -499,7 +500,8 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
     float* __restrict__ den_out, float* __restrict__ final_s, float* __restrict__ final_z, int T, int N,
-    int nseg, int seg_len, int prefixed) {
+    int nseg, int seg_len, int prefixed, int* __restrict__ hdr_out, PlanWords plan) {
+    plan_write(hdr_out, plan);
     using Cfg = FwdPipeCfg<KD, DH>;
     constexpr int NT = 256;      // threads per group
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, DS = DH / 4;
@@ -1119,7 +1121,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     const half_t* __restrict__ g, const half_t* __restrict__ o, const float* __restrict__ den_raw,
     half_t* __restrict__ dq, const float* __restrict__ wsS, const float* __restrict__ wsZ,
     float* __restrict__ wsR, float* __restrict__ wsr, float* __restrict__ gz_ws, int T, int N, int nseg,
-    int seg_len, int prefixed, int s_nseg, int s_ratio) {
+    int seg_len, int prefixed, int s_nseg, int s_ratio, const int* __restrict__ hdr_in, PlanWords plan) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     constexpr int C = Cfg::C, LDQ = Cfg::LDQ, LDV = Cfg::LDV, LDA = Cfg::LDA, KS = Cfg::KS;
@@ -1157,6 +1159,10 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
     const half_t* gb = g + (int64_t)n * DH;
     const half_t* ob = o + (int64_t)n * DH;
     half_t* dqb = dq + (int64_t)n * KDG + koff;
+    if (!plan_matches(hdr_in, plan)) {      // the saved buffer was written for another plan
+        poison_rows<KD>(dqb, k_stride, t_begin, t_end);
+        return;
+    }
 
     f4 ST[NCT][NKT], RT[NCT][NKT];
 #pragma unroll
@@ -1414,7 +1420,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     const half_t* __restrict__ g, half_t* __restrict__ dk, half_t* __restrict__ dv,
     const float* __restrict__ wsR, const float* __restrict__ wsr, const float* __restrict__ den_ws,
     const float* __restrict__ gz_ws, const uint8_t* __restrict__ pad_mask, int H, int T, int N,
-    int nseg, int seg_len, int prefixed) {
+    int nseg, int seg_len, int prefixed, const int* __restrict__ hdr_in, PlanWords plan) {
     using Cfg = CausalCfg<KD, DH, NW>;
     constexpr int NT = Cfg::NT;
     static_assert(!SPLIT || NW == 8, "the role split needs 8 waves");
@@ -1451,6 +1457,11 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     const half_t* gb = g + (int64_t)n * DH;
     half_t* dkb = dk + (int64_t)n * KD;
     half_t* dvb = dv + (int64_t)n * DH;
+    if (!plan_matches(hdr_in, plan)) {
+        poison_rows<KD>(dkb, k_stride, t_begin, t_end);
+        poison_rows<DH>(dvb, v_stride, t_begin, t_end);
+        return;
+    }
 
     f4 RT[NCT][NKT], RR[NKT2][NCT2];
 #pragma unroll
@@ -2139,9 +2150,19 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv_roles(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, half_t* __restrict__ dk, half_t* __restrict__ dv,
     const float* __restrict__ wsR, const float* __restrict__ wsr, const float* __restrict__ den_ws,
-    const float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len, int prefixed) {
+    const float* __restrict__ gz_ws, int T, int N, int nseg, int seg_len, int prefixed,
+    const int* __restrict__ hdr_in, PlanWords plan) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int nsq = N * nseg;
+    if (!plan_matches(hdr_in, plan)) {
+        const bool is_dk = (int)blockIdx.x < nsq;
+        int n, seg;
+        seq_seg_of_block(is_dk ? blockIdx.x : blockIdx.x - nsq, N, nseg, n, seg);
+        const int t_begin = seg * seg_len, t_end = min(T, t_begin + seg_len);
+        if (is_dk) poison_rows<KD>(dk + (int64_t)n * KD, (int64_t)N * KD, t_begin, t_end);
+        else poison_rows<DH>(dv + (int64_t)n * DH, (int64_t)N * DH, t_begin, t_end);
+        return;
+    }
     if ((int)blockIdx.x < nsq)
         dkdv_role_dk<KD, DH, NW>(smem_raw, blockIdx.x, q, v, g, dk, wsR, wsr, den_ws, gz_ws, T, N, nseg, seg_len, prefixed);
     else

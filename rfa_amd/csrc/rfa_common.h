@@ -54,6 +54,37 @@ constexpr int lds_pad(int F) { return (F % 128 == 0) ? 24 : 8; }
 
 constexpr int kThreads = 256;   // threads per workgroup
 constexpr int kChunk = 64;      // time steps per chunk
+constexpr int kXcds = 8;        // accelerator dies of an MI355X; workgroups are dealt to them round-robin by index
+
+// Description of the forward pass that filled a saved-state buffer: the first 16 ints of the
+// buffer.  The forward kernel writes it, the backward kernels compare it with the plan they were
+// launched for and, if the two differ, fill their outputs with NaN instead of reading segment
+// totals laid out for another plan.
+struct PlanWords {
+    int w[16];   // magic, version, layout, K, d, nseg, seg_len, prefixed, T lo, T hi, N lo, N hi, 0...
+};
+constexpr int kPlanMagic = 0x52464153;   // "RFAS"
+
+__device__ __forceinline__ void plan_write(int* __restrict__ hdr, const PlanWords& p) {
+    if (hdr && blockIdx.x == 0 && threadIdx.x < 16) hdr[threadIdx.x] = p.w[threadIdx.x];
+}
+
+// same answer in every wave of the workgroup
+__device__ __forceinline__ bool plan_matches(const int* __restrict__ hdr, const PlanWords& p) {
+    if (!hdr) return true;
+    const int lane = threadIdx.x & 63;
+    const bool bad = lane < 16 && hdr[lane] != p.w[lane];
+    return !__any(bad);
+}
+
+// rows [t_begin, t_end) of one sequence of a time-major fp16 tensor <- NaN
+template <int F>
+__device__ __forceinline__ void poison_rows(_Float16* __restrict__ base, int64_t row_stride, int t_begin, int t_end) {
+    const unsigned short nan16 = 0x7E00;
+    unsigned short* b = reinterpret_cast<unsigned short*>(base);
+    for (int64_t e = threadIdx.x; e < (int64_t)(t_end - t_begin) * F; e += blockDim.x)
+        b[(int64_t)(t_begin + e / F) * row_stride + e % F] = nan16;
+}
 
 __device__ __forceinline__ f4 mfma32(h8 a, h8 b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);

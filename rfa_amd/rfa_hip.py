@@ -9,7 +9,7 @@ work is enqueued on the current torch stream.
 """
 from __future__ import annotations
 
-from typing import List
+from typing import List, Optional
 
 import torch
 from torch import Tensor
@@ -166,7 +166,8 @@ def backward_saved(q: Tensor, k: Tensor, v: Tensor, grad_attn: Tensor, out: Tens
     d = v.shape[2]
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     with _on_device(q.device):
-        nbytes = lib.rfa_causal_backward_workspace_bytes(T, N, K, d)
+        # sized for the plan of the forward call that wrote `saved`
+        nbytes = lib.rfa_causal_backward_saved_workspace_bytes(saved.data_ptr(), T, N, K, d)
         ws = _workspace(nbytes, q.device)
         _lib.check(lib.rfa_causal_backward_saved(q.data_ptr(), k.data_ptr(), v.data_ptr(), grad_attn.data_ptr(),
                                                  out.data_ptr(), saved.data_ptr(), saved.numel(), dq.data_ptr(), dk.data_ptr(),
@@ -474,22 +475,35 @@ def cross_readout_backward(phi_q: Tensor, s: Tensor, z: Tensor, grad_attn: Tenso
 # ---------------------------------------------------------------------------
 # incremental decoding (state updated in place)
 # ---------------------------------------------------------------------------
-def incremental(phi_q: Tensor, phi_k: Tensor, v: Tensor, s: Tensor, z: Tensor) -> Tensor:
-    """phi_q, phi_k fp16 [steps, N, K]; v fp16 [steps, N, d]; s fp32 [N,K,d], z fp32 [N,K] updated in place."""
+def incremental(phi_q: Tensor, phi_k: Tensor, v: Tensor, s: Tensor, z: Tensor, s_out: Optional[Tensor] = None,
+                z_out: Optional[Tensor] = None) -> Tensor:
+    """phi_q, phi_k fp16 [steps, N, K]; v fp16 [steps, N, d]; s fp32 [N,K,d], z fp32 [N,K].
+
+    Without s_out / z_out the state is advanced in place; with them s and z are only read and the
+    advanced state is written to s_out, z_out (same shapes, fp32)."""
     _check_qkv(phi_q, phi_k, v)
     steps, N, K = phi_q.shape
     d = v.shape[2]
     _check_f32_cuda("s", s, (N, K, d))
     _check_f32_cuda("z", z, (N, K))
+    _require((s_out is None) == (z_out is None), ValueError, lambda: "s_out and z_out go together")
+    if s_out is None:
+        s_out, z_out = s, z
+    else:
+        _check_f32_cuda("s_out", s_out, (N, K, d))
+        _check_f32_cuda("z_out", z_out, (N, K))
     out = torch.empty_like(v)
     with _on_device(v.device):
-        _lib.check(_lib.load().rfa_incremental(phi_q.data_ptr(), phi_k.data_ptr(), v.data_ptr(), s.data_ptr(),
-                                               z.data_ptr(), out.data_ptr(), steps, N, K, d, _stream_ptr(v.device)))
+        _lib.check(_lib.load().rfa_incremental_out(phi_q.data_ptr(), phi_k.data_ptr(), v.data_ptr(), s.data_ptr(),
+                                                   z.data_ptr(), s_out.data_ptr(), z_out.data_ptr(), out.data_ptr(),
+                                                   steps, N, K, d, _stream_ptr(v.device)))
     return out
 
 
-def incremental_fused(q: Tensor, k: Tensor, v: Tensor, w: Tensor, scale: float, s: Tensor, z: Tensor) -> Tensor:
-    """q, k, v fp16 [steps, B, H, d]; w fp16 [H, D, d]; s fp32 [B,H,2D,d], z fp32 [B,H,2D] updated in place."""
+def incremental_fused(q: Tensor, k: Tensor, v: Tensor, w: Tensor, scale: float, s: Tensor, z: Tensor,
+                      s_out: Optional[Tensor] = None, z_out: Optional[Tensor] = None) -> Tensor:
+    """q, k, v fp16 [steps, B, H, d]; w fp16 [H, D, d]; s fp32 [B,H,2D,d], z fp32 [B,H,2D]: advanced in
+    place, or only read when s_out / z_out (same shapes) are given to receive the advanced state."""
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_half_cuda(name, t, 4)
     _require(q.shape == k.shape == v.shape, ValueError, lambda: "q, k, v must have one shape [steps, bsz, heads, head_dim]")
@@ -499,11 +513,17 @@ def incremental_fused(q: Tensor, k: Tensor, v: Tensor, w: Tensor, scale: float, 
     _require(w.shape[0] == H and w.shape[2] == d, ValueError, lambda: "random_matrices must be [heads, proj_dim, head_dim]")
     _check_f32_cuda("s", s, (B, H, 2 * D, d))
     _check_f32_cuda("z", z, (B, H, 2 * D))
+    _require((s_out is None) == (z_out is None), ValueError, lambda: "s_out and z_out go together")
+    if s_out is None:
+        s_out, z_out = s, z
+    else:
+        _check_f32_cuda("s_out", s_out, (B, H, 2 * D, d))
+        _check_f32_cuda("z_out", z_out, (B, H, 2 * D))
     out = torch.empty_like(v)
     with _on_device(v.device):
-        _lib.check(_lib.load().rfa_incremental_fused(
+        _lib.check(_lib.load().rfa_incremental_fused_out(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), w.data_ptr(), float(scale), s.data_ptr(), z.data_ptr(),
-            out.data_ptr(), steps, B, H, D, d, _stream_ptr(v.device)))
+            s_out.data_ptr(), z_out.data_ptr(), out.data_ptr(), steps, B, H, D, d, _stream_ptr(v.device)))
     return out
 
 

@@ -22,3 +22,19 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def knobs():
+    """knobs(nseg=2, prefix=1): set launch-heuristic overrides of the library for one test; every
+    knob is back at -1 (the heuristic) afterwards."""
+    from rfa_amd import _lib
+    touched = []
+
+    def set_(**kw):
+        for name, value in kw.items():
+            touched.append(name)
+            _lib.tuning_set(name, value)
+    yield set_
+    for name in touched:
+        _lib.tuning_set(name, -1)

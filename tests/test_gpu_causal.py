@@ -131,18 +131,14 @@ def test_saved_pair_clamped_and_unclamped_rows():
 
 @pytest.mark.parametrize("nseg,scanned", [(1, None), (2, None), (3, None), (8, None), (16, None),
                                           (2, "1"), (3, "1"), (11, "1"), (8, "0"), (1, "1")])
-def test_every_segment_count_gives_the_same_answer(nseg, scanned, monkeypatch):
-    """RFA_HIP_NSEG overrides the number of time segments per sequence; the plain pair, the
+def test_every_segment_count_gives_the_same_answer(nseg, scanned, knobs):
+    """The "nseg" knob overrides the number of time segments per sequence; the plain pair, the
     saved pair and the prefill state must meet the oracle for any of them (ragged last segment,
-    single-chunk segments, one segment for the whole sequence).  RFA_HIP_PREFIX forces the
+    single-chunk segments, one segment for the whole sequence).  The "prefix" knob forces the
     consumers to add up the segment totals themselves ("0") or to read totals that a scan
     kernel turned into running sums first ("1"); unset, five segments or more take the scan."""
     from rfa_amd import rfa_hip
-    monkeypatch.setenv("RFA_HIP_NSEG", str(nseg))
-    if scanned is None:
-        monkeypatch.delenv("RFA_HIP_PREFIX", raising=False)
-    else:
-        monkeypatch.setenv("RFA_HIP_PREFIX", scanned)
+    knobs(nseg=nseg, prefix=-1 if scanned is None else int(scanned))
     T, B, H, d, D = 700, 1, 3, 64, 64
     cpu = _features(T, B, H, d, D, seed=5000)
     pq, pk, v, g = (t.cuda() for t in cpu)
@@ -162,17 +158,12 @@ def test_every_segment_count_gives_the_same_answer(nseg, scanned, monkeypatch):
 
 
 @pytest.mark.parametrize("nseg,same", [(8, False), (4, False), (6, False), (8, True), (5, False)])
-def test_wide_state_backward_on_half_as_many_segments(nseg, same, monkeypatch):
+def test_wide_state_backward_on_half_as_many_segments(nseg, same, knobs):
     """K = 256, d = 128: with scanned totals the saved-pair backward runs on segments twice as long
-    as the forward's (even segment counts; RFA_HIP_NSEG_SAME keeps them equal); out and gradients
+    as the forward's (even segment counts; the "nseg_same" knob keeps them equal); out and gradients
     must meet the oracle either way, and the plain pair as well."""
     from rfa_amd import rfa_hip
-    monkeypatch.setenv("RFA_HIP_NSEG", str(nseg))
-    monkeypatch.delenv("RFA_HIP_PREFIX", raising=False)
-    if same:
-        monkeypatch.setenv("RFA_HIP_NSEG_SAME", "1")
-    else:
-        monkeypatch.delenv("RFA_HIP_NSEG_SAME", raising=False)
+    knobs(nseg=nseg, prefix=-1, nseg_same=1 if same else -1)
     T, B, H, d, D = 1100, 1, 2, 128, 128
     cpu = _features(T, B, H, d, D, seed=5100)
     pq, pk, v, g = (t.cuda() for t in cpu)
@@ -257,3 +248,37 @@ def test_two_threads_on_two_streams_agree_with_one():
     for i in range(2):
         for a, b in zip(got[i], want[i]):
             assert torch.equal(a, b)
+
+
+def test_saved_buffer_carries_the_plan_of_its_forward(knobs):
+    """The forward writes its plan into the saved buffer and the library remembers it: a backward
+    call runs with that plan whatever the knobs say by then; a buffer the library has no record
+    of (here: a copy) whose header differs from the current plan yields NaN gradients, never
+    numbers computed from totals laid out for another plan; another shape is an error."""
+    import ctypes
+    from rfa_amd import _lib, rfa_hip
+    T, B, H, d, D = 700, 1, 3, 64, 64
+    cpu = _features(T, B, H, d, D, seed=5200)
+    pq, pk, v, g = (t.cuda() for t in cpu)
+    want = _oracle_bwd(*cpu)
+    knobs(nseg=4, prefix=0)
+    out, saved = rfa_hip.forward_save(pq, pk, v)
+    words = (ctypes.c_int32 * 16)()
+    _lib.check(_lib.load().rfa_causal_saved_describe(saved.data_ptr(), words, None))
+    assert words[0] == 0x52464153 and (words[3], words[4], words[5], words[7]) == (2 * D, d, 4, 0)
+    assert (words[8], words[10]) == (T, B * H) and saved.numel() == _lib.load().rfa_causal_saved_state_bytes(T, B * H, 2 * D, d)
+    knobs(nseg=8, prefix=1)                     # the knobs move between forward and backward
+    for name, a, b in zip(("dq", "dk", "dv"), rfa_hip.backward_saved(pq, pk, v, g, out, saved), want):
+        assert _rel(a.float().cpu(), b) <= GRAD_RTOL, name
+    stray = torch.empty(saved.numel() + 4096, dtype=torch.uint8, device="cuda")[:saved.numel()].copy_(saved)
+    assert stray.data_ptr() != saved.data_ptr()
+    big = torch.empty(1 << 24, dtype=torch.uint8, device="cuda")       # room for the 8-segment layout
+    big[:saved.numel()].copy_(saved)
+    grads = rfa_hip.backward_saved(pq, pk, v, g, out, big)
+    assert all(torch.isnan(t.float()).all() for t in grads)
+    knobs(nseg=4, prefix=0)                     # back on the forward's plan: the copy is as good as the original
+    for name, a, b in zip(("dq", "dk", "dv"), rfa_hip.backward_saved(pq, pk, v, g, out, stray), want):
+        assert _rel(a.float().cpu(), b) <= GRAD_RTOL, name
+    with pytest.raises(_lib.RfaHipError, match="another shape"):
+        rfa_hip.backward_saved(pq[:640].contiguous(), pk[:640].contiguous(), v[:640].contiguous(), g[:640].contiguous(),
+                               out[:640].contiguous(), saved)

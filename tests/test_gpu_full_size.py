@@ -156,7 +156,7 @@ def test_decode_full_size_config4():
 
 
 @pytest.mark.parametrize("nseg", [None, 2])
-def test_element_offsets_beyond_32_bits(nseg, monkeypatch):
+def test_element_offsets_beyond_32_bits(nseg, knobs):
     """phi tensors of 2.28e9 elements (4.6 GB each): every kernel forms offsets past 2**31 elements
     and 2**32 bytes.  Sequences are independent, so a handful of them run as a small problem of
     their own (same cut into segments) must reproduce their slices of the large run bit for bit;
@@ -165,10 +165,7 @@ def test_element_offsets_beyond_32_bits(nseg, monkeypatch):
     T, B, H, d, D = 1088, 2050, 8, 64, 64          # 17 chunks of 64 steps, 16400 sequences
     N, K = B * H, 2 * D
     assert T * N * K > 2 ** 31
-    if nseg is not None:
-        monkeypatch.setenv("RFA_HIP_NSEG", str(nseg))
-    else:
-        monkeypatch.setenv("RFA_HIP_NSEG", "1")
+    knobs(nseg=nseg if nseg is not None else 1)
     print(f"offsets beyond 32 bits: T={T} N={N} K={K} d={d} segments={nseg or 1}", flush=True)
     torch.manual_seed(77)
     unit = lambda t: t / t.norm(dim=-1, keepdim=True)

@@ -90,6 +90,39 @@ def test_causal_module_decode_equals_training_forward():
     assert (quad[8:].float() - full[8:].float()).abs().max().item() <= 2e-2
 
 
+def test_causal_module_decode_leaves_earlier_states_alone():
+    """The reference builds a new state every step (causal_attention.py:42-43, 262): a tensor the
+    caller holds from step t is unchanged after step t + 1.  decode_inplace = True advances the
+    tensors where they are, with the same numbers."""
+    from rfa_amd import CausalAttention
+    torch.manual_seed(3)
+    T, B, E, H, d, D = 6, 2, 128, 2, 64, 64
+    m = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half().eval()
+    x = torch.randn(T, B, E).cuda().half()
+    W = O.make_w(d, D, H).cuda().half()
+    with torch.no_grad():
+        state, held, rows = {}, [], []
+        for t in range(T):
+            rows.append(m(x[t:t + 1], W, saved_state=state))
+            held.append((state["prev_s"], state["prev_z"], state["prev_s"].clone(), state["prev_z"].clone()))
+        for s, z, s_then, z_then in held:
+            assert torch.equal(s, s_then) and torch.equal(z, z_then)
+        assert len({h[0].data_ptr() for h in held}) == T
+        m.decode_inplace = True
+        state2, rows2 = {}, []
+        for t in range(T):
+            rows2.append(m(x[t:t + 1], W, saved_state=state2))
+            if t == 1:
+                ptr = state2["prev_s"].data_ptr()
+        assert state2["prev_s"].data_ptr() == ptr
+        assert torch.equal(torch.cat(rows), torch.cat(rows2)) and torch.equal(state["prev_s"], state2["prev_s"])
+        # a user-supplied fp16 state is converted (a private copy), never written
+        half_state = {"prev_s": held[2][0].half(), "prev_z": held[2][1].half()}
+        keep = half_state["prev_s"].clone()
+        m(x[3:4], W, saved_state=half_state)
+        assert half_state["prev_s"].dtype == torch.float32 and torch.equal(keep, held[2][0].half())
+
+
 def test_causal_module_training_step_runs_and_matches_oracle():
     from rfa_amd import CausalAttention
     torch.manual_seed(1)

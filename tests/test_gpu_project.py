@@ -40,14 +40,11 @@ def _linear64(x, w, b, H, d):
 
 @pytest.mark.parametrize("streaming", [False, True])
 @pytest.mark.parametrize("L,B,E,H,d,D", SHAPES)
-def test_qkv_projection_with_feature_map(L, B, E, H, d, D, streaming, monkeypatch):
+def test_qkv_projection_with_feature_map(L, B, E, H, d, D, streaming, knobs):
     """Both kernels: the one that keeps its rows of x in LDS (picked when they fit) and the one
-    that streams x and the weights together (forced by RFA_HIP_PROJECT_STREAMING)."""
+    that streams x and the weights together (forced by the "project_streaming" knob)."""
     from rfa_amd import rfa_hip
-    if streaming:
-        monkeypatch.setenv("RFA_HIP_PROJECT_STREAMING", "1")
-    else:
-        monkeypatch.delenv("RFA_HIP_PROJECT_STREAMING", raising=False)
+    knobs(project_streaming=1 if streaming else -1)
     x, ws, bs = _inputs(L, B, E, H, d, 900 + L, 3)
     bs[1] = None                                       # one projection without bias
     wf = (_randn(H, D, d, seed=77) * 0.9).half()

@@ -25,13 +25,30 @@ def test_shape_support_and_workspace_queries():
     assert lib.rfa_shape_supported(128, 64) == 1 and lib.rfa_shape_supported(256, 128) == 1
     assert lib.rfa_shape_supported(100, 64) == 0 and lib.rfa_shape_supported(128, 48) == 0
     assert lib.rfa_feature_map_supported(64, 64) == 1 and lib.rfa_feature_map_supported(48, 64) == 0
-    assert lib.rfa_causal_num_segments(1024, 64) >= 1
-    assert lib.rfa_causal_num_segments(64, 1) == 1          # one chunk cannot be split
+    assert lib.rfa_causal_num_segments(1024, 64, 128, 64) >= 1
+    assert lib.rfa_causal_num_segments(64, 1, 128, 64) == 1          # one chunk cannot be split
     assert lib.rfa_causal_forward_workspace_bytes(0, 4, 128, 64) == 0
     fw = lib.rfa_causal_forward_workspace_bytes(1024, 64, 128, 64)
     bw = lib.rfa_causal_backward_workspace_bytes(1024, 64, 128, 64)
     assert bw > fw >= 0 and bw >= 2 * 1024 * 64 * 4
     assert lib.rfa_feature_map_backward_workspace_bytes(8192, 8, 64, 64) >= 8 * 64 * 64 * 4
+
+
+def test_tuning_knobs_round_trip():
+    lib = _lib.load()
+    assert _lib.tuning_get("nseg") == -1
+    with _lib.tuning(nseg=3, prefix=1):
+        assert _lib.tuning_get("nseg") == 3 and _lib.tuning_get("prefix") == 1
+        assert lib.rfa_causal_num_segments(1024, 64, 128, 64) == 3
+    assert _lib.tuning_get("nseg") == -1 and _lib.tuning_get("prefix") == -1
+    with pytest.raises(_lib.RfaHipError, match="no knob"):
+        _lib.tuning_set("no_such_knob", 1)
+    # the saved buffer grows by its 256-byte header and follows the plan
+    with _lib.tuning(nseg=1):
+        one = lib.rfa_causal_saved_state_bytes(1024, 64, 128, 64)
+    with _lib.tuning(nseg=4, prefix=0):
+        four = lib.rfa_causal_saved_state_bytes(1024, 64, 128, 64)
+    assert one >= 256 + 64 * (128 * 64 + 128) * 4 + 1024 * 64 * 4 and four >= one + 3 * 64 * 128 * 64 * 4
 
 
 def test_errors_are_reported_before_any_gpu_work():
