@@ -78,6 +78,19 @@ int rfa_causal_forward(const void* q, const void* k, const void* v, void* out, i
                        int64_t N, int K, int d, void* workspace, size_t workspace_bytes,
                        void* stream);
 
+/* rfa_causal_forward for callers that cannot allocate and have no workspace to pass (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): no counterpart in the
+ * reference.  Same kernels and results as rfa_causal_forward; the segment totals live in a static
+ * device array of rfa_static_scratch_bytes() = 16 MiB that every GPU the library runs on holds
+ * until the process ends.  The call allocates and frees nothing.  Shapes whose
+ * rfa_causal_forward_workspace_bytes exceed the array return RFA_ERR_WORKSPACE.  All calls on one
+ * GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads)
+ * race; calls on one stream, one after the other, are fine (nothing in the array has to start
+ * at zero: every total the scan reads is written earlier in the same call). */
+size_t rfa_static_scratch_bytes(void);
+int rfa_causal_forward_noalloc(const void* q, const void* k, const void* v, void* out, int64_t T,
+                               int64_t N, int K, int d, void* stream);
+
 /* Prefill for incremental decoding: rfa_causal_forward over a prompt of T steps that also
  * returns the state after the last step, s fp32 [N, K, d] and z fp32 [N, K] (every element
  * written; zero for T = 0), from which rfa_incremental / rfa_incremental_fused continue.

@@ -42,6 +42,8 @@ SIGNATURES = {
     "rfa_causal_saved_describe": (c_int, [c_void_p, POINTER(ctypes.c_int32), c_void_p]),
     "rfa_causal_forward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
     "rfa_causal_forward": (c_int, [c_void_p] * 4 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "rfa_static_scratch_bytes": (c_size_t, []),
+    "rfa_causal_forward_noalloc": (c_int, [c_void_p] * 4 + [c_int64, c_int64, c_int, c_int, c_void_p]),
     "rfa_causal_prefill": (c_int, [c_void_p] * 6 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "rfa_causal_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
     "rfa_causal_backward": (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),

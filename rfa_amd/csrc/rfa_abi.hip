@@ -713,6 +713,9 @@ int check_causal_dims(int64_t T, int64_t N, int K, int d) {
 // until the process ends.  In host code such a name is a stand-in, not a device address: the
 // address on the current device comes from hipGetSymbolAddress, once per device.
 static __device__ int g_selftest_word;        // result word of rfa_selftest_layout
+// workspace of rfa_causal_forward_noalloc: the segment totals of one forward call
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
 
@@ -728,6 +731,16 @@ int cached_symbol_address(std::atomic<void*>* cache, hipError_t (*lookup)(void**
         cache[dev].store(p, std::memory_order_release);
     }
     *out = p;
+    return RFA_OK;
+}
+
+// this device's copy of `scratch`: host code uses this pointer, never the array's name
+int static_scratch_address(unsigned char** out) {
+    static std::atomic<void*> cache[kMaxDevices];
+    void* ptr = nullptr;
+    if (int rc = cached_symbol_address(cache, [](void** q) { return hipGetSymbolAddress(q, HIP_SYMBOL(scratch)); }, &ptr))
+        return rc;
+    *out = static_cast<unsigned char*>(ptr);
     return RFA_OK;
 }
 
@@ -945,6 +958,25 @@ int rfa_causal_forward(const void* q, const void* k, const void* v, void* out, i
                        int K, int d, void* workspace, size_t workspace_bytes, void* stream) {
     return causal_forward_impl(q, k, v, out, T, N, K, d, nullptr, 0, false, nullptr, nullptr, workspace,
                                workspace_bytes, stream);
+}
+
+size_t rfa_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int rfa_causal_forward_noalloc(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
+                               int K, int d, void* stream) {
+    if (int rc = check_causal_dims(T, N, K, d)) return rc;
+    if (T == 0 || N == 0) return RFA_OK;
+    const size_t need = rfa_causal_forward_workspace_bytes(T, N, K, d);
+    if (need > kStaticScratchBytes)
+        return fail(RFA_ERR_WORKSPACE,
+                    "rfa_causal_forward_noalloc: this shape needs %zu bytes of segment totals, the static scratch "
+                    "holds %zu; use rfa_causal_forward with a caller-owned workspace", need, kStaticScratchBytes);
+    unsigned char* ptr = nullptr;       // this device's copy of the static array
+    if (int rc = static_scratch_address(&ptr)) return rc;
+    // every slot of the segment totals that the scan reads is written by the totals pass of the same
+    // call first, so what an earlier call left in the array does not matter
+    return causal_forward_impl(q, k, v, out, T, N, K, d, nullptr, 0, false, nullptr, nullptr, ptr, kStaticScratchBytes,
+                               stream);
 }
 
 int rfa_causal_prefill(const void* q, const void* k, const void* v, void* out, float* s, float* z, int64_t T,
