@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "rfa_causal.h"
+#include "rfa_sliced.h"
 #include "rfa_project.h"
 #include "rfa_decode.h"
 #include "rfa_featuremap.h"
@@ -44,13 +45,14 @@ int fail(int code, const char* fmt, ...) {
 namespace prof {
 enum Id { SEG_STATE, CAUSAL_FWD, CAUSAL_BWD_DQ, CAUSAL_BWD_DKDV, CROSS_READOUT, CROSS_READOUT_BWD,
           CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, MASKED_FWD, MASKED_PREP, MASKED_DQ, MASKED_DKDV, PROJECT_PHI, WGRAD_PARTIAL, WGRAD_REDUCE, TOTALS_SCAN, ZERO_FILL,
-          SELFTEST, BUILD_W, DECODE_TOUCH, COUNT };
+          SELFTEST, BUILD_W, DECODE_TOUCH, CAUSAL_BWD_SLICED, COUNT };
 const char* const kNames[COUNT] = {"k_segment_state", "k_causal_fwd", "k_causal_bwd_dq", "k_causal_bwd_dkdv",
                                    "k_cross_readout", "k_cross_readout_bwd", "k_cross_state_bwd", "k_decode_step",
                                    "k_feature_map_fwd", "k_feature_map_bwd", "k_feature_map_dw_reduce",
                                    "k_masked_fwd", "k_masked_bwd_prep", "k_masked_dq", "k_masked_dkdv", "k_project_phi",
                                    "k_weight_grad_partial", "k_weight_grad_reduce", "k_totals_scan",
-                                   "k_zero_f32", "k_selftest", "k_build_random_matrices", "k_touch_rows"};
+                                   "k_zero_f32", "k_selftest", "k_build_random_matrices", "k_touch_rows",
+                                   "k_sliced_bwd"};
 struct Rec { int id; hipEvent_t a, b; };
 std::mutex mu;
 bool enabled = false;
@@ -154,7 +156,25 @@ struct ScanPlan {
     int seg_len;   // steps per segment (multiple of 64)
     int prefixed;  // the consumers read one pre-scanned state (k_totals_scan) instead of adding up the
                    // segment totals themselves
+    int layout;    // what a saving forward leaves for the backward (SavedLayout)
 };
+
+// What rfa_causal_forward_save hands to the backward besides the raw denominators:
+//   LAYOUT_SEGMENTS  the per-segment state totals; the backward runs the two segment sweeps
+//   LAYOUT_FINAL     the state after the last step; the backward walks whole sequences backwards
+//                    in state slices (rfa_sliced.h), one launch, every chunk read once
+enum SavedLayout { LAYOUT_SEGMENTS = 0, LAYOUT_FINAL = 1 };
+
+bool sliced_supported(int K, int d) { return (K == 64 || K == 128) && (d == 64 || d == 128); }
+
+// The sliced backward has N * (K / 64 + d / 64) workgroups that never wait for each other: taken
+// when they cover most of the compute units ("sliced" knob: 0 never, 1 whenever a kernel exists).
+int choose_saved_layout(int64_t N, int K, int d) {
+    if (!sliced_supported(K, d)) return LAYOUT_SEGMENTS;
+    const int knob = tune::get(tune::SLICED);
+    if (knob >= 0) return knob ? LAYOUT_FINAL : LAYOUT_SEGMENTS;
+    return N * (K / rfa::kSliceWidth + d / rfa::kSliceWidth) * 10 >= (int64_t)device_cus() * 6 ? LAYOUT_FINAL : LAYOUT_SEGMENTS;
+}
 
 // Whether the consumers read one pre-scanned state instead of adding up the segment totals
 // themselves, (nseg - 1) / 2 states of K * d floats on average per workgroup: worth its pass over
@@ -170,8 +190,9 @@ bool use_scanned_totals(int nseg, int K, int d) {
 // chunks per segment, at most 16 segments (the consumer sums the totals of all
 // earlier segments).
 ScanPlan make_plan(int64_t T, int64_t N, int K, int d) {
-    ScanPlan p{1, rfa::kChunk, 0};
+    ScanPlan p{1, rfa::kChunk, 0, LAYOUT_SEGMENTS};
     if (T <= 0 || N <= 0) return p;
+    p.layout = choose_saved_layout(N, K, d);
     const int64_t nchunks = (T + rfa::kChunk - 1) / rfa::kChunk;
     int64_t want = (device_cus() + N - 1) / N;
     const int knob = tune::get(tune::NSEG);
@@ -192,13 +213,12 @@ ScanPlan make_plan(int64_t T, int64_t N, int K, int d) {
 
 // ---- description of a saved-state buffer ---------------------------------------------
 constexpr size_t kSavedHeaderBytes = 256;
-enum SavedLayout { LAYOUT_SEGMENTS = 0 };
 
-rfa::PlanWords plan_words(int layout, int64_t T, int64_t N, int K, int d, const ScanPlan& p) {
+rfa::PlanWords plan_words(int64_t T, int64_t N, int K, int d, const ScanPlan& p) {
     rfa::PlanWords w{};
     w.w[0] = rfa::kPlanMagic;
     w.w[1] = 1;
-    w.w[2] = layout;
+    w.w[2] = p.layout;
     w.w[3] = K;
     w.w[4] = d;
     w.w[5] = p.nseg;
@@ -302,7 +322,7 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     if (p.prefixed) launch_totals_scan<false>(wsS, (int64_t)KD * DH, wsZ, KD, N, p.nseg, st);
-    const rfa::PlanWords pw = plan_words(LAYOUT_SEGMENTS, T, N, KD, DH, p);
+    const rfa::PlanWords pw = plan_words(T, N, KD, DH, p);
     if constexpr (PIPE) {
         auto kern = rfa::k_causal_fwd_pipe<KD, DH>;
         if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
@@ -345,7 +365,7 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
     const ScanPlan p = backward_plan(pf, KD, DH, savedS != nullptr, &s_ratio);
     const int prefixed_s = pf.prefixed;
     const int prefixed = p.prefixed;   // of dR, dr
-    const rfa::PlanWords pw = plan_words(LAYOUT_SEGMENTS, T, N, KD, DH, pf);
+    const rfa::PlanWords pw = plan_words(T, N, KD, DH, pf);
     constexpr int NW = causal_waves(KD, DH);
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     float* wsS = reinterpret_cast<float*>(ws + wl.S);
@@ -432,10 +452,30 @@ int launch_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_
     return RFA_OK;
 }
 
+// backward of a forward that left its final state (LAYOUT_FINAL): one launch, no workspace
+template <int KD, int DH>
+int launch_sliced_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, const rfa::half_t* g,
+                           const rfa::half_t* out, rfa::half_t* dq, rfa::half_t* dk, rfa::half_t* dv, int T, int N,
+                           const ScanPlan& pf, const int* savedHdr, const float* finalS, const float* finalZ,
+                           const float* savedDen, hipStream_t st) {
+    if constexpr (KD <= 128) {
+        using Cfg = rfa::SlicedBwdCfg<KD, DH>;
+        auto kern = rfa::k_sliced_bwd<KD, DH>;
+        if (int rc = set_lds(kern, Cfg::kLds)) return rc;
+        const int64_t grid = (int64_t)rfa::kXcds * ((N + rfa::kXcds - 1) / rfa::kXcds) * (Cfg::NA + Cfg::NB);
+        RFA_LAUNCH(CAUSAL_BWD_SLICED, kern, dim3((unsigned)grid), dim3(rfa::kSlicedThreads), Cfg::kLds, st, q, k, v, g, out,
+                   savedDen, finalS, finalZ, dq, dk, dv, T, N, savedHdr, plan_words(T, N, KD, DH, pf));
+        RFA_HIP_TRY(hipGetLastError());
+        return RFA_OK;
+    } else {
+        return fail(RFA_ERR_UNSUPPORTED, "no sliced backward for K=%d d=%d", KD, DH);
+    }
+}
+
 // ---- cross attention launchers ---------------------------------------------------
 // time split for kernels whose workgroups do not depend on each other
 ScanPlan make_free_plan(int64_t T, int64_t N) {
-    ScanPlan p{1, rfa::kChunk, 0};
+    ScanPlan p{1, rfa::kChunk, 0, LAYOUT_SEGMENTS};
     if (T <= 0 || N <= 0) return p;
     const int64_t nchunks = (T + rfa::kChunk - 1) / rfa::kChunk;
     int64_t target = 2 * device_cus();      // workgroups to aim for: two per compute unit
@@ -896,14 +936,16 @@ size_t rfa_causal_backward_workspace_bytes(int64_t T, int64_t N, int K, int d) {
     if (K == 256 && d == 128) { return CALL(256, 128); }
 
 // The saved buffer: a 256-byte header (rfa::PlanWords: the plan of the forward that wrote the
-// buffer), the segment totals S (fragment order), z, and the raw denominators.
+// buffer), then S and z -- the segment totals (S in fragment order) or, with LAYOUT_FINAL, the
+// state after the last step ([N][K][d], [N][K]) -- and the raw denominators.
 struct SavedLayoutBytes { size_t S, Z, den, total; };
 
 static SavedLayoutBytes saved_layout(int64_t T, int64_t N, int K, int d, const ScanPlan& p) {
     SavedLayoutBytes l{};
     size_t off = kSavedHeaderBytes;
-    l.S = off; off += align_up((size_t)N * p.nseg * K * d * 4);
-    l.Z = off; off += align_up((size_t)N * p.nseg * K * 4);
+    const size_t states = (size_t)N * (p.layout == LAYOUT_FINAL ? 1 : p.nseg);
+    l.S = off; off += align_up(states * K * d * 4);
+    l.Z = off; off += align_up(states * K * 4);
     l.den = off; off += align_up((size_t)T * N * 4);
     l.total = off;
     return l;
@@ -920,7 +962,7 @@ size_t rfa_causal_saved_state_bytes(int64_t T, int64_t N, int K, int d) {
 static int saved_plan(const char* fn, const void* saved, int64_t T, int64_t N, int K, int d, ScanPlan* p) {
     rfa::PlanWords w;
     if (saved && registry::get(saved, &w)) {
-        const rfa::PlanWords same = plan_words(w.w[2], T, N, K, d, ScanPlan{w.w[5], w.w[6], w.w[7]});
+        const rfa::PlanWords same = plan_words(T, N, K, d, ScanPlan{w.w[5], w.w[6], w.w[7], w.w[2]});
         if (memcmp(&w, &same, sizeof(w)) != 0)
             return fail(RFA_ERR_WORKSPACE,
                         "%s: the saved buffer was written by a forward call of another shape (T=%lld N=%lld K=%d d=%d), "
@@ -928,7 +970,7 @@ static int saved_plan(const char* fn, const void* saved, int64_t T, int64_t N, i
                         (long long)(((int64_t)w.w[9] << 32) | (uint32_t)w.w[8]),
                         (long long)(((int64_t)w.w[11] << 32) | (uint32_t)w.w[10]), w.w[3], w.w[4], (long long)T,
                         (long long)N, K, d);
-        *p = ScanPlan{w.w[5], w.w[6], w.w[7]};
+        *p = ScanPlan{w.w[5], w.w[6], w.w[7], w.w[2]};
         return RFA_OK;
     }
     *p = make_plan(T, N, K, d);
@@ -939,6 +981,7 @@ size_t rfa_causal_backward_saved_workspace_bytes(const void* saved, int64_t T, i
     if (T <= 0 || N <= 0 || !rfa_shape_supported(K, d)) return 0;
     ScanPlan p;
     if (saved_plan("rfa_causal_backward_saved_workspace_bytes", saved, T, N, K, d, &p) != RFA_OK) return 0;
+    if (p.layout == LAYOUT_FINAL) return 0;
     return layout_workspace(T, N, K, d, p, true).total;
 }
 
@@ -1026,8 +1069,15 @@ static int causal_forward_impl(const void* q, const void* k, const void* v, void
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
         return fail(RFA_ERR_ALIGNMENT, "rfa_causal_forward: tensors must be 16-byte aligned");
     const Workspace wl = layout_workspace(T, N, K, d, p, false);
-    // with a saved buffer the segment totals go there and the workspace is not touched
-    if (!want_saved && wl.total > 0 && (!workspace || workspace_bytes < wl.total || !aligned16(workspace)))
+    if (want_saved && p.layout == LAYOUT_FINAL) {
+        // the buffer gets the state after the last step; the segment totals stay in the workspace
+        final_s = savedS;
+        final_z = savedZ;
+        savedS = nullptr;
+        savedZ = nullptr;
+    }
+    // with the segment totals in the saved buffer the workspace is not touched
+    if (!savedS && wl.total > 0 && (!workspace || workspace_bytes < wl.total || !aligned16(workspace)))
         return fail(RFA_ERR_WORKSPACE, "rfa_causal_forward: workspace of %zu bytes required, got %zu", wl.total,
                     workspace ? workspace_bytes : (size_t)0);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -1036,7 +1086,7 @@ static int causal_forward_impl(const void* q, const void* k, const void* v, void
     auto* vh = static_cast<const rfa::half_t*>(v);
     auto* oh = static_cast<rfa::half_t*>(out);
     char* ws = static_cast<char*>(workspace);
-    if (want_saved) registry::put(saved, plan_words(LAYOUT_SEGMENTS, T, N, K, d, p));
+    if (want_saved) registry::put(saved, plan_words(T, N, K, d, p));
 #define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedHdr, savedS, savedZ, savedDen, final_s, final_z, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_FWD)
 #undef RFA_CALL_FWD
@@ -1097,8 +1147,9 @@ static int causal_backward_impl(const void* q, const void* k, const void* v, con
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(grad_attn) || !aligned16(dq) ||
         !aligned16(dk) || !aligned16(dv))
         return fail(RFA_ERR_ALIGNMENT, "rfa_causal_backward: tensors must be 16-byte aligned");
+    const bool sliced = have_saved && p.layout == LAYOUT_FINAL;
     const Workspace wl = layout_workspace(T, N, K, d, p, true);
-    if (!workspace || workspace_bytes < wl.total || !aligned16(workspace))
+    if (!sliced && (!workspace || workspace_bytes < wl.total || !aligned16(workspace)))
         return fail(RFA_ERR_WORKSPACE, "rfa_causal_backward: workspace of %zu bytes required, got %zu", wl.total,
                     workspace ? workspace_bytes : (size_t)0);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -1111,6 +1162,11 @@ static int causal_backward_impl(const void* q, const void* k, const void* v, con
     auto* dkh = static_cast<rfa::half_t*>(dk);
     auto* dvh = static_cast<rfa::half_t*>(dv);
     char* ws = static_cast<char*>(workspace);
+    if (sliced) {
+#define RFA_CALL_SL(KD, DH) launch_sliced_backward<KD, DH>(qh, kh, vh, gh, outh, dqh, dkh, dvh, (int)T, (int)N, p, savedHdr, savedS, savedZ, savedDen, st)
+        RFA_DISPATCH_KD(K, d, RFA_CALL_SL)
+#undef RFA_CALL_SL
+    }
 #define RFA_CALL_BWD(KD, DH) launch_backward<KD, DH>(qh, kh, vh, gh, outh, dqh, dkh, dvh, (int)T, (int)N, p, ws, wl, savedHdr, savedS, savedZ, savedDen, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_BWD)
 #undef RFA_CALL_BWD

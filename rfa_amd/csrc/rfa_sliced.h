@@ -1,0 +1,518 @@
+// Causal random-feature attention without time segments (gfx950): parallelism from slices of
+// the state instead of from cutting the sequence.
+//
+// The chunked scan of rfa_causal.h cuts a sequence into time segments so that bsz * heads
+// sequences fill the GPU; every segment then needs the state at its first step, which costs a
+// pass over k, v (forward) and over q, g (backward) for the segment totals, and two sweeps over
+// the sequence in the backward (dQ needs the sum over earlier steps, dK and dV the sum over later
+// ones).  Here a workgroup walks a whole sequence and owns a slice of the state:
+//
+//   backward, feature slice  [koff, koff + 64) of phi:   dQ[:, slice], dK[:, slice]
+//       carries S[slice, :] and R[slice, :]   (reads g, out, v whole; q, k slice)
+//   backward, value slice    [coff, coff + 64) of v:      dV[:, slice]
+//       carries R[:, slice]                    (reads q, k whole; g slice)
+//
+// with  S = sum_{s <= t} phi_k[s] (x) v[s],  R = sum_{s > t} phi_q[s] (x) g^[s],  g^ = g / den
+// (rfa.py:66-103).  Both run backwards in time.  R grows as the sweep proceeds; S of the chunk
+// before the current one is the forward's final state minus what the sweep has passed, so the
+// backward needs no totals pass, no second sweep, and reads every chunk of q, k, v, g, out once
+// from HBM (the slices of one sequence sit on one XCD and walk in step, so the rows they share
+// come out of that L2).  The dQ/dK slices and the dV slices of a sequence are separate
+// workgroups of one launch.
+//
+// Formulas per 64-step chunk (Q, K: 64 x KD;  V, G^: 64 x DH;  gz_i = [den_raw_i > 1] * -(g_i . out_i) / den_i):
+//     P  = tril(G^ V^T + gz 1^T)              A = tril(Q K^T)
+//     dQ = P K + G^ S_prev^T + gz z_prev^T     (S_prev, z_prev: state before the chunk)
+//     dK = P^T Q + V R_next^T + 1 r_next^T     (R_next, r_next: sums over later chunks)
+//     dV = A^T G^ + K R_next
+#pragma once
+#include <type_traits>
+
+#include "rfa_common.h"
+
+namespace rfa {
+
+constexpr int kSliceWidth = 64;    // features (dQ/dK role) or value columns (dV role) per workgroup
+constexpr int kSlicedThreads = 512; // 8 waves, two per SIMD
+
+// Workgroup index -> (sequence, role).  The wps workgroups of a sequence get indices that are
+// equal mod kXcds, i.e. the same XCD, and consecutive positions there.
+__device__ __forceinline__ void seq_role_of_block(int b, int wps, int& n, int& role) {
+    const int xcd = b % kXcds, l = b / kXcds;
+    role = l % wps;
+    n = kXcds * (l / wps) + xcd;
+}
+
+template <int KD, int DH>
+struct SlicedBwdCfg {
+    static constexpr int C = kChunk, KSL = kSliceWidth, CSL = kSliceWidth;
+    static constexpr int NA = KD / KSL;             // dQ/dK workgroups per sequence
+    static constexpr int NB = DH / CSL;             // dV workgroups per sequence
+    static constexpr int LDS_ = KSL + lds_pad(KSL); // row stride of a 64-wide slice array
+    static constexpr int LDQ = KD + lds_pad(KD);
+    static constexpr int LDV = DH + lds_pad(DH);
+    static constexpr int LDA = C + 8;
+    // dQ/dK role: two stages of [Q slice | K slice | V | G^ | gz], one P
+    static constexpr size_t kStageA = (size_t)(2 * C * LDS_ + 2 * C * LDV) * 2 + C * 4;
+    static constexpr size_t kLdsA = 2 * kStageA + (size_t)C * LDA * 2;
+    // dV role: two stages of [Q | K | G^ slice], one A^T
+    static constexpr size_t kStageB = (size_t)(2 * C * LDQ + C * LDS_) * 2;
+    static constexpr size_t kLdsB = 2 * kStageB + (size_t)C * LDA * 2;
+    static constexpr size_t kLds = kLdsA > kLdsB ? kLdsA : kLdsB;
+    static_assert(kStageA % 16 == 0 && kStageB % 16 == 0, "stage alignment");
+};
+
+// ---------------------------------------------------------------------------
+// dQ, dK for features [koff, koff + 64) of one sequence.  8 waves, two per SIMD, in two groups
+// that share the chunk arrays and the P tiles and otherwise run their own loop (same number of
+// barriers):  waves 0-3 carry -S^T and -z and produce dQ, waves 4-7 carry R^T and r and produce
+// dK.  Wave (group, wf) owns features kw = koff + 16 wf .. + 15:
+//   NS[ct] = -S^T tile (c = 16ct + 4G + e, k = kw + i),  RT[ct] = R^T tile,  nz = -z and r as
+//   tiles (k = kw + 4G + e).  S and z are carried negated so that the MFMA can step them
+//   backwards by adding K^T V.
+// ---------------------------------------------------------------------------
+template <int KD, int DH>
+__device__ __forceinline__ void sliced_bwd_dqdk(
+    unsigned char* smem, int n, int koff, const half_t* __restrict__ q, const half_t* __restrict__ k,
+    const half_t* __restrict__ v, const half_t* __restrict__ g, const half_t* __restrict__ o,
+    const float* __restrict__ den_raw, half_t* __restrict__ dq, half_t* __restrict__ dk,
+    const float* __restrict__ final_s, const float* __restrict__ final_z, int T, int N) {
+    using Cfg = SlicedBwdCfg<KD, DH>;
+    constexpr int NT = kSlicedThreads, C = Cfg::C, KSL = Cfg::KSL;
+    constexpr int LDK = Cfg::LDS_, LDV = Cfg::LDV, LDA = Cfg::LDA;
+    constexpr int NCT = DH / 16;
+    constexpr int PPR = DH / 8, VP = ChunkRegs<DH, NT>::kPieces;
+    half_t* Ps = reinterpret_cast<half_t*>(smem + 2 * Cfg::kStageA);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, G = lane >> 4;
+    const int wf = w & 3;
+    const bool dq_group = w < 4;
+    const int kl = 16 * wf;                     // first feature of this wave, local to the slice arrays
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+    const half_t* qb = q + (int64_t)n * KD + koff;
+    const half_t* kb = k + (int64_t)n * KD + koff;
+    const half_t* vb = v + (int64_t)n * DH;
+    const half_t* gb = g + (int64_t)n * DH;
+    const half_t* ob = o + (int64_t)n * DH;
+    half_t* dqb = dq + (int64_t)n * KD + koff;
+    half_t* dkb = dk + (int64_t)n * KD + koff;
+    RFA_TICK_INIT();
+    constexpr int TB = 0;
+
+    // Two register sets of chunk rows: while chunk c is worked on, the rows of chunks c - 1 and
+    // c - 2 are on their way, so a load has two chunk periods to arrive.
+    struct RowSet {
+        ChunkRegs<KSL, NT> rq, rk;
+        ChunkRegs<DH, NT> rv, rg, ro;
+        float dn[VP];
+    };
+    RowSet s0, s1;
+    // branch-free: c may be a chunk that is never used (clamped by the caller to an existing one)
+    auto prefetch = [&](RowSet& r, int c) __attribute__((always_inline)) {
+        const int t0 = c * C, rows = T - t0;
+        chunk_g2r<KSL, NT>(r.rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<KSL, NT>(r.rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<DH, NT>(r.rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+        chunk_g2r<DH, NT>(r.rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+        chunk_g2r<DH, NT>(r.ro, ob + (int64_t)t0 * v_stride, v_stride, rows, tid);
+#pragma unroll
+        for (int it = 0; it < VP; ++it) {
+            const int r_ = min((tid + NT * it) / PPR, r.rg.rows - 1);
+            r.dn[it] = den_raw[(int64_t)(t0 + r_) * N + n];
+        }
+    };
+
+    struct Stage { half_t *Qs, *Ks, *Vs, *Gs; float* gzs; };
+    auto stage_of = [&](int ci) __attribute__((always_inline)) {
+        Stage st;
+        st.Qs = reinterpret_cast<half_t*>(smem + (ci & 1) * Cfg::kStageA);
+        st.Ks = st.Qs + C * LDK;
+        st.Vs = st.Ks + C * LDK;
+        st.Gs = st.Vs + C * LDV;                 // G / den
+        st.gzs = reinterpret_cast<float*>(st.Gs + C * LDV);
+        return st;
+    };
+
+    // rows in `r` -> LDS: Q, K slices, V, G^ = G / den, gz from g . out (the PPR lanes holding one
+    // row are adjacent); first barrier of the chunk; then chunk c_next is requested into `r`
+    auto stage_in = [&](const Stage& st, RowSet& r, int c_next) __attribute__((always_inline)) {
+        chunk_r2s<KSL, NT>(r.rq, st.Qs, LDK, tid);
+        chunk_r2s<KSL, NT>(r.rk, st.Ks, LDK, tid);
+        chunk_r2s<DH, NT>(r.rv, st.Vs, LDV, tid);
+#pragma unroll
+        for (int it = 0; it < VP; ++it) {
+            const int pc = tid + NT * it;
+            const int r_ = pc / PPR, c8 = pc % PPR;
+            union { uint4 u; h8 h; } xg, xo;
+            xg.u = r.rg.v[it];
+            xo.u = r.ro.v[it];
+            float dot = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dot += (float)xg.h[e] * (float)xo.h[e];
+#pragma unroll
+            for (int m = 1; m < PPR; m <<= 1) dot += __shfl_xor(dot, m, 64);
+            const bool valid = r_ < r.rg.rows;
+            const float inv = valid ? 1.0f / fmaxf(r.dn[it], 1.0f) : 0.f;
+            const float gzv = (valid && r.dn[it] > 1.0f) ? -dot * inv : 0.f;
+            h8 y;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)xg.h[e] * inv);
+            *reinterpret_cast<h8*>(st.Gs + r_ * LDV + c8 * 8) = y;
+            if (c8 == 0) st.gzs[r_] = gzv;
+        }
+        RFA_TICK(TB + 1);
+        __syncthreads();
+        RFA_TICK(TB + 2);
+        prefetch(r, c_next);
+        RFA_TICK(TB + 3);
+    };
+
+    // P = tril(G^ V^T + gz 1^T) as X^T tiles (m = j, n = i): the sixteen tiles of the chunk, two
+    // per wave, no branch around the products (the element mask j <= i zeroes what lies above
+    // the diagonal; a product under a wave-uniform branch whose result is read right after the
+    // join has been seen to be read too early)
+    auto p_tiles = [&](const Stage& st) __attribute__((always_inline)) {
+#pragma unroll
+        for (int s_ = 0; s_ < 2; ++s_) {
+            const int it = w >> 1, jt = 2 * (w & 1) + s_;
+            const int i = 16 * it + row;
+            const float gzi = st.gzs[i];
+            f4 xt = f4_zero();
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs)
+                xt = mfma32(row8(st.Vs, LDV, 16 * jt + row, cs * 32, G), row8(st.Gs, LDV, i, cs * 32, G), xt);
+            h4 pv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int j = 16 * jt + 4 * G + e;
+                pv[e] = (j <= i) ? (half_t)(xt[e] + gzi) : (half_t)0.f;
+            }
+            *reinterpret_cast<h4*>(Ps + i * LDA + 16 * jt + 4 * G) = pv;
+        }
+    };
+
+    const int n_chunks = (T + C - 1) / C;
+    prefetch(s0, n_chunks - 1);
+    prefetch(s1, max(n_chunks - 2, 0));
+
+    if (dq_group) {
+        f4 NS[NCT], nz;
+        {
+            const float* sp = final_s + ((int64_t)n * KD + koff + kl + row) * DH + 4 * G;
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct) {
+                const f4 x = *reinterpret_cast<const f4*>(sp + 16 * ct);
+                NS[ct][0] = -x[0]; NS[ct][1] = -x[1]; NS[ct][2] = -x[2]; NS[ct][3] = -x[3];
+            }
+            const f4 x = *reinterpret_cast<const f4*>(final_z + (int64_t)n * KD + koff + kl + 4 * G);
+            nz[0] = -x[0]; nz[1] = -x[1]; nz[2] = -x[2]; nz[3] = -x[3];
+        }
+        const h8 ones = h8_ones();
+        // RAGGED: the chunk may have fewer than 64 steps (only the last chunk of the sequence, the
+        // first one worked on); full chunks store unconditionally
+        auto chunk_body = [&](auto ragged_tag, int ci, RowSet& r, int c_next) __attribute__((always_inline)) {
+            constexpr bool RAGGED = decltype(ragged_tag)::value;
+            const int t0 = ci * C;
+            const Stage st = stage_of(ci);
+            stage_in(st, r, c_next);
+            p_tiles(st);
+            // the state one chunk back: -S_prev = -S + K^T V, -z_prev = -z + K^T 1
+            h8 kf[2];        // K column fragments: K[j = 32js + 8G + e][k = kl + i]
+#pragma unroll
+            for (int js = 0; js < 2; ++js) kf[js] = col8(st.Ks, LDK, js * 32, kl, lane);
+#pragma unroll
+            for (int js = 0; js < 2; ++js) {
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct)
+                    NS[ct] = mfma32(col8(st.Vs, LDV, js * 32, 16 * ct, lane), kf[js], NS[ct]);
+                nz = mfma32(kf[js], ones, nz);
+            }
+            RFA_TICK(TB + 4);
+            __syncthreads();
+            RFA_TICK(TB + 5);
+            // dQ^T tiles (m = k, n = i)
+            f4 yt[4];       // -(S_prev G^T)
+#pragma unroll
+            for (int it = 0; it < 4; ++it) yt[it] = f4_zero();
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 bg[4];
+#pragma unroll
+                for (int it = 0; it < 4; ++it) bg[it] = row_split8(st.Gs, LDV, 16 * it + row, cs * 32, G);
+                __builtin_amdgcn_sched_barrier(0);
+                h8 hi, lo;
+                acc_to_operand(NS[2 * cs], NS[2 * cs + 1], hi, lo);
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    yt[it] = mfma32(hi, bg[it], yt[it]);
+                    yt[it] = mfma32(lo, bg[it], yt[it]);
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int i = 16 * it + row;
+                const float gzi = st.gzs[i];
+                f4 acc;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] = -(yt[it][e] + gzi * nz[e]);
+                acc = mfma32(kf[0], row8(Ps, LDA, i, 0, G), acc);
+                if (it >= 2) acc = mfma32(kf[1], row8(Ps, LDA, i, 32, G), acc);
+                if (!RAGGED || t0 + i < T)
+                    *reinterpret_cast<h4*>(dqb + (int64_t)(t0 + i) * k_stride + kl + 4 * G) = to_h4(acc);
+            }
+            RFA_TICK(TB + 6);
+            // no barrier here: the next chunk goes to the other stage, whose last readers passed the
+            // first barrier of this chunk; P is rewritten after the first barrier of the next one
+        };
+        chunk_body(std::true_type{}, n_chunks - 1, s0, max(n_chunks - 3, 0));
+        for (int ci = n_chunks - 2; ci >= 0; ci -= 2) {
+            chunk_body(std::false_type{}, ci, s1, max(ci - 2, 0));
+            if (ci - 1 < 0) break;
+            chunk_body(std::false_type{}, ci - 1, s0, max(ci - 3, 0));
+        }
+    } else {
+        f4 RT[NCT], racc = f4_zero();
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct) RT[ct] = f4_zero();
+        auto chunk_body = [&](auto ragged_tag, int ci, RowSet& r, int c_next) __attribute__((always_inline)) {
+            constexpr bool RAGGED = decltype(ragged_tag)::value;
+            const int t0 = ci * C;
+            const Stage st = stage_of(ci);
+            stage_in(st, r, c_next);
+            p_tiles(st);
+            RFA_TICK(TB + 4);
+            __syncthreads();
+            RFA_TICK(TB + 5);
+            // dK^T tiles (m = k, n = j), then R += G^T Q, r += Q^T gz
+            h8 qf[2];    // Q column fragments: Q[i = 32is + 8G + e][k = kl + lane i]
+#pragma unroll
+            for (int is = 0; is < 2; ++is) qf[is] = col8(st.Qs, LDK, is * 32, kl, lane);
+            f4 dkacc[4];
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                f4 acc = racc;
+                if (jt < 2) acc = mfma32(qf[0], col8(Ps, LDA, 0, 16 * jt, lane), acc);
+                acc = mfma32(qf[1], col8(Ps, LDA, 32, 16 * jt, lane), acc);
+                dkacc[jt] = acc;
+            }
+#pragma unroll
+            for (int cs = 0; cs < DH / 32; ++cs) {
+                h8 bvv[4];
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) bvv[jt] = row_split8(st.Vs, LDV, 16 * jt + row, cs * 32, G);
+                __builtin_amdgcn_sched_barrier(0);
+                h8 hi, lo;
+                acc_to_operand(RT[2 * cs], RT[2 * cs + 1], hi, lo);
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    dkacc[jt] = mfma32(hi, bvv[jt], dkacc[jt]);
+                    dkacc[jt] = mfma32(lo, bvv[jt], dkacc[jt]);
+                }
+            }
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                const int jj = 16 * jt + row;
+                if (!RAGGED || t0 + jj < T)
+                    *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + kl + 4 * G) = to_h4(dkacc[jt]);
+            }
+#pragma unroll
+            for (int is = 0; is < 2; ++is) {
+                h8 ghi, glo;
+                f8_to_operand(*reinterpret_cast<const f4*>(st.gzs + is * 32 + 8 * G),
+                              *reinterpret_cast<const f4*>(st.gzs + is * 32 + 8 * G + 4), ghi, glo);
+                racc = mfma32(qf[is], ghi, racc);
+                racc = mfma32(qf[is], glo, racc);
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct)
+                    RT[ct] = mfma32(col8(st.Gs, LDV, is * 32, 16 * ct, lane), qf[is], RT[ct]);
+            }
+            RFA_TICK(TB + 7);
+        };
+        chunk_body(std::true_type{}, n_chunks - 1, s0, max(n_chunks - 3, 0));
+        for (int ci = n_chunks - 2; ci >= 0; ci -= 2) {
+            chunk_body(std::false_type{}, ci, s1, max(ci - 2, 0));
+            if (ci - 1 < 0) break;
+            chunk_body(std::false_type{}, ci - 1, s0, max(ci - 3, 0));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// dV for value columns [coff, coff + 64) of one sequence.  8 waves, two per SIMD: wave (jh, wc)
+// owns columns cw = coff + 16 wc .. + 15 and produces the dV rows of the 16-step tiles 2jh, 2jh + 1
+// of every chunk; RR[kt] = R tile (k = 16kt + 4G + e, c = cw + i), all KD feature rows, is kept by
+// both waves of a column tile (the same updates in the same order: identical bits).
+// ---------------------------------------------------------------------------
+template <int KD, int DH>
+__device__ __forceinline__ void sliced_bwd_dv(
+    unsigned char* smem, int n, int coff, const half_t* __restrict__ q, const half_t* __restrict__ k,
+    const half_t* __restrict__ g, const float* __restrict__ den_raw, half_t* __restrict__ dv, int T, int N) {
+    using Cfg = SlicedBwdCfg<KD, DH>;
+    constexpr int NT = kSlicedThreads, C = Cfg::C, CSL = Cfg::CSL;
+    constexpr int LDQ = Cfg::LDQ, LDG = Cfg::LDS_, LDA = Cfg::LDA;
+    constexpr int NKT = KD / 16;
+    constexpr int PPR = CSL / 8, VP = ChunkRegs<CSL, NT>::kPieces;
+    half_t* ATs = reinterpret_cast<half_t*>(smem + 2 * Cfg::kStageB);    // AT[j][i] = A[i][j]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row = lane & 15, G = lane >> 4;
+    const int wc = w & 3, jh = w >> 2;
+    const int cl = 16 * wc;                     // first column of this wave, local to the slice array
+    const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
+    const half_t* qb = q + (int64_t)n * KD;
+    const half_t* kb = k + (int64_t)n * KD;
+    const half_t* gb = g + (int64_t)n * DH + coff;
+    half_t* dvb = dv + (int64_t)n * DH + coff;
+    RFA_TICK_INIT();
+    constexpr int TB = 10;
+
+    f4 RR[NKT];
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt) RR[kt] = f4_zero();
+
+    struct RowSet {
+        ChunkRegs<KD, NT> rq, rk;
+        ChunkRegs<CSL, NT> rg;
+        float den[VP];
+    };
+    RowSet s0, s1;
+    auto prefetch = [&](RowSet& r, int c) __attribute__((always_inline)) {
+        const int t0 = c * C, rows = T - t0;
+        chunk_g2r<KD, NT>(r.rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<KD, NT>(r.rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+        chunk_g2r<CSL, NT>(r.rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+#pragma unroll
+        for (int it = 0; it < VP; ++it) {
+            const int r_ = min((tid + NT * it) / PPR, r.rg.rows - 1);
+            r.den[it] = den_raw[(int64_t)(t0 + r_) * N + n];
+        }
+    };
+
+    auto chunk_body = [&](auto ragged_tag, int ci, RowSet& r, int c_next) __attribute__((always_inline)) {
+        constexpr bool RAGGED = decltype(ragged_tag)::value;
+        const int t0 = ci * C;
+        unsigned char* stage = smem + (ci & 1) * Cfg::kStageB;
+        half_t* Qs = reinterpret_cast<half_t*>(stage);
+        half_t* Ks = Qs + C * LDQ;
+        half_t* Gs = Ks + C * LDQ;               // G / den, this slice's columns
+
+        chunk_r2s<KD, NT>(r.rk, Ks, LDQ, tid);
+        chunk_r2s<KD, NT>(r.rq, Qs, LDQ, tid);
+        float inv_den[VP];
+#pragma unroll
+        for (int it = 0; it < VP; ++it) inv_den[it] = 1.0f / fmaxf(r.den[it], 1.0f);
+        chunk_r2s_scaled<CSL, NT>(r.rg, inv_den, Gs, LDG, tid);
+        RFA_TICK(TB + 1);
+        __syncthreads();
+        RFA_TICK(TB + 2);
+        prefetch(r, c_next);
+        RFA_TICK(TB + 3);
+
+        // ---- A = tril(Q K^T) tiles (m = i, n = j), stored transposed: the sixteen tiles of the
+        // chunk, two per wave, no branch around the products (see p_tiles of the dQ/dK role)
+#pragma unroll
+        for (int s_ = 0; s_ < 2; ++s_) {
+            const int it = w >> 1, jt = 2 * (w & 1) + s_;
+            const int j = 16 * jt + row;
+            f4 a_ = f4_zero();
+#pragma unroll
+            for (int ks = 0; ks < KD / 32; ++ks)
+                a_ = mfma32(row8(Qs, LDQ, 16 * it + row, ks * 32, G), row8(Ks, LDQ, j, ks * 32, G), a_);
+            h4 av;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int i = 16 * it + 4 * G + e;
+                av[e] = (i >= j) ? (half_t)a_[e] : (half_t)0.f;
+            }
+            *reinterpret_cast<h4*>(ATs + j * LDA + 16 * it + 4 * G) = av;
+        }
+        RFA_TICK(TB + 4);
+        __syncthreads();
+        RFA_TICK(TB + 5);
+
+        // ---- dV^T tiles (m = c, n = j) for j tiles 2jh, 2jh + 1, then R += Q^T G^
+        {
+            h8 gf[2];     // G^ column fragments: G^[i = 32is + 8G + e][c = cl + lane i]
+#pragma unroll
+            for (int is = 0; is < 2; ++is) gf[is] = col8(Gs, LDG, is * 32, cl, lane);
+            f4 dvacc[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int jr = 16 * (2 * jh + u) + row;
+                // rows i < 32 of A^T only reach the first two j tiles: their operand is all zero for
+                // the other half, and multiplying by zeros keeps the two halves on one code path
+                f4 acc = mfma32(gf[0], row8(ATs, LDA, jr, 0, G), f4_zero());
+                acc = mfma32(gf[1], row8(ATs, LDA, jr, 32, G), acc);
+                dvacc[u] = acc;
+            }
+#pragma unroll
+            for (int ks = 0; ks < KD / 32; ++ks) {
+                h8 bkk[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) bkk[u] = row_split8(Ks, LDQ, 16 * (2 * jh + u) + row, ks * 32, G);
+                __builtin_amdgcn_sched_barrier(0);
+                h8 hi, lo;
+                acc_to_operand(RR[2 * ks], RR[2 * ks + 1], hi, lo);
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    dvacc[u] = mfma32(hi, bkk[u], dvacc[u]);
+                    dvacc[u] = mfma32(lo, bkk[u], dvacc[u]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int jj = 16 * (2 * jh + u) + row;
+                if (!RAGGED || t0 + jj < T)
+                    *reinterpret_cast<h4*>(dvb + (int64_t)(t0 + jj) * v_stride + cl + 4 * G) = to_h4(dvacc[u]);
+            }
+#pragma unroll
+            for (int is = 0; is < 2; ++is)
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt) RR[kt] = mfma32(col8(Qs, LDQ, is * 32, 16 * kt, lane), gf[is], RR[kt]);
+        }
+        RFA_TICK(TB + 7);
+    };
+
+    const int n_chunks = (T + C - 1) / C;
+    prefetch(s0, n_chunks - 1);
+    prefetch(s1, max(n_chunks - 2, 0));
+    RFA_TICK(TB + 0);
+    chunk_body(std::true_type{}, n_chunks - 1, s0, max(n_chunks - 3, 0));
+    for (int ci = n_chunks - 2; ci >= 0; ci -= 2) {
+        chunk_body(std::false_type{}, ci, s1, max(ci - 2, 0));
+        if (ci - 1 < 0) break;
+        chunk_body(std::false_type{}, ci - 1, s0, max(ci - 3, 0));
+    }
+}
+
+// grid = kXcds * ceil(N / kXcds) * (NA + NB); kSlicedThreads threads.  hdr_in / plan: see plan_matches.
+template <int KD, int DH>
+__global__ __launch_bounds__(kSlicedThreads) void k_sliced_bwd(
+    const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
+    const half_t* __restrict__ g, const half_t* __restrict__ o, const float* __restrict__ den_raw,
+    const float* __restrict__ final_s, const float* __restrict__ final_z, half_t* __restrict__ dq,
+    half_t* __restrict__ dk, half_t* __restrict__ dv, int T, int N, const int* __restrict__ hdr_in, PlanWords plan) {
+    using Cfg = SlicedBwdCfg<KD, DH>;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    int n, role;
+    seq_role_of_block(blockIdx.x, Cfg::NA + Cfg::NB, n, role);
+    if (n >= N) return;
+    if (!plan_matches(hdr_in, plan)) {
+        if (role < Cfg::NA) {
+            poison_rows<kSliceWidth>(dq + (int64_t)n * KD + role * kSliceWidth, (int64_t)N * KD, 0, T);
+            poison_rows<kSliceWidth>(dk + (int64_t)n * KD + role * kSliceWidth, (int64_t)N * KD, 0, T);
+        } else {
+            poison_rows<kSliceWidth>(dv + (int64_t)n * DH + (role - Cfg::NA) * kSliceWidth, (int64_t)N * DH, 0, T);
+        }
+        return;
+    }
+    if (role < Cfg::NA)
+        sliced_bwd_dqdk<KD, DH>(smem_raw, n, role * kSliceWidth, q, k, v, g, o, den_raw, dq, dk, final_s, final_z, T, N);
+    else
+        sliced_bwd_dv<KD, DH>(smem_raw, n, (role - Cfg::NA) * kSliceWidth, q, k, g, den_raw, dv, T, N);
+}
+
+}  // namespace rfa

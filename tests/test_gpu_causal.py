@@ -282,3 +282,53 @@ def test_saved_buffer_carries_the_plan_of_its_forward(knobs):
     with pytest.raises(_lib.RfaHipError, match="another shape"):
         rfa_hip.backward_saved(pq[:640].contiguous(), pk[:640].contiguous(), v[:640].contiguous(), g[:640].contiguous(),
                                out[:640].contiguous(), saved)
+
+
+SLICED_SHAPES = [
+    # T, B, H, d, D: every (K, d) the sliced backward exists for, ragged tails, one step, sequence
+    # counts that are no multiple of the 8 XCDs, a long sequence (many backward steps of the state)
+    (128, 2, 4, 64, 64),
+    (1, 1, 1, 64, 64),
+    (63, 1, 2, 64, 64),
+    (65, 3, 1, 64, 64),
+    (200, 1, 3, 64, 64),
+    (640, 1, 11, 64, 64),
+    (192, 1, 2, 64, 32),     # K = 64: one feature slice
+    (160, 1, 2, 128, 64),    # d = 128, K = 128: two value slices
+    (330, 1, 3, 128, 32),    # d = 128, K = 64
+    (70, 65, 8, 64, 64),     # N = 520
+    (4100, 1, 2, 64, 64),    # 65 chunks
+]
+
+
+@pytest.mark.parametrize("T,B,H,d,D", SLICED_SHAPES)
+def test_sliced_backward_matches_oracle(T, B, H, d, D, knobs):
+    """The "sliced" knob makes the saving forward leave its final state and the backward walk whole
+    sequences backwards in state slices (one launch, every chunk read once).  Same tolerances as the
+    segment sweeps; dv does not depend on the stepped-back state and agrees with the segment
+    backward to fp16 rounding of G / den."""
+    from rfa_amd import _lib, rfa_hip
+    cpu = _features(T, B, H, d, D, seed=8000 + T)
+    pq, pk, v, g = (t.cuda() for t in cpu)
+    print(f"causal sliced backward T={T} N={B*H} K={2*D} d={d}", flush=True)
+    knobs(sliced=0)
+    out0, saved0 = rfa_hip.forward_save(pq, pk, v)
+    seg = rfa_hip.backward_saved(pq, pk, v, g, out0, saved0)
+    knobs(sliced=1)
+    out, saved = rfa_hip.forward_save(pq, pk, v)
+    assert torch.equal(out, out0)
+    import ctypes
+    words = (ctypes.c_int32 * 16)()
+    _lib.check(_lib.load().rfa_causal_saved_describe(saved.data_ptr(), words, None))
+    assert words[2] == 1                                    # the final-state layout
+    assert _lib.load().rfa_causal_backward_saved_workspace_bytes(saved.data_ptr(), T, B * H, 2 * D, d) == 0
+    got = rfa_hip.backward_saved(pq, pk, v, g, out, saved)
+    want = _oracle_bwd(*cpu)
+    for name, a, b in zip(("dq", "dk", "dv"), got, want):
+        assert torch.isfinite(a.float()).all(), name
+        assert _rel(a.float().cpu(), b) <= GRAD_RTOL, (name, _rel(a.float().cpu(), b))
+    assert _rel(got[2].float(), seg[2].float()) <= 2e-3
+    # deterministic, and the knob may move between forward and backward
+    knobs(sliced=0)
+    again = rfa_hip.backward_saved(pq, pk, v, g, out, saved)
+    assert all(torch.equal(a, b) for a, b in zip(got, again))

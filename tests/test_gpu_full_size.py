@@ -188,23 +188,31 @@ def test_element_offsets_beyond_32_bits(nseg, knobs):
     grads = rfa_hip.backward(pq, pk, v, g)
     for nm, big, ref in zip(("dq", "dk", "dv"), grads, rfa_hip.backward(sq, sk, sv, sg)):
         assert torch.equal(big[:, idx], ref), nm
-    # the saving pair (what RFA.apply runs)
+    # the saving pair (what RFA.apply runs), with either backward: the two segment sweeps and the
+    # one sweep in state slices (the small call must take the same one to agree bit for bit)
     from rfa_amd.rfa import RFA
-    lq, lk, lv = (t.detach().requires_grad_(True) for t in (pq, pk, v))
-    o2 = RFA.apply(lq, lk, lv)
-    o2.backward(g)
-    mq, mk, mv = (t.detach().requires_grad_(True) for t in (sq, sk, sv))
-    o3 = RFA.apply(mq, mk, mv)
-    o3.backward(sg)
-    assert torch.equal(o2.detach()[:, idx], o3.detach())
-    for nm, big, ref in (("dq", lq.grad, mq.grad), ("dk", lk.grad, mk.grad), ("dv", lv.grad, mv.grad)):
-        assert torch.equal(big[:, idx], ref), nm
+    for sliced in (0, 1):
+        knobs(sliced=sliced)
+        lq, lk, lv = (t.detach().requires_grad_(True) for t in (pq, pk, v))
+        o2 = RFA.apply(lq, lk, lv)
+        o2.backward(g)
+        mq, mk, mv = (t.detach().requires_grad_(True) for t in (sq, sk, sv))
+        o3 = RFA.apply(mq, mk, mv)
+        o3.backward(sg)
+        assert torch.equal(o2.detach()[:, idx], o3.detach())
+        for nm, big, ref in (("dq", lq.grad, mq.grad), ("dk", lk.grad, mk.grad), ("dv", lv.grad, mv.grad)):
+            assert torch.equal(big[:, idx], ref), (sliced, nm)
+        if sliced:      # oracle on the last sequence for the sliced backward too
+            cq, ck, cv, cg = (t[:, N - 1:].float().cpu() for t in (pq, pk, v, g))
+            for nm, got, want in zip(("dq", "dk", "dv"), (lq.grad, lk.grad, lv.grad), O.causal_backward_chunked(cq, ck, cv, cg)):
+                assert _rel(got[:, N - 1:].float().cpu(), want) <= 1e-2, nm
+        del o2, o3, lq, lk, lv, mq, mk, mv
     # oracle on the last sequence
     cq, ck, cv, cg = (t[:, N - 1:].float().cpu() for t in (pq, pk, v, g))
     assert (out[:, N - 1:].float().cpu() - O.causal_forward_chunked(cq, ck, cv)).abs().max().item() <= 2e-3
     for nm, got, want in zip(("dq", "dk", "dv"), grads, O.causal_backward_chunked(cq, ck, cv, cg)):
         assert _rel(got[:, N - 1:].float().cpu(), want) <= 1e-2, nm
-    del grads, o2, o3, lq, lk, lv
+    del grads
 
     # cross attention over the same tensors (source = target length here)
     s, z = rfa_hip.cross_state(pk.view(T, B, H, K), v.view(T, B, H, d))
