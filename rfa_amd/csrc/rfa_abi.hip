@@ -165,7 +165,7 @@ struct ScanPlan {
 //                    in state slices (rfa_sliced.h), one launch, every chunk read once
 enum SavedLayout { LAYOUT_SEGMENTS = 0, LAYOUT_FINAL = 1 };
 
-bool sliced_supported(int K, int d) { return (K == 64 || K == 128) && (d == 64 || d == 128); }
+bool sliced_supported(int K, int d) { return (K == 64 || K == 128) && d == 64; }
 
 // The sliced backward has N * (K / 64 + d / 64) workgroups that never wait for each other: taken
 // when they cover most of the compute units ("sliced" knob: 0 never, 1 whenever a kernel exists).
@@ -458,7 +458,7 @@ int launch_sliced_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa
                            const rfa::half_t* out, rfa::half_t* dq, rfa::half_t* dk, rfa::half_t* dv, int T, int N,
                            const ScanPlan& pf, const int* savedHdr, const float* finalS, const float* finalZ,
                            const float* savedDen, hipStream_t st) {
-    if constexpr (KD <= 128) {
+    if constexpr (KD <= 128 && DH == 64) {
         using Cfg = rfa::SlicedBwdCfg<KD, DH>;
         auto kern = rfa::k_sliced_bwd<KD, DH>;
         if (int rc = set_lds(kern, Cfg::kLds)) return rc;

@@ -1,15 +1,15 @@
-// Causal random-feature attention without time segments (gfx950): parallelism from slices of
-// the state instead of from cutting the sequence.
+// Causal random-feature attention backward without time segments (gfx950): parallelism from
+// slices of the state instead of from cutting the sequence.
 //
 // The chunked scan of rfa_causal.h cuts a sequence into time segments so that bsz * heads
 // sequences fill the GPU; every segment then needs the state at its first step, which costs a
-// pass over k, v (forward) and over q, g (backward) for the segment totals, and two sweeps over
-// the sequence in the backward (dQ needs the sum over earlier steps, dK and dV the sum over later
-// ones).  Here a workgroup walks a whole sequence and owns a slice of the state:
+// pass over q, g for the segment totals, and two sweeps over the sequence (dQ needs the sum over
+// earlier steps, dK and dV the sum over later ones).  Here a workgroup walks a whole sequence
+// and owns a slice of the state:
 //
-//   backward, feature slice  [koff, koff + 64) of phi:   dQ[:, slice], dK[:, slice]
+//   feature slice  [koff, koff + 64) of phi:   dQ[:, slice], dK[:, slice]
 //       carries S[slice, :] and R[slice, :]   (reads g, out, v whole; q, k slice)
-//   backward, value slice    [coff, coff + 64) of v:      dV[:, slice]
+//   value slice    [coff, coff + 64) of v:      dV[:, slice]
 //       carries R[:, slice]                    (reads q, k whole; g slice)
 //
 // with  S = sum_{s <= t} phi_k[s] (x) v[s],  R = sum_{s > t} phi_q[s] (x) g^[s],  g^ = g / den
@@ -25,6 +25,13 @@
 //     dQ = P K + G^ S_prev^T + gz z_prev^T     (S_prev, z_prev: state before the chunk)
 //     dK = P^T Q + V R_next^T + 1 r_next^T     (R_next, r_next: sums over later chunks)
 //     dV = A^T G^ + K R_next
+//
+// A workgroup is a pipeline of 12 waves, three per SIMD.  Waves 0-3 (loader group) bring chunk c
+// from HBM into LDS and form its masked tile matrix (P or A^T); waves 4-7 and 8-11 work on chunk
+// c + 1 (the one staged an iteration earlier): dQ and dK in the feature-slice role, the two
+// halves of the dV rows in the value-slice role.  The groups meet at two workgroup barriers per
+// chunk; the chunk arrays and the tile matrix are double buffered.  Only the loader group issues
+// loads and only the others issue stores, so neither kind waits for the other.
 #pragma once
 #include <type_traits>
 
@@ -32,8 +39,9 @@
 
 namespace rfa {
 
-constexpr int kSliceWidth = 64;    // features (dQ/dK role) or value columns (dV role) per workgroup
-constexpr int kSlicedThreads = 512; // 8 waves, two per SIMD
+constexpr int kSliceWidth = 64;     // features (dQ/dK role) or value columns (dV role) per workgroup
+constexpr int kSlicedThreads = 768; // 12 waves: loader group + two product groups
+constexpr int kGroupThreads = 256;  // threads per group
 
 // Workgroup index -> (sequence, role).  The wps workgroups of a sequence get indices that are
 // equal mod kXcds, i.e. the same XCD, and consecutive positions there.
@@ -52,24 +60,47 @@ struct SlicedBwdCfg {
     static constexpr int LDQ = KD + lds_pad(KD);
     static constexpr int LDV = DH + lds_pad(DH);
     static constexpr int LDA = C + 8;
-    // dQ/dK role: two stages of [Q slice | K slice | V | G^ | gz], one P
-    static constexpr size_t kStageA = (size_t)(2 * C * LDS_ + 2 * C * LDV) * 2 + C * 4;
-    static constexpr size_t kLdsA = 2 * kStageA + (size_t)C * LDA * 2;
-    // dV role: two stages of [Q | K | G^ slice], one A^T
-    static constexpr size_t kStageB = (size_t)(2 * C * LDQ + C * LDS_) * 2;
-    static constexpr size_t kLdsB = 2 * kStageB + (size_t)C * LDA * 2;
-    static constexpr size_t kLds = kLdsA > kLdsB ? kLdsA : kLdsB;
+    // dQ/dK role, per stage: Q slice | K slice | V | G^ | P | gz
+    static constexpr size_t kStageA = (size_t)(2 * C * LDS_ + 2 * C * LDV + C * LDA) * 2 + C * 4;
+    // dV role, per stage: Q | K | G^ slice | A^T
+    static constexpr size_t kStageB = (size_t)(2 * C * LDQ + C * LDS_ + C * LDA) * 2;
+    static constexpr size_t kLds = 2 * (kStageA > kStageB ? kStageA : kStageB);
     static_assert(kStageA % 16 == 0 && kStageB % 16 == 0, "stage alignment");
 };
 
+__device__ __forceinline__ void wg_sync() { __syncthreads(); }
+
+// 64 rows x F halves of a full chunk: thread-private row pointers (set up once) plus the
+// chunk's offset; no clamping, no address arithmetic beyond one 64-bit add per piece
+template <int F>
+struct RowPtrs {
+    static constexpr int kPieces = ChunkRegs<F, kGroupThreads>::kPieces;
+    const half_t* p[kPieces];
+    __device__ __forceinline__ void init(const half_t* base, int64_t row_stride, int tid) {
+        constexpr int PPR = F / 8;
+#pragma unroll
+        for (int it = 0; it < kPieces; ++it) {
+            const int pc = tid + kGroupThreads * it;
+            p[it] = base + (int64_t)(pc / PPR) * row_stride + (pc % PPR) * 8;
+        }
+    }
+    __device__ __forceinline__ void load_full(ChunkRegs<F, kGroupThreads>& r, int64_t chunk_off) const {
+        r.rows = kChunk;
+#pragma unroll
+        for (int it = 0; it < kPieces; ++it) {
+            r.v[it] = *reinterpret_cast<const uint4*>(p[it] + chunk_off);
+            r.drop[it] = 0;
+        }
+    }
+};
+
 // ---------------------------------------------------------------------------
-// dQ, dK for features [koff, koff + 64) of one sequence.  8 waves, two per SIMD, in two groups
-// that share the chunk arrays and the P tiles and otherwise run their own loop (same number of
-// barriers):  waves 0-3 carry -S^T and -z and produce dQ, waves 4-7 carry R^T and r and produce
-// dK.  Wave (group, wf) owns features kw = koff + 16 wf .. + 15:
-//   NS[ct] = -S^T tile (c = 16ct + 4G + e, k = kw + i),  RT[ct] = R^T tile,  nz = -z and r as
-//   tiles (k = kw + 4G + e).  S and z are carried negated so that the MFMA can step them
-//   backwards by adding K^T V.
+// dQ, dK for features [koff, koff + 64) of one sequence.
+//   loader group: stages Q, K slices, V, G^ = G / den and gz, then P = tril(G^ V^T + gz 1^T)
+//   dQ group: wave wf owns features kw = koff + 16 wf .. + 15; NS[ct] = -S^T tile
+//             (c = 16ct + 4G + e, k = kw + i), nz = -z tile (k = kw + 4G + e).  S and z are
+//             carried negated so that the MFMA can step them backwards by adding K^T V.
+//   dK group: same features; RT[ct] = R^T tile, r as a tile.
 // ---------------------------------------------------------------------------
 template <int KD, int DH>
 __device__ __forceinline__ void sliced_bwd_dqdk(
@@ -78,126 +109,166 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
     const float* __restrict__ den_raw, half_t* __restrict__ dq, half_t* __restrict__ dk,
     const float* __restrict__ final_s, const float* __restrict__ final_z, int T, int N) {
     using Cfg = SlicedBwdCfg<KD, DH>;
-    constexpr int NT = kSlicedThreads, C = Cfg::C, KSL = Cfg::KSL;
+    constexpr int NT = kGroupThreads, C = Cfg::C, KSL = Cfg::KSL;
     constexpr int LDK = Cfg::LDS_, LDV = Cfg::LDV, LDA = Cfg::LDA;
     constexpr int NCT = DH / 16;
     constexpr int PPR = DH / 8, VP = ChunkRegs<DH, NT>::kPieces;
-    half_t* Ps = reinterpret_cast<half_t*>(smem + 2 * Cfg::kStageA);
+    constexpr size_t kStage = Cfg::kLds / 2;
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int grp = w >> 2, wf = w & 3;
+    const int tid = threadIdx.x & (NT - 1);     // thread inside its group
     const int row = lane & 15, G = lane >> 4;
-    const int wf = w & 3;
-    const bool dq_group = w < 4;
     const int kl = 16 * wf;                     // first feature of this wave, local to the slice arrays
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
-    const half_t* qb = q + (int64_t)n * KD + koff;
-    const half_t* kb = k + (int64_t)n * KD + koff;
-    const half_t* vb = v + (int64_t)n * DH;
-    const half_t* gb = g + (int64_t)n * DH;
-    const half_t* ob = o + (int64_t)n * DH;
-    half_t* dqb = dq + (int64_t)n * KD + koff;
-    half_t* dkb = dk + (int64_t)n * KD + koff;
+    const int n_chunks = (T + C - 1) / C;
     RFA_TICK_INIT();
-    constexpr int TB = 0;
 
-    // Two register sets of chunk rows: while chunk c is worked on, the rows of chunks c - 1 and
-    // c - 2 are on their way, so a load has two chunk periods to arrive.
-    struct RowSet {
-        ChunkRegs<KSL, NT> rq, rk;
-        ChunkRegs<DH, NT> rv, rg, ro;
-        float dn[VP];
-    };
-    RowSet s0, s1;
-    // branch-free: c may be a chunk that is never used (clamped by the caller to an existing one)
-    auto prefetch = [&](RowSet& r, int c) __attribute__((always_inline)) {
-        const int t0 = c * C, rows = T - t0;
-        chunk_g2r<KSL, NT>(r.rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
-        chunk_g2r<KSL, NT>(r.rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
-        chunk_g2r<DH, NT>(r.rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
-        chunk_g2r<DH, NT>(r.rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
-        chunk_g2r<DH, NT>(r.ro, ob + (int64_t)t0 * v_stride, v_stride, rows, tid);
-#pragma unroll
-        for (int it = 0; it < VP; ++it) {
-            const int r_ = min((tid + NT * it) / PPR, r.rg.rows - 1);
-            r.dn[it] = den_raw[(int64_t)(t0 + r_) * N + n];
-        }
-    };
-
-    struct Stage { half_t *Qs, *Ks, *Vs, *Gs; float* gzs; };
-    auto stage_of = [&](int ci) __attribute__((always_inline)) {
+    struct Stage { half_t *Qs, *Ks, *Vs, *Gs, *Ps; float* gzs; };
+    auto stage_of = [&](int i) __attribute__((always_inline)) {
         Stage st;
-        st.Qs = reinterpret_cast<half_t*>(smem + (ci & 1) * Cfg::kStageA);
+        st.Qs = reinterpret_cast<half_t*>(smem + (i & 1) * kStage);
         st.Ks = st.Qs + C * LDK;
         st.Vs = st.Ks + C * LDK;
         st.Gs = st.Vs + C * LDV;                 // G / den
-        st.gzs = reinterpret_cast<float*>(st.Gs + C * LDV);
+        st.Ps = st.Gs + C * LDV;
+        st.gzs = reinterpret_cast<float*>(st.Ps + C * LDA);
         return st;
     };
 
-    // rows in `r` -> LDS: Q, K slices, V, G^ = G / den, gz from g . out (the PPR lanes holding one
-    // row are adjacent); first barrier of the chunk; then chunk c_next is requested into `r`
-    auto stage_in = [&](const Stage& st, RowSet& r, int c_next) __attribute__((always_inline)) {
-        chunk_r2s<KSL, NT>(r.rq, st.Qs, LDK, tid);
-        chunk_r2s<KSL, NT>(r.rk, st.Ks, LDK, tid);
-        chunk_r2s<DH, NT>(r.rv, st.Vs, LDV, tid);
+    // Iteration i = 0 .. n_chunks: the loader group stages chunk n_chunks - 1 - i (none in the last
+    // iteration), the product groups work on chunk n_chunks - i (none in the first).  Every wave
+    // passes exactly two barriers per iteration.
+    if (grp == 0) {
+        const half_t* qb = q + (int64_t)n * KD + koff;
+        const half_t* kb = k + (int64_t)n * KD + koff;
+        const half_t* vb = v + (int64_t)n * DH;
+        const half_t* gb = g + (int64_t)n * DH;
+        const half_t* ob = o + (int64_t)n * DH;
+        RowPtrs<KSL> pq, pk;
+        RowPtrs<DH> pv, pg, po;
+        pq.init(qb, k_stride, tid);
+        pk.init(kb, k_stride, tid);
+        pv.init(vb, v_stride, tid);
+        pg.init(gb, v_stride, tid);
+        po.init(ob, v_stride, tid);
+        // Two register sets of chunk rows: while chunk c is staged, the rows of chunks c - 1 and
+        // c - 2 are on their way, so a load has two chunk periods to arrive.
+        struct RowSet {
+            ChunkRegs<KSL, NT> rq, rk;
+            ChunkRegs<DH, NT> rv, rg, ro;
+            float dn[VP];
+        };
+        RowSet s0, s1;
+        // the last chunk of the sequence may be short: clamped row addresses
+        auto prefetch_ragged = [&](RowSet& r, int c) __attribute__((always_inline)) {
+            const int t0 = c * C, rows = T - t0;
+            chunk_g2r<KSL, NT>(r.rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+            chunk_g2r<KSL, NT>(r.rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+            chunk_g2r<DH, NT>(r.rv, vb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+            chunk_g2r<DH, NT>(r.rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
+            chunk_g2r<DH, NT>(r.ro, ob + (int64_t)t0 * v_stride, v_stride, rows, tid);
 #pragma unroll
-        for (int it = 0; it < VP; ++it) {
-            const int pc = tid + NT * it;
-            const int r_ = pc / PPR, c8 = pc % PPR;
-            union { uint4 u; h8 h; } xg, xo;
-            xg.u = r.rg.v[it];
-            xo.u = r.ro.v[it];
-            float dot = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) dot += (float)xg.h[e] * (float)xo.h[e];
-#pragma unroll
-            for (int m = 1; m < PPR; m <<= 1) dot += __shfl_xor(dot, m, 64);
-            const bool valid = r_ < r.rg.rows;
-            const float inv = valid ? 1.0f / fmaxf(r.dn[it], 1.0f) : 0.f;
-            const float gzv = (valid && r.dn[it] > 1.0f) ? -dot * inv : 0.f;
-            h8 y;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)xg.h[e] * inv);
-            *reinterpret_cast<h8*>(st.Gs + r_ * LDV + c8 * 8) = y;
-            if (c8 == 0) st.gzs[r_] = gzv;
-        }
-        RFA_TICK(TB + 1);
-        __syncthreads();
-        RFA_TICK(TB + 2);
-        prefetch(r, c_next);
-        RFA_TICK(TB + 3);
-    };
-
-    // P = tril(G^ V^T + gz 1^T) as X^T tiles (m = j, n = i): the sixteen tiles of the chunk, two
-    // per wave, no branch around the products (the element mask j <= i zeroes what lies above
-    // the diagonal; a product under a wave-uniform branch whose result is read right after the
-    // join has been seen to be read too early)
-    auto p_tiles = [&](const Stage& st) __attribute__((always_inline)) {
-#pragma unroll
-        for (int s_ = 0; s_ < 2; ++s_) {
-            const int it = w >> 1, jt = 2 * (w & 1) + s_;
-            const int i = 16 * it + row;
-            const float gzi = st.gzs[i];
-            f4 xt = f4_zero();
-#pragma unroll
-            for (int cs = 0; cs < DH / 32; ++cs)
-                xt = mfma32(row8(st.Vs, LDV, 16 * jt + row, cs * 32, G), row8(st.Gs, LDV, i, cs * 32, G), xt);
-            h4 pv;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int j = 16 * jt + 4 * G + e;
-                pv[e] = (j <= i) ? (half_t)(xt[e] + gzi) : (half_t)0.f;
+            for (int it = 0; it < VP; ++it) {
+                const int r_ = min((tid + NT * it) / PPR, r.rg.rows - 1);
+                r.dn[it] = den_raw[(int64_t)(t0 + r_) * N + n];
             }
-            *reinterpret_cast<h4*>(Ps + i * LDA + 16 * jt + 4 * G) = pv;
+        };
+        // a full chunk; c may be a chunk that is never used (the caller clamps it to an existing
+        // one: no branch around the loads)
+        auto prefetch = [&](RowSet& r, int c) __attribute__((always_inline)) {
+            const int64_t t0 = (int64_t)c * C;
+            pq.load_full(r.rq, t0 * k_stride);
+            pk.load_full(r.rk, t0 * k_stride);
+            pv.load_full(r.rv, t0 * v_stride);
+            pg.load_full(r.rg, t0 * v_stride);
+            po.load_full(r.ro, t0 * v_stride);
+#pragma unroll
+            for (int it = 0; it < VP; ++it) r.dn[it] = den_raw[(t0 + (tid + NT * it) / PPR) * N + n];
+        };
+        // rows in `r` -> LDS: Q, K slices, V, G^ = G / den, gz from g . out (the PPR lanes holding
+        // one row are adjacent); barrier; chunk c_next requested into `r`; P tiles; barrier
+        auto stage_chunk = [&](int i, RowSet& r, int c_next, bool do_prefetch) __attribute__((always_inline)) {
+            const Stage st = stage_of(i);
+            chunk_r2s<KSL, NT>(r.rq, st.Qs, LDK, tid);
+            chunk_r2s<KSL, NT>(r.rk, st.Ks, LDK, tid);
+            chunk_r2s<DH, NT>(r.rv, st.Vs, LDV, tid);
+#pragma unroll
+            for (int it = 0; it < VP; ++it) {
+                const int pc = tid + NT * it;
+                const int r_ = pc / PPR, c8 = pc % PPR;
+                union { uint4 u; h8 h; } xg, xo;
+                xg.u = r.rg.v[it];
+                xo.u = r.ro.v[it];
+                float dot = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) dot += (float)xg.h[e] * (float)xo.h[e];
+#pragma unroll
+                for (int m = 1; m < PPR; m <<= 1) dot += __shfl_xor(dot, m, 64);
+                const bool valid = r_ < r.rg.rows;
+                const float inv = valid ? 1.0f / fmaxf(r.dn[it], 1.0f) : 0.f;
+                const float gzv = (valid && r.dn[it] > 1.0f) ? -dot * inv : 0.f;
+                h8 y;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)xg.h[e] * inv);
+                *reinterpret_cast<h8*>(st.Gs + r_ * LDV + c8 * 8) = y;
+                if (c8 == 0) st.gzs[r_] = gzv;
+            }
+            RFA_TICK_AT(1, 0);
+            wg_sync();
+            RFA_TICK_AT(2, 0);
+            if (do_prefetch) prefetch(r, c_next);
+            RFA_TICK_AT(3, 0);
+            // P = tril(G^ V^T + gz 1^T) as X^T tiles (m = j, n = i): row block wf, all four column
+            // tiles, no branch around the products (the element mask j <= i zeroes what lies above
+            // the diagonal; a product under a wave-uniform branch whose result is read right after
+            // the join has been seen to be read too early)
+            {
+                const int ii = 16 * wf + row;
+                const float gzi = st.gzs[ii];
+                f4 xt[4];
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) xt[jt] = f4_zero();
+#pragma unroll
+                for (int cs = 0; cs < DH / 32; ++cs) {
+                    const h8 bg = row8(st.Gs, LDV, ii, cs * 32, G);
+#pragma unroll
+                    for (int jt = 0; jt < 4; ++jt) xt[jt] = mfma32(row8(st.Vs, LDV, 16 * jt + row, cs * 32, G), bg, xt[jt]);
+                }
+#pragma unroll
+                for (int jt = 0; jt < 4; ++jt) {
+                    h4 pv_;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int j = 16 * jt + 4 * G + e;
+                        pv_[e] = (j <= ii) ? (half_t)(xt[jt][e] + gzi) : (half_t)0.f;
+                    }
+                    *reinterpret_cast<h4*>(st.Ps + ii * LDA + 16 * jt + 4 * G) = pv_;
+                }
+            }
+            RFA_TICK_AT(4, 0);
+            wg_sync();
+            RFA_TICK_AT(5, 0);
+        };
+
+        // With a single chunk nothing but that (possibly short) chunk may be read.  Otherwise
+        // every chunk but the last is full, and chunks past the start are requested again as
+        // chunk 0 (never used) rather than under a branch.
+        const bool multi = n_chunks > 1;
+        prefetch_ragged(s0, n_chunks - 1);
+        if (multi) prefetch(s1, n_chunks - 2);
+        // i = 0 stages the last chunk from s0
+        stage_chunk(0, s0, max(n_chunks - 3, 0), multi);
+        for (int i = 1; i < n_chunks; i += 2) {
+            stage_chunk(i, s1, max(n_chunks - 3 - i, 0), true);
+            if (i + 1 >= n_chunks) break;
+            stage_chunk(i + 1, s0, max(n_chunks - 4 - i, 0), true);
         }
-    };
-
-    const int n_chunks = (T + C - 1) / C;
-    prefetch(s0, n_chunks - 1);
-    prefetch(s1, max(n_chunks - 2, 0));
-
-    if (dq_group) {
+        wg_sync();      // the last iteration: the product groups finish chunk 0
+        wg_sync();
+    } else if (grp == 1) {
+        half_t* dqb = dq + (int64_t)n * KD + koff;
         f4 NS[NCT], nz;
         {
             const float* sp = final_s + ((int64_t)n * KD + koff + kl + row) * DH + 4 * G;
@@ -212,12 +283,10 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
         const h8 ones = h8_ones();
         // RAGGED: the chunk may have fewer than 64 steps (only the last chunk of the sequence, the
         // first one worked on); full chunks store unconditionally
-        auto chunk_body = [&](auto ragged_tag, int ci, RowSet& r, int c_next) __attribute__((always_inline)) {
+        auto chunk_body = [&](auto ragged_tag, int i) __attribute__((always_inline)) {
             constexpr bool RAGGED = decltype(ragged_tag)::value;
-            const int t0 = ci * C;
-            const Stage st = stage_of(ci);
-            stage_in(st, r, c_next);
-            p_tiles(st);
+            const int t0 = (n_chunks - i) * C;
+            const Stage st = stage_of(i - 1);
             // the state one chunk back: -S_prev = -S + K^T V, -z_prev = -z + K^T 1
             h8 kf[2];        // K column fragments: K[j = 32js + 8G + e][k = kl + i]
 #pragma unroll
@@ -229,9 +298,6 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
                     NS[ct] = mfma32(col8(st.Vs, LDV, js * 32, 16 * ct, lane), kf[js], NS[ct]);
                 nz = mfma32(kf[js], ones, nz);
             }
-            RFA_TICK(TB + 4);
-            __syncthreads();
-            RFA_TICK(TB + 5);
             // dQ^T tiles (m = k, n = i)
             f4 yt[4];       // -(S_prev G^T)
 #pragma unroll
@@ -250,41 +316,38 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
                     yt[it] = mfma32(lo, bg[it], yt[it]);
                 }
             }
+            RFA_TICK_AT(11, 256);
+            wg_sync();
+            RFA_TICK_AT(12, 256);
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
-                const int i = 16 * it + row;
-                const float gzi = st.gzs[i];
+                const int ii = 16 * it + row;
+                const float gzi = st.gzs[ii];
                 f4 acc;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) acc[e] = -(yt[it][e] + gzi * nz[e]);
-                acc = mfma32(kf[0], row8(Ps, LDA, i, 0, G), acc);
-                if (it >= 2) acc = mfma32(kf[1], row8(Ps, LDA, i, 32, G), acc);
-                if (!RAGGED || t0 + i < T)
-                    *reinterpret_cast<h4*>(dqb + (int64_t)(t0 + i) * k_stride + kl + 4 * G) = to_h4(acc);
+                acc = mfma32(kf[0], row8(st.Ps, LDA, ii, 0, G), acc);
+                if (it >= 2) acc = mfma32(kf[1], row8(st.Ps, LDA, ii, 32, G), acc);
+                if (!RAGGED || t0 + ii < T)
+                    *reinterpret_cast<h4*>(dqb + (int64_t)(t0 + ii) * k_stride + kl + 4 * G) = to_h4(acc);
             }
-            RFA_TICK(TB + 6);
-            // no barrier here: the next chunk goes to the other stage, whose last readers passed the
-            // first barrier of this chunk; P is rewritten after the first barrier of the next one
+            RFA_TICK_AT(13, 256);
+            wg_sync();
+            RFA_TICK_AT(14, 256);
         };
-        chunk_body(std::true_type{}, n_chunks - 1, s0, max(n_chunks - 3, 0));
-        for (int ci = n_chunks - 2; ci >= 0; ci -= 2) {
-            chunk_body(std::false_type{}, ci, s1, max(ci - 2, 0));
-            if (ci - 1 < 0) break;
-            chunk_body(std::false_type{}, ci - 1, s0, max(ci - 3, 0));
-        }
+        wg_sync();      // the first iteration: the loader group stages the last chunk
+        wg_sync();
+        chunk_body(std::true_type{}, 1);
+        for (int i = 2; i <= n_chunks; ++i) chunk_body(std::false_type{}, i);
     } else {
+        half_t* dkb = dk + (int64_t)n * KD + koff;
         f4 RT[NCT], racc = f4_zero();
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct) RT[ct] = f4_zero();
-        auto chunk_body = [&](auto ragged_tag, int ci, RowSet& r, int c_next) __attribute__((always_inline)) {
+        auto chunk_body = [&](auto ragged_tag, int i) __attribute__((always_inline)) {
             constexpr bool RAGGED = decltype(ragged_tag)::value;
-            const int t0 = ci * C;
-            const Stage st = stage_of(ci);
-            stage_in(st, r, c_next);
-            p_tiles(st);
-            RFA_TICK(TB + 4);
-            __syncthreads();
-            RFA_TICK(TB + 5);
+            const int t0 = (n_chunks - i) * C;
+            const Stage st = stage_of(i - 1);
             // dK^T tiles (m = k, n = j), then R += G^T Q, r += Q^T gz
             h8 qf[2];    // Q column fragments: Q[i = 32is + 8G + e][k = kl + lane i]
 #pragma unroll
@@ -293,8 +356,8 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) {
                 f4 acc = racc;
-                if (jt < 2) acc = mfma32(qf[0], col8(Ps, LDA, 0, 16 * jt, lane), acc);
-                acc = mfma32(qf[1], col8(Ps, LDA, 32, 16 * jt, lane), acc);
+                if (jt < 2) acc = mfma32(qf[0], col8(st.Ps, LDA, 0, 16 * jt, lane), acc);
+                acc = mfma32(qf[1], col8(st.Ps, LDA, 32, 16 * jt, lane), acc);
                 dkacc[jt] = acc;
             }
 #pragma unroll
@@ -311,6 +374,7 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
                     dkacc[jt] = mfma32(lo, bvv[jt], dkacc[jt]);
                 }
             }
+            wg_sync();
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) {
                 const int jj = 16 * jt + row;
@@ -328,131 +392,170 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
                 for (int ct = 0; ct < NCT; ++ct)
                     RT[ct] = mfma32(col8(st.Gs, LDV, is * 32, 16 * ct, lane), qf[is], RT[ct]);
             }
-            RFA_TICK(TB + 7);
+            wg_sync();
         };
-        chunk_body(std::true_type{}, n_chunks - 1, s0, max(n_chunks - 3, 0));
-        for (int ci = n_chunks - 2; ci >= 0; ci -= 2) {
-            chunk_body(std::false_type{}, ci, s1, max(ci - 2, 0));
-            if (ci - 1 < 0) break;
-            chunk_body(std::false_type{}, ci - 1, s0, max(ci - 3, 0));
-        }
+        wg_sync();
+        wg_sync();
+        chunk_body(std::true_type{}, 1);
+        for (int i = 2; i <= n_chunks; ++i) chunk_body(std::false_type{}, i);
     }
 }
 
 // ---------------------------------------------------------------------------
-// dV for value columns [coff, coff + 64) of one sequence.  8 waves, two per SIMD: wave (jh, wc)
-// owns columns cw = coff + 16 wc .. + 15 and produces the dV rows of the 16-step tiles 2jh, 2jh + 1
-// of every chunk; RR[kt] = R tile (k = 16kt + 4G + e, c = cw + i), all KD feature rows, is kept by
-// both waves of a column tile (the same updates in the same order: identical bits).
+// dV for value columns [coff, coff + 64) of one sequence.
+//   loader group: stages Q, K (all KD features) and the G^ slice, then A^T = tril(Q K^T)^T
+//   dV groups jh = 0, 1: wave (jh, wc) owns columns cw = coff + 16 wc .. + 15 and produces the dV
+//             rows of the 16-step tiles 2jh, 2jh + 1 of every chunk; RR[kt] = R tile
+//             (k = 16kt + 4G + e, c = cw + i), all KD feature rows, is kept by both waves of a
+//             column tile (the same updates in the same order: identical bits).
 // ---------------------------------------------------------------------------
 template <int KD, int DH>
 __device__ __forceinline__ void sliced_bwd_dv(
     unsigned char* smem, int n, int coff, const half_t* __restrict__ q, const half_t* __restrict__ k,
     const half_t* __restrict__ g, const float* __restrict__ den_raw, half_t* __restrict__ dv, int T, int N) {
     using Cfg = SlicedBwdCfg<KD, DH>;
-    constexpr int NT = kSlicedThreads, C = Cfg::C, CSL = Cfg::CSL;
+    constexpr int NT = kGroupThreads, C = Cfg::C, CSL = Cfg::CSL;
     constexpr int LDQ = Cfg::LDQ, LDG = Cfg::LDS_, LDA = Cfg::LDA;
     constexpr int NKT = KD / 16;
     constexpr int PPR = CSL / 8, VP = ChunkRegs<CSL, NT>::kPieces;
-    half_t* ATs = reinterpret_cast<half_t*>(smem + 2 * Cfg::kStageB);    // AT[j][i] = A[i][j]
+    constexpr size_t kStage = Cfg::kLds / 2;
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int grp = w >> 2, wc = w & 3;
+    const int tid = threadIdx.x & (NT - 1);
     const int row = lane & 15, G = lane >> 4;
-    const int wc = w & 3, jh = w >> 2;
     const int cl = 16 * wc;                     // first column of this wave, local to the slice array
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
-    const half_t* qb = q + (int64_t)n * KD;
-    const half_t* kb = k + (int64_t)n * KD;
-    const half_t* gb = g + (int64_t)n * DH + coff;
-    half_t* dvb = dv + (int64_t)n * DH + coff;
+    const int n_chunks = (T + C - 1) / C;
     RFA_TICK_INIT();
-    constexpr int TB = 10;
 
-    f4 RR[NKT];
-#pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) RR[kt] = f4_zero();
-
-    struct RowSet {
-        ChunkRegs<KD, NT> rq, rk;
-        ChunkRegs<CSL, NT> rg;
-        float den[VP];
-    };
-    RowSet s0, s1;
-    auto prefetch = [&](RowSet& r, int c) __attribute__((always_inline)) {
-        const int t0 = c * C, rows = T - t0;
-        chunk_g2r<KD, NT>(r.rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
-        chunk_g2r<KD, NT>(r.rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
-        chunk_g2r<CSL, NT>(r.rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
-#pragma unroll
-        for (int it = 0; it < VP; ++it) {
-            const int r_ = min((tid + NT * it) / PPR, r.rg.rows - 1);
-            r.den[it] = den_raw[(int64_t)(t0 + r_) * N + n];
-        }
+    struct Stage { half_t *Qs, *Ks, *Gs, *ATs; };
+    auto stage_of = [&](int i) __attribute__((always_inline)) {
+        Stage st;
+        st.Qs = reinterpret_cast<half_t*>(smem + (i & 1) * kStage);
+        st.Ks = st.Qs + C * LDQ;
+        st.Gs = st.Ks + C * LDQ;                 // G / den, this slice's columns
+        st.ATs = st.Gs + C * LDG;                // AT[j][i] = A[i][j]
+        return st;
     };
 
-    auto chunk_body = [&](auto ragged_tag, int ci, RowSet& r, int c_next) __attribute__((always_inline)) {
-        constexpr bool RAGGED = decltype(ragged_tag)::value;
-        const int t0 = ci * C;
-        unsigned char* stage = smem + (ci & 1) * Cfg::kStageB;
-        half_t* Qs = reinterpret_cast<half_t*>(stage);
-        half_t* Ks = Qs + C * LDQ;
-        half_t* Gs = Ks + C * LDQ;               // G / den, this slice's columns
-
-        chunk_r2s<KD, NT>(r.rk, Ks, LDQ, tid);
-        chunk_r2s<KD, NT>(r.rq, Qs, LDQ, tid);
-        float inv_den[VP];
+    if (grp == 0) {
+        const half_t* qb = q + (int64_t)n * KD;
+        const half_t* kb = k + (int64_t)n * KD;
+        const half_t* gb = g + (int64_t)n * DH + coff;
+        RowPtrs<KD> pq, pk;
+        RowPtrs<CSL> pg;
+        pq.init(qb, k_stride, tid);
+        pk.init(kb, k_stride, tid);
+        pg.init(gb, v_stride, tid);
+        struct RowSet {
+            ChunkRegs<KD, NT> rq, rk;
+            ChunkRegs<CSL, NT> rg;
+            float den[VP];
+        };
+        RowSet s0, s1;
+        auto prefetch_ragged = [&](RowSet& r, int c) __attribute__((always_inline)) {
+            const int t0 = c * C, rows = T - t0;
+            chunk_g2r<KD, NT>(r.rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+            chunk_g2r<KD, NT>(r.rq, qb + (int64_t)t0 * k_stride, k_stride, rows, tid);
+            chunk_g2r<CSL, NT>(r.rg, gb + (int64_t)t0 * v_stride, v_stride, rows, tid);
 #pragma unroll
-        for (int it = 0; it < VP; ++it) inv_den[it] = 1.0f / fmaxf(r.den[it], 1.0f);
-        chunk_r2s_scaled<CSL, NT>(r.rg, inv_den, Gs, LDG, tid);
-        RFA_TICK(TB + 1);
-        __syncthreads();
-        RFA_TICK(TB + 2);
-        prefetch(r, c_next);
-        RFA_TICK(TB + 3);
-
-        // ---- A = tril(Q K^T) tiles (m = i, n = j), stored transposed: the sixteen tiles of the
-        // chunk, two per wave, no branch around the products (see p_tiles of the dQ/dK role)
-#pragma unroll
-        for (int s_ = 0; s_ < 2; ++s_) {
-            const int it = w >> 1, jt = 2 * (w & 1) + s_;
-            const int j = 16 * jt + row;
-            f4 a_ = f4_zero();
-#pragma unroll
-            for (int ks = 0; ks < KD / 32; ++ks)
-                a_ = mfma32(row8(Qs, LDQ, 16 * it + row, ks * 32, G), row8(Ks, LDQ, j, ks * 32, G), a_);
-            h4 av;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int i = 16 * it + 4 * G + e;
-                av[e] = (i >= j) ? (half_t)a_[e] : (half_t)0.f;
+            for (int it = 0; it < VP; ++it) {
+                const int r_ = min((tid + NT * it) / PPR, r.rg.rows - 1);
+                r.den[it] = den_raw[(int64_t)(t0 + r_) * N + n];
             }
-            *reinterpret_cast<h4*>(ATs + j * LDA + 16 * it + 4 * G) = av;
-        }
-        RFA_TICK(TB + 4);
-        __syncthreads();
-        RFA_TICK(TB + 5);
+        };
+        auto prefetch = [&](RowSet& r, int c) __attribute__((always_inline)) {
+            const int64_t t0 = (int64_t)c * C;
+            pk.load_full(r.rk, t0 * k_stride);
+            pq.load_full(r.rq, t0 * k_stride);
+            pg.load_full(r.rg, t0 * v_stride);
+#pragma unroll
+            for (int it = 0; it < VP; ++it) r.den[it] = den_raw[(t0 + (tid + NT * it) / PPR) * N + n];
+        };
+        auto stage_chunk = [&](int i, RowSet& r, int c_next, bool do_prefetch) __attribute__((always_inline)) {
+            const Stage st = stage_of(i);
+            chunk_r2s<KD, NT>(r.rk, st.Ks, LDQ, tid);
+            chunk_r2s<KD, NT>(r.rq, st.Qs, LDQ, tid);
+            float inv_den[VP];
+#pragma unroll
+            for (int it = 0; it < VP; ++it) inv_den[it] = 1.0f / fmaxf(r.den[it], 1.0f);
+            chunk_r2s_scaled<CSL, NT>(r.rg, inv_den, st.Gs, LDG, tid);
+            RFA_TICK_AT(1, 0);
+            wg_sync();
+            RFA_TICK_AT(2, 0);
+            if (do_prefetch) prefetch(r, c_next);
+            RFA_TICK_AT(3, 0);
+            // A = tril(Q K^T) tiles (m = i, n = j), stored transposed: column block wc, all four row
+            // tiles, no branch around the products
+            {
+                const int j = 16 * wc + row;
+                f4 a_[4];
+#pragma unroll
+                for (int it = 0; it < 4; ++it) a_[it] = f4_zero();
+#pragma unroll
+                for (int ks = 0; ks < KD / 32; ++ks) {
+                    const h8 bk = row8(st.Ks, LDQ, j, ks * 32, G);
+#pragma unroll
+                    for (int it = 0; it < 4; ++it) a_[it] = mfma32(row8(st.Qs, LDQ, 16 * it + row, ks * 32, G), bk, a_[it]);
+                }
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    h4 av;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int ii = 16 * it + 4 * G + e;
+                        av[e] = (ii >= j) ? (half_t)a_[it][e] : (half_t)0.f;
+                    }
+                    *reinterpret_cast<h4*>(st.ATs + j * LDA + 16 * it + 4 * G) = av;
+                }
+            }
+            RFA_TICK_AT(4, 0);
+            wg_sync();
+            RFA_TICK_AT(5, 0);
+        };
 
-        // ---- dV^T tiles (m = c, n = j) for j tiles 2jh, 2jh + 1, then R += Q^T G^
-        {
+        const bool multi = n_chunks > 1;
+        prefetch_ragged(s0, n_chunks - 1);
+        if (multi) prefetch(s1, n_chunks - 2);
+        stage_chunk(0, s0, max(n_chunks - 3, 0), multi);
+        for (int i = 1; i < n_chunks; i += 2) {
+            stage_chunk(i, s1, max(n_chunks - 3 - i, 0), true);
+            if (i + 1 >= n_chunks) break;
+            stage_chunk(i + 1, s0, max(n_chunks - 4 - i, 0), true);
+        }
+        wg_sync();
+        wg_sync();
+    } else {
+        const int jh = grp - 1;
+        half_t* dvb = dv + (int64_t)n * DH + coff;
+        f4 RR[NKT];
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt) RR[kt] = f4_zero();
+        auto chunk_body = [&](auto ragged_tag, int i) __attribute__((always_inline)) {
+            constexpr bool RAGGED = decltype(ragged_tag)::value;
+            const int t0 = (n_chunks - i) * C;
+            const Stage st = stage_of(i - 1);
+            // dV^T tiles (m = c, n = j) for j tiles 2jh, 2jh + 1, then R += Q^T G^
             h8 gf[2];     // G^ column fragments: G^[i = 32is + 8G + e][c = cl + lane i]
 #pragma unroll
-            for (int is = 0; is < 2; ++is) gf[is] = col8(Gs, LDG, is * 32, cl, lane);
+            for (int is = 0; is < 2; ++is) gf[is] = col8(st.Gs, LDG, is * 32, cl, lane);
             f4 dvacc[2];
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int jr = 16 * (2 * jh + u) + row;
-                // rows i < 32 of A^T only reach the first two j tiles: their operand is all zero for
-                // the other half, and multiplying by zeros keeps the two halves on one code path
-                f4 acc = mfma32(gf[0], row8(ATs, LDA, jr, 0, G), f4_zero());
-                acc = mfma32(gf[1], row8(ATs, LDA, jr, 32, G), acc);
+                // rows i < 32 of A^T only reach the first two j tiles: their operand is all zero
+                // for the other group, and multiplying by zeros keeps both groups on one code path
+                f4 acc = mfma32(gf[0], row8(st.ATs, LDA, jr, 0, G), f4_zero());
+                acc = mfma32(gf[1], row8(st.ATs, LDA, jr, 32, G), acc);
                 dvacc[u] = acc;
             }
 #pragma unroll
             for (int ks = 0; ks < KD / 32; ++ks) {
                 h8 bkk[2];
 #pragma unroll
-                for (int u = 0; u < 2; ++u) bkk[u] = row_split8(Ks, LDQ, 16 * (2 * jh + u) + row, ks * 32, G);
+                for (int u = 0; u < 2; ++u) bkk[u] = row_split8(st.Ks, LDQ, 16 * (2 * jh + u) + row, ks * 32, G);
                 __builtin_amdgcn_sched_barrier(0);
                 h8 hi, lo;
                 acc_to_operand(RR[2 * ks], RR[2 * ks + 1], hi, lo);
@@ -462,6 +565,9 @@ __device__ __forceinline__ void sliced_bwd_dv(
                     dvacc[u] = mfma32(lo, bkk[u], dvacc[u]);
                 }
             }
+            RFA_TICK_AT(11, 256);
+            wg_sync();
+            RFA_TICK_AT(12, 256);
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int jj = 16 * (2 * jh + u) + row;
@@ -471,20 +577,16 @@ __device__ __forceinline__ void sliced_bwd_dv(
 #pragma unroll
             for (int is = 0; is < 2; ++is)
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt) RR[kt] = mfma32(col8(Qs, LDQ, is * 32, 16 * kt, lane), gf[is], RR[kt]);
-        }
-        RFA_TICK(TB + 7);
-    };
-
-    const int n_chunks = (T + C - 1) / C;
-    prefetch(s0, n_chunks - 1);
-    prefetch(s1, max(n_chunks - 2, 0));
-    RFA_TICK(TB + 0);
-    chunk_body(std::true_type{}, n_chunks - 1, s0, max(n_chunks - 3, 0));
-    for (int ci = n_chunks - 2; ci >= 0; ci -= 2) {
-        chunk_body(std::false_type{}, ci, s1, max(ci - 2, 0));
-        if (ci - 1 < 0) break;
-        chunk_body(std::false_type{}, ci - 1, s0, max(ci - 3, 0));
+                for (int kt = 0; kt < NKT; ++kt)
+                    RR[kt] = mfma32(col8(st.Qs, LDQ, is * 32, 16 * kt, lane), gf[is], RR[kt]);
+            RFA_TICK_AT(13, 256);
+            wg_sync();
+            RFA_TICK_AT(14, 256);
+        };
+        wg_sync();
+        wg_sync();
+        chunk_body(std::true_type{}, 1);
+        for (int i = 2; i <= n_chunks; ++i) chunk_body(std::false_type{}, i);
     }
 }
 
