@@ -1,7 +1,9 @@
-"""Builds librfa_hip.so (the C-ABI kernel library) for gfx950 with hipcc.
+"""Builds librfa_hip.so (the C-ABI kernel library) for gfx950 with hipcc, and
+_rfa_hip_ext.so, the PyTorch C++ binding of that library (host code only, g++).
 
-Usage:  python -m rfa_amd.build [--verbose] [--resource-usage]
-The library is written next to this file; it is what rfa_amd._lib loads.
+Usage:  python -m rfa_amd.build [--verbose] [--resource-usage] [--no-ext]
+Both are written next to this file; rfa_amd._lib loads the first with ctypes, rfa_amd.rfa_hip
+imports the second when it is there.
 """
 from __future__ import annotations
 
@@ -50,6 +52,40 @@ def build(verbose: bool = False, extra_flags=()) -> str:
     return LIB_PATH
 
 
+EXT_NAME = "_rfa_hip_ext"
+EXT_PATH = os.path.join(HERE, EXT_NAME + ".so")
+
+
+def build_ext(verbose: bool = False) -> str:
+    """The torch binding: one host C++ file compiled against torch's headers and linked to
+    librfa_hip.so (found next to it at run time through $ORIGIN).  No kernels, nothing for hipcc."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-DTORCH_EXTENSION_NAME={EXT_NAME}",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-Wno-deprecated-declarations",
+           *[f"-I{p}" for p in ce.include_paths()], f"-I{sysconfig.get_paths()['include']}", f"-I{rocm}/include",
+           os.path.join(CSRC, "rfa_torch_ext.cpp"), "-o", EXT_PATH,
+           f"-L{torch_lib}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
+           f"-L{HERE}", "-l:librfa_hip.so", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("building the torch binding failed:\n" + proc.stdout)
+    if verbose and proc.stdout.strip():
+        print(proc.stdout)
+    return EXT_PATH
+
+
 if __name__ == "__main__":
     extra = ["-Rpass-analysis=kernel-resource-usage"] if "--resource-usage" in sys.argv else []
-    print(build(verbose=True if extra else ("--verbose" in sys.argv or "-v" in sys.argv), extra_flags=extra))
+    verbose = True if extra else ("--verbose" in sys.argv or "-v" in sys.argv)
+    print(build(verbose=verbose, extra_flags=extra))
+    if "--no-ext" not in sys.argv and not extra:
+        print(build_ext(verbose=verbose))

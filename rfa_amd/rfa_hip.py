@@ -3,9 +3,16 @@ reference's pybind extension ``rfa_cuda`` stood
 (random_feature_attention/cuda/rfa_cuda.cpp:39-42), with the same two entry
 points ``forward(q, k, v)`` and ``backward(q, k, v, grad_attn)`` and the same
 argument order and return arity, plus the entry points for the other parts of
-the path.  Tensors are validated here (the reference validated nothing,
+the path.  Tensors are validated (the reference validated nothing,
 cuda/forward.cu:156-159) and handed to the C ABI as raw device pointers; the
 work is enqueued on the current torch stream.
+
+Two bindings of the same library stand behind these names.  ``_rfa_hip_ext`` is a PyTorch C++
+extension (csrc/rfa_torch_ext.cpp: TORCH_CHECK, device guard, current HIP stream, outputs from
+torch's allocator, a few microseconds of host time per call) and is used when it has been built;
+the functions written out in this file do the same through ctypes and need nothing but the
+shared library.  ``use_binding("ext" | "ctypes")`` switches, ``binding()`` tells which is active;
+the environment variable RFA_AMD_BINDING picks the initial one.
 """
 from __future__ import annotations
 
@@ -592,3 +599,52 @@ def masked_backward(phi_q: Tensor, phi_k: Tensor, v: Tensor, grad_attn: Tensor, 
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), T, Tp, B, H, K, d, ws.data_ptr(), nbytes,
             _stream_ptr(v.device)))
     return [dq, dk, dv]
+
+
+# ---------------------------------------------------------------------------
+# binding selection
+# ---------------------------------------------------------------------------
+_BOUND = ("supported", "feature_map_supported", "selftest_layout", "forward", "backward", "prefill", "forward_save",
+          "backward_saved", "build_random_matrices", "build_random_matrices_backward", "feature_map_forward",
+          "feature_map_backward", "feature_map_backward_pair", "project_feature_map", "linear_weight_grad", "cross_state",
+          "cross_state_backward", "cross_readout", "cross_readout_backward", "incremental", "incremental_fused",
+          "masked_forward", "masked_backward")
+_CTYPES_IMPL = {name: globals()[name] for name in _BOUND}
+_active = "ctypes"
+
+try:
+    from . import _rfa_hip_ext as _ext      # built by rfa_amd.build.build_ext
+except ImportError:
+    _ext = None
+
+
+def ext_available() -> bool:
+    return _ext is not None
+
+
+def binding() -> str:
+    """"ext" or "ctypes": which binding the functions of this module currently go through."""
+    return _active
+
+
+def use_binding(name: str) -> None:
+    global _active
+    if name == "ext":
+        if _ext is None:
+            raise ImportError("the torch binding _rfa_hip_ext has not been built (python -m rfa_amd.build)")
+        impl = {n: getattr(_ext, n) for n in _BOUND}
+    elif name == "ctypes":
+        impl = _CTYPES_IMPL
+    else:
+        raise ValueError(f"binding must be 'ext' or 'ctypes' (got {name!r})")
+    globals().update(impl)
+    _active = name
+
+
+def _initial_binding() -> None:
+    import os
+    want = os.environ.get("RFA_AMD_BINDING", "ext" if _ext is not None else "ctypes")
+    use_binding(want)
+
+
+_initial_binding()

@@ -38,3 +38,16 @@ def knobs():
     yield set_
     for name in touched:
         _lib.tuning_set(name, -1)
+
+
+@pytest.fixture(params=["ext", "ctypes"])
+def binding(request):
+    """Runs a test once through each binding of the kernel library: the PyTorch C++ extension and
+    the ctypes wrappers (use with pytest.mark.usefixtures("binding"))."""
+    from rfa_amd import rfa_hip
+    if request.param == "ext" and not rfa_hip.ext_available():
+        pytest.skip("the torch binding has not been built")
+    before = rfa_hip.binding()
+    rfa_hip.use_binding(request.param)
+    yield request.param
+    rfa_hip.use_binding(before)

@@ -10,7 +10,7 @@ import torch
 
 from oracle import rfa_oracle as O
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("binding")]
 
 OUT_ATOL = 2e-3
 GRAD_RTOL = 1e-2

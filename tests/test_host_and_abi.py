@@ -44,11 +44,14 @@ def test_tuning_knobs_round_trip():
     with pytest.raises(_lib.RfaHipError, match="no knob"):
         _lib.tuning_set("no_such_knob", 1)
     # the saved buffer grows by its 256-byte header and follows the plan
-    with _lib.tuning(nseg=1):
+    with _lib.tuning(nseg=1, sliced=0):
         one = lib.rfa_causal_saved_state_bytes(1024, 64, 128, 64)
-    with _lib.tuning(nseg=4, prefix=0):
+    with _lib.tuning(nseg=4, prefix=0, sliced=0):
         four = lib.rfa_causal_saved_state_bytes(1024, 64, 128, 64)
     assert one >= 256 + 64 * (128 * 64 + 128) * 4 + 1024 * 64 * 4 and four >= one + 3 * 64 * 128 * 64 * 4
+    # with the final-state layout the buffer holds one state per sequence whatever the segment count
+    with _lib.tuning(nseg=4, sliced=1):
+        assert lib.rfa_causal_saved_state_bytes(1024, 64, 128, 64) == one
 
 
 def test_errors_are_reported_before_any_gpu_work():
@@ -73,6 +76,7 @@ def test_errors_are_reported_before_any_gpu_work():
         _lib.check(-3)
 
 
+@pytest.mark.usefixtures("binding")
 def test_host_wrappers_reject_cpu_and_wrong_dtype():
     from rfa_amd import RFA, rfa_hip
     q = torch.zeros(4, 2, 128, dtype=torch.float16)
@@ -184,6 +188,25 @@ def test_random_matrix_generators():
     assert np.allclose(unit @ unit.T, np.eye(16), atol=1e-10)      # orthogonal directions
     np.random.seed(2)
     assert softmax_kernel_error(16, 2048, rrf(head_dim=16, proj_dim=2048), iters=5) < 0.15
+
+
+def test_both_bindings_expose_the_same_functions():
+    """The torch extension and the ctypes wrappers stand behind one set of names."""
+    from rfa_amd import rfa_hip
+    assert rfa_hip.ext_available(), "python -m rfa_amd.build builds the torch binding"
+    before = rfa_hip.binding()
+    try:
+        for name in ("ext", "ctypes"):
+            rfa_hip.use_binding(name)
+            assert rfa_hip.binding() == name
+            for fn in rfa_hip._BOUND:
+                assert callable(getattr(rfa_hip, fn)), (name, fn)
+            assert rfa_hip.supported(128, 64) and not rfa_hip.supported(100, 64)
+        with pytest.raises(ValueError):
+            rfa_hip.use_binding("pybind")
+    finally:
+        rfa_hip.use_binding(before)
+    assert before == "ext"          # the default when the extension is there
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
