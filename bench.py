@@ -28,12 +28,12 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the bench configuration, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
 # passes summarised in profiles/bench_cfg2_hbm_traffic.md (counters scaled on the 512 MiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "k_segment_state": 25430824,
-    "k_causal_fwd": 59003656,
-    "k_causal_bwd_dq": 92586196,
+    "k_segment_state": 25430665,
+    "k_causal_fwd": 61162601,
+    "k_causal_bwd_dq": 92586196,       # the two-sweep backward (tuning knob sliced = 0)
     "k_causal_bwd_dkdv": 86253280,
-    "k_sliced_bwd": None,
-    "k_decode_step": 68884953,
+    "k_sliced_bwd": 105340904,
+    "k_decode_step": 68884930,
 }
 
 
@@ -55,6 +55,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip decode / cross / feature-map figures")
+    ap.add_argument("--skip", default="", help="comma-separated extras to leave out (decode_module: the per-token "
+                    "module decode loop and its HIP graph)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every box of this build has one GPU and the path needs no "
@@ -188,11 +190,11 @@ def main():
     }
 
     if not args.no_extras:
-        result["extras"] = extras(torch, O, lib, _lib, rfa_hip, dev, stream)
+        result["extras"] = extras(torch, O, lib, _lib, rfa_hip, dev, stream, set(filter(None, args.skip.split(","))))
     print(json.dumps(result))
 
 
-def extras(torch, O, lib, _lib, rfa_hip, dev, stream):
+def extras(torch, O, lib, _lib, rfa_hip, dev, stream, skip=()):
     ex = {}
     p = lambda t: t.data_ptr()
     # ---- decode (config 4): B64 H16 d64 D64, 2048 steps after a 512-token prefill
@@ -253,59 +255,60 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream):
                                        s0[:1, :2].cpu().reshape(2, K, d), z0[:1, :2].cpu().reshape(2, K))
     ex["decode"]["parity_max_abs"] = (outs[:8, :1, :2].float().cpu().reshape(8, 2, d) - want).abs().max().item()
     del qs, ks, vs, outs
-    # (3) through the API the reference exposes: one CausalAttention.forward(x[1], W, saved_state=state)
-    # per token (causal_attention.py:249-265), q/k/v/out projections included; eager calls, then the
-    # same step captured once into a HIP graph (state advanced in place) and replayed
-    from rfa_amd import CausalAttention
-    torch.manual_seed(0)
-    E = H * d
-    dec = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).to(dev).half().eval()
-    xs = (torch.randn(256, B, E, generator=g) * 0.5).half().to(dev)
-    shape4 = (B, H, K, d)
-    with torch.no_grad():
-        state = {"prev_s": s0.view(shape4).clone(), "prev_z": z0.view(B, H, K).clone()}
-        y_first = dec(xs[0:1], W, saved_state=state).clone()
-        for t in range(1, 16):
-            dec(xs[t:t + 1], W, saved_state=state)
-        torch.cuda.synchronize()
-        _lib.check(lib.rfa_profile_reset()); _lib.check(lib.rfa_profile_enable(1))
-        t0 = time.perf_counter()
-        for t in range(steps):
-            dec(xs[t % 256:t % 256 + 1], W, saved_state=state)
-        torch.cuda.synchronize()
-        eager_s = time.perf_counter() - t0
-        _lib.check(lib.rfa_profile_enable(0))
-        step_kernel_us = {n_: round(1e3 * ms_ / c_, 2) for n_, (ms_, c_) in _lib.profile_totals().items()}
-        dec.decode_inplace = True
-        gstate = {"prev_s": s0.view(shape4).clone(), "prev_z": z0.view(B, H, K).clone()}
-        gs, gz = gstate["prev_s"], gstate["prev_z"]
-        xg = xs[0:1].clone()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(3):
-                dec(xg, W, saved_state=gstate)
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            yg = dec(xg, W, saved_state=gstate)
-        in_place = gstate["prev_s"] is gs and gstate["prev_z"] is gz
-        gs.copy_(s0.view(shape4)); gz.copy_(z0.view(B, H, K))
-        graph.replay()
-        torch.cuda.synchronize()
-        graph_ok = bool(in_place and torch.equal(yg, y_first))
-        for _ in range(16):
+    if "decode_module" not in skip:
+        # (3) through the API the reference exposes: one CausalAttention.forward(x[1], W, saved_state=state)
+        # per token (causal_attention.py:249-265), q/k/v/out projections included; eager calls, then the
+        # same step captured once into a HIP graph (state advanced in place) and replayed
+        from rfa_amd import CausalAttention
+        torch.manual_seed(0)
+        E = H * d
+        dec = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).to(dev).half().eval()
+        xs = (torch.randn(256, B, E, generator=g) * 0.5).half().to(dev)
+        shape4 = (B, H, K, d)
+        with torch.no_grad():
+            state = {"prev_s": s0.view(shape4).clone(), "prev_z": z0.view(B, H, K).clone()}
+            y_first = dec(xs[0:1], W, saved_state=state).clone()
+            for t in range(1, 16):
+                dec(xs[t:t + 1], W, saved_state=state)
+            torch.cuda.synchronize()
+            _lib.check(lib.rfa_profile_reset()); _lib.check(lib.rfa_profile_enable(1))
+            t0 = time.perf_counter()
+            for t in range(steps):
+                dec(xs[t % 256:t % 256 + 1], W, saved_state=state)
+            torch.cuda.synchronize()
+            eager_s = time.perf_counter() - t0
+            _lib.check(lib.rfa_profile_enable(0))
+            step_kernel_us = {n_: round(1e3 * ms_ / c_, 2) for n_, (ms_, c_) in _lib.profile_totals().items()}
+            dec.decode_inplace = True
+            gstate = {"prev_s": s0.view(shape4).clone(), "prev_z": z0.view(B, H, K).clone()}
+            gs, gz = gstate["prev_s"], gstate["prev_z"]
+            xg = xs[0:1].clone()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    dec(xg, W, saved_state=gstate)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                yg = dec(xg, W, saved_state=gstate)
+            in_place = gstate["prev_s"] is gs and gstate["prev_z"] is gz
+            gs.copy_(s0.view(shape4)); gz.copy_(z0.view(B, H, K))
             graph.replay()
-        graph_ms = _event_time_ms(torch, graph.replay, steps)
-    ex["decode"]["module_per_token"] = {
-        "workload": "CausalAttention(embed 1024, 16 heads).forward(x[1, 64, 1024], W, saved_state) per token, 2048 tokens",
-        "eager_us_per_step": round(1e6 * eager_s / steps, 2), "eager_tokens_per_s": round(B * steps / eager_s, 1),
-        "hip_graph_replay_us_per_step": round(1e3 * graph_ms, 2),
-        "hip_graph_tokens_per_s": round(B / (graph_ms * 1e-3), 1),
-        "decode_kernel_us": step_kernel_us.get("k_decode_step"), "library_kernels_us": step_kernel_us,
-        "graph_equals_eager": graph_ok}
-    del dec, graph, xs, state, gstate
+            torch.cuda.synchronize()
+            graph_ok = bool(in_place and torch.equal(yg, y_first))
+            for _ in range(16):
+                graph.replay()
+            graph_ms = _event_time_ms(torch, graph.replay, steps)
+        ex["decode"]["module_per_token"] = {
+            "workload": "CausalAttention(embed 1024, 16 heads).forward(x[1, 64, 1024], W, saved_state) per token, 2048 tokens",
+            "eager_us_per_step": round(1e6 * eager_s / steps, 2), "eager_tokens_per_s": round(B * steps / eager_s, 1),
+            "hip_graph_replay_us_per_step": round(1e3 * graph_ms, 2),
+            "hip_graph_tokens_per_s": round(B / (graph_ms * 1e-3), 1),
+            "decode_kernel_us": step_kernel_us.get("k_decode_step"), "library_kernels_us": step_kernel_us,
+            "graph_equals_eager": graph_ok}
+        del dec, graph, xs, state, gstate
 
     # ---- cross attention (config 3): T256 S512 B32 H8, lengths U[256, 512]
     Tt, S, B, H = 256, 512, 32, 8
