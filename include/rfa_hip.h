@@ -108,8 +108,9 @@ int rfa_causal_backward(const void* q, const void* k, const void* v, const void*
 
 /* Training-step variants (no counterpart in the reference, whose autograd Function
  * saves only q, k, v: rfa.py:124).  rfa_causal_forward_save additionally writes what
- * the backward pass can reuse into `saved` (rfa_causal_saved_state_bytes bytes: the
- * per-segment state totals and the raw denominators, fp32); rfa_causal_backward_saved
+ * the backward pass can reuse into `saved` (rfa_causal_saved_state_bytes bytes, fp32: the
+ * raw denominators and either the per-segment state totals or, where the backward runs as
+ * one launch over state slices, the state after the last step); rfa_causal_backward_saved
  * reads them, and the forward output `out` (fp16 [T, N, d], as written by that forward
  * call), instead of recomputing the forward pass: with num = out * den the term
  * g . num of rfa.py:91 is (g . out) * den.  `saved` and `out` must come from a forward
@@ -148,6 +149,9 @@ int rfa_causal_num_segments(int64_t T, int64_t N, int K, int d);
  *   "nseg_same"  1: the K = 256, d = 128 backward keeps the forward's segment length
  *   "free_wg"  workgroups the cross-attention readout and state backward aim for
  *   "project_streaming"  1: rfa_project_feature_map uses its streaming kernel for every shape
+ *   "sliced"  1/0: rfa_causal_forward_save writes the final-state layout, whose backward is one
+ *             launch that walks whole sequences by state slices (K <= 128, d = 64 only) / the
+ *             segment-totals layout of the two-sweep backward
  * Initial values come from the environment variables RFA_HIP_<NAME>, read once per process and
  * never on the launch path.  No counterpart in the reference. */
 int rfa_tuning_set(const char* name, int value);
