@@ -210,8 +210,9 @@ int rfa_feature_map_backward_pair(const void* x0, const void* x1, const void* w,
  *   x        : fp16 [R, E]      R = seq_len * bsz rows, E a multiple of 64
  *   weights  : np pointers (1 <= np <= 3) to fp16 [H*d, E], torch.nn.Linear.weight layout
  *   biases   : np pointers to fp16 [H*d] (8-byte aligned); the array or any entry may be NULL
- *   y        : np pointers to fp16 [R, H, d]   y_p = x W_p^T + b_p, always written (the
- *              backward of the feature map needs it)
+ *   y        : np pointers to fp16 [R, H, d]   y_p = x W_p^T + b_p (the backward of the feature
+ *              map needs it); an entry may be NULL where phi[p] is not: that projection then
+ *              leaves only phi(y_p) behind (inference, no backward pass)
  *   phi      : np pointers to fp16 [R, H, 2D], or NULL entries (or a NULL array): projection p
  *              gets phi(y_p) only where phi[p] is non-NULL
  *   w_feat   : fp16 [H, D, d] as for rfa_feature_map_forward; may be NULL if no phi is asked for

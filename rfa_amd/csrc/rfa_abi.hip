@@ -1578,7 +1578,8 @@ int rfa_project_feature_map(const void* x, const void* const* weights, const voi
         pa.b[p] = biases ? static_cast<const rfa::half_t*>(biases[p]) : nullptr;
         pa.y[p] = static_cast<rfa::half_t*>(y[p]);
         pa.phi[p] = phi ? static_cast<rfa::half_t*>(phi[p]) : nullptr;
-        if (!pa.w[p] || !pa.y[p]) return fail(RFA_ERR_NULL_POINTER, "rfa_project_feature_map: NULL weight or output %d", p);
+        if (!pa.w[p] || (!pa.y[p] && !pa.phi[p]))
+            return fail(RFA_ERR_NULL_POINTER, "rfa_project_feature_map: NULL weight %d, or neither y nor phi asked for", p);
         if (!aligned16(pa.w[p]) || !aligned16(pa.y[p]) || !aligned16(pa.phi[p]) ||
             (reinterpret_cast<uintptr_t>(pa.b[p]) & 7u))
             return fail(RFA_ERR_ALIGNMENT, "rfa_project_feature_map: tensors must be 16-byte aligned (bias: 8)");

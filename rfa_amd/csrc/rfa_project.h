@@ -174,11 +174,13 @@ __global__ __launch_bounds__(kThreads) void k_project_phi(
                 ss += (float)yh[e] * (float)yh[e];
                 op[ct / 2][4 * (ct % 2) + e] = yh[e];
             }
-            *reinterpret_cast<h4*>(Ps + i * LDP + 16 * ct + 4 * G) = yh;
+            if (y) *reinterpret_cast<h4*>(Ps + i * LDP + 16 * ct + 4 * G) = yh;
         }
-        wave_lds_order();
-        wave_rows_s2g<DH>(Ps, LDP, y, r0, R, H, h, lane);
-        wave_lds_order();
+        if (y) {        // NULL: the caller keeps only phi(y) (no backward pass will ask for y)
+            wave_lds_order();
+            wave_rows_s2g<DH>(Ps, LDP, y, r0, R, H, h, lane);
+            wave_lds_order();
+        }
         if (phi) {
             ss = sum_over_groups(ss);
             const float inv = 1.0f / (sqrtf(ss) + 1e-3f);
@@ -364,11 +366,13 @@ __global__ __launch_bounds__(kThreads) void k_project_phi_rows(
                     ss += (float)yh[e] * (float)yh[e];
                     op[ct / 2][4 * (ct % 2) + e] = yh[e];
                 }
-                *reinterpret_cast<h4*>(Ps + i * LDP + 16 * ct + 4 * G) = yh;
+                if (y) *reinterpret_cast<h4*>(Ps + i * LDP + 16 * ct + 4 * G) = yh;
             }
-            wave_lds_order();
-            wave_rows_s2g<DH>(Ps, LDP, y, r0, R, H, h, lane);
-            wave_lds_order();
+            if (y) {
+                wave_lds_order();
+                wave_rows_s2g<DH>(Ps, LDP, y, r0, R, H, h, lane);
+                wave_lds_order();
+            }
             if (phi) {
                 ss = sum_over_groups(ss);
                 const float inv = 1.0f / (sqrtf(ss) + 1e-3f);

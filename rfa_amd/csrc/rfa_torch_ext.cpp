@@ -236,9 +236,11 @@ std::tuple<Tensor, Tensor, Tensor> feature_map_backward_pair(const Tensor& x0, c
 }
 
 // ---- projections ----------------------------------------------------------------------
-std::tuple<std::vector<Tensor>, std::vector<c10::optional<Tensor>>> project_feature_map(
+// keep_y = false: a projection whose phi is asked for returns None in place of y (nothing will
+// differentiate through it)
+std::tuple<std::vector<c10::optional<Tensor>>, std::vector<c10::optional<Tensor>>> project_feature_map(
     const Tensor& x, const std::vector<Tensor>& weights, const std::vector<c10::optional<Tensor>>& biases,
-    const std::vector<bool>& want_phi, const c10::optional<Tensor>& w, int64_t heads, double scale) {
+    const std::vector<bool>& want_phi, const c10::optional<Tensor>& w, int64_t heads, double scale, bool keep_y) {
     check_half("x", x, 3);
     const int64_t L = x.size(0), B = x.size(1), E = x.size(2);
     const size_t n = weights.size();
@@ -268,12 +270,11 @@ std::tuple<std::vector<Tensor>, std::vector<c10::optional<Tensor>>> project_feat
                           w->sizes(), " must be [", heads, ", D, ", d, "] on x's device");
         D = w->size(1);
     }
-    std::vector<Tensor> ys;
-    std::vector<c10::optional<Tensor>> phis;
+    std::vector<c10::optional<Tensor>> ys, phis;
     std::array<const void*, 3> wp{}, bp{};
     std::array<void*, 3> yp{}, pp{};
     for (size_t p = 0; p < n; ++p) {
-        ys.push_back(torch::empty({L, B, heads, d}, x.options()));
+        ys.push_back(keep_y || !want_phi[p] ? c10::optional<Tensor>(torch::empty({L, B, heads, d}, x.options())) : c10::nullopt);
         phis.push_back(want_phi[p] ? c10::optional<Tensor>(torch::empty({L, B, heads, 2 * D}, x.options())) : c10::nullopt);
         wp[p] = ptr(weights[p]);
         bp[p] = ptr(biases[p]);
@@ -518,7 +519,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("feature_map_backward_pair", &feature_map_backward_pair, py::arg("x0"), py::arg("x1"), py::arg("w"),
           py::arg("grad_phi0"), py::arg("grad_phi1"), py::arg("scale"));
     m.def("project_feature_map", &project_feature_map, py::arg("x"), py::arg("weights"), py::arg("biases"),
-          py::arg("want_phi"), py::arg("w"), py::arg("heads"), py::arg("scale"));
+          py::arg("want_phi"), py::arg("w"), py::arg("heads"), py::arg("scale"), py::arg("keep_y") = true);
     m.def("linear_weight_grad", &linear_weight_grad, py::arg("x"), py::arg("dys"), py::arg("want_bias"));
     m.def("cross_state", &cross_state, py::arg("phi_k"), py::arg("v"), py::arg("key_padding_mask") = py::none());
     m.def("cross_state_backward", &cross_state_backward, py::arg("phi_k"), py::arg("v"), py::arg("ds"), py::arg("dz"),

@@ -33,12 +33,15 @@ class _ProjectHeads(torch.autograd.Function):
         n = len(want_phi)
         weights, biases = list(params[0::2]), list(params[1::2])
         wf = None if w_feat is None else w_feat.contiguous()
+        # y of a projection that goes through the feature map is only kept for the backward pass
+        keep_y = any(ctx.needs_input_grad)
         ys, phis = rfa_hip.project_feature_map(x.contiguous(), [w.contiguous() for w in weights], biases, list(want_phi),
-                                               wf, heads, scale)
+                                               wf, heads, scale, keep_y)
         ctx.scale, ctx.heads, ctx.want_phi = scale, heads, want_phi
         ctx.has_bias = tuple(b is not None for b in biases)
         ctx.has_wf = w_feat is not None
-        ctx.save_for_backward(x, *([wf] if wf is not None else []), *weights, *[y for y, f in zip(ys, want_phi) if f])
+        if keep_y:
+            ctx.save_for_backward(x, *([wf] if wf is not None else []), *weights, *[y for y, f in zip(ys, want_phi) if f])
         return tuple(phis[p] if want_phi[p] else ys[p] for p in range(n))
 
     @staticmethod

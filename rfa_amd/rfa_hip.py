@@ -265,13 +265,15 @@ def feature_map_forward(x: Tensor, w: Tensor, scale: float) -> Tensor:
     return phi
 
 
-def project_feature_map(x: Tensor, weights, biases, want_phi, w: Optional[Tensor], heads: int, scale: float):
+def project_feature_map(x: Tensor, weights, biases, want_phi, w: Optional[Tensor], heads: int, scale: float,
+                        keep_y: bool = True):
     """Linear projections of x to heads, with the feature map applied to some of them, in one launch.
 
     x fp16 [L, B, E]; weights: 1..3 fp16 [heads*d, E] (torch.nn.Linear.weight); biases: a matching
     list of fp16 [heads*d] or None entries; want_phi: one bool per projection; w fp16 [heads, D, d]
     (None allowed when no phi is wanted).  Returns (ys, phis): ys[p] fp16 [L, B, heads, d];
-    phis[p] fp16 [L, B, heads, 2D] or None.
+    phis[p] fp16 [L, B, heads, 2D] or None.  keep_y=False: ys[p] is None (and never written) where
+    phis[p] is produced -- for callers that will not differentiate through the feature map.
     """
     import ctypes
     _check_half_cuda("x", x, 3)
@@ -297,14 +299,15 @@ def project_feature_map(x: Tensor, weights, biases, want_phi, w: Optional[Tensor
         D = w.shape[1]
     else:
         D = 32
-    ys = [torch.empty((L, B, heads, d), dtype=torch.float16, device=x.device) for _ in range(n)]
+    ys = [torch.empty((L, B, heads, d), dtype=torch.float16, device=x.device) if keep_y or not f else None
+          for f in want_phi]
     phis = [torch.empty((L, B, heads, 2 * D), dtype=torch.float16, device=x.device) if f else None for f in want_phi]
     arr = ctypes.c_void_p * n
     ptr = lambda t: None if t is None else t.data_ptr()
     with _on_device(x.device):
         _lib.check(_lib.load().rfa_project_feature_map(
             x.data_ptr(), arr(*[wt.data_ptr() for wt in weights]), arr(*[ptr(b) for b in biases]),
-            arr(*[t.data_ptr() for t in ys]), arr(*[ptr(t) for t in phis]), n, ptr(w) if any(want_phi) else None,
+            arr(*[ptr(t) for t in ys]), arr(*[ptr(t) for t in phis]), n, ptr(w) if any(want_phi) else None,
             L * B, E, heads, D, d, float(scale), _stream_ptr(x.device)))
     return ys, phis
 

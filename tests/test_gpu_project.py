@@ -66,6 +66,39 @@ def test_qkv_projection_with_feature_map(L, B, E, H, d, D, streaming, knobs):
             assert (phi - ref).abs().max().item() <= 4e-3
 
 
+@pytest.mark.parametrize("streaming", [False, True])
+def test_projection_without_keeping_y(streaming, knobs):
+    """keep_y=False (what the modules ask for when nothing requires a gradient): phi and the plain
+    projection come out bit-identical to the keeping call, y of the phi projections is not produced."""
+    from rfa_amd import rfa_hip
+    from rfa_amd.projection import project_heads
+    knobs(project_streaming=1 if streaming else -1)
+    L, B, E, H, d, D = 200, 3, 256, 4, 64, 64
+    x, ws, bs = _inputs(L, B, E, H, d, 4321, 3)
+    wf = (_randn(H, D, d, seed=78) * 0.9).half().cuda()
+    args = (x.cuda(), [w.cuda() for w in ws], [b.cuda() for b in bs], [True, True, False], wf, H, O.SCALE)
+    print(f"project+phi without y, streaming={streaming}", flush=True)
+    ys, phis = rfa_hip.project_feature_map(*args)
+    ys0, phis0 = rfa_hip.project_feature_map(*args, keep_y=False)
+    assert ys0[0] is None and ys0[1] is None and phis0[2] is None
+    assert torch.equal(ys0[2], ys[2]) and torch.equal(phis0[0], phis[0]) and torch.equal(phis0[1], phis[1])
+    layers = []
+    for w, b in zip(ws, bs):
+        lin = torch.nn.Linear(E, H * d).cuda().half()
+        lin.weight.data.copy_(w); lin.bias.data.copy_(b)
+        layers.append(lin)
+    with torch.no_grad():
+        outs = project_heads(x.cuda(), layers, (True, True, False), H, wf, O.SCALE)
+    assert torch.equal(outs[0], phis[0]) and torch.equal(outs[1], phis[1]) and torch.equal(outs[2], ys[2])
+    with pytest.raises(Exception, match="neither y nor phi"):
+        from rfa_amd import _lib
+        import ctypes
+        arr = ctypes.c_void_p * 1
+        xx = x.cuda()
+        _lib.check(_lib.load().rfa_project_feature_map(xx.data_ptr(), arr(ws[0].cuda().data_ptr()), None, arr(None), None, 1,
+                                                       None, L * B, E, H, D, d, O.SCALE, None))
+
+
 def test_plain_projection_is_a_linear_layer():
     """No phi requested: out_proj-style use, one projection, with and without bias."""
     from rfa_amd import rfa_hip
