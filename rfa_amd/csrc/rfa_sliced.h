@@ -40,7 +40,7 @@
 namespace rfa {
 
 constexpr int kSliceWidth = 64;     // features (dQ/dK role) or value columns (dV role) per workgroup
-constexpr int kSlicedThreads = 768; // 12 waves: loader group + two product groups
+constexpr int kSlicedThreads = 512; // 8 waves: loader group (4) + four product waves
 constexpr int kGroupThreads = 256;  // threads per group
 
 // Workgroup index -> (sequence, role).  The wps workgroups of a sequence get indices that are
@@ -117,10 +117,11 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int grp = w >> 2, wf = w & 3;
-    const int tid = threadIdx.x & (NT - 1);     // thread inside its group
+    const int grp = w < 4 ? 0 : 1 + ((w - 4) >> 1);     // loader | dQ waves 4, 5 | dK waves 6, 7
+    const int wf = w & 3;                       // loader: row block of the P tiles
+    const int tid = threadIdx.x & (NT - 1);     // thread inside the loader group
     const int row = lane & 15, G = lane >> 4;
-    const int kl = 16 * wf;                     // first feature of this wave, local to the slice arrays
+    const int kl0 = 32 * (w & 1);               // product waves: first of this wave's 32 features, local to the slice arrays
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
     const int n_chunks = (T + C - 1) / C;
     RFA_TICK_INIT();
@@ -269,16 +270,17 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
         wg_sync();
     } else if (grp == 1) {
         half_t* dqb = dq + (int64_t)n * KD + koff;
-        f4 NS[NCT], nz;
-        {
-            const float* sp = final_s + ((int64_t)n * KD + koff + kl + row) * DH + 4 * G;
+        f4 NS[2][NCT], nz[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            const float* sp = final_s + ((int64_t)n * KD + koff + kl0 + 16 * kt + row) * DH + 4 * G;
 #pragma unroll
             for (int ct = 0; ct < NCT; ++ct) {
                 const f4 x = *reinterpret_cast<const f4*>(sp + 16 * ct);
-                NS[ct][0] = -x[0]; NS[ct][1] = -x[1]; NS[ct][2] = -x[2]; NS[ct][3] = -x[3];
+                NS[kt][ct][0] = -x[0]; NS[kt][ct][1] = -x[1]; NS[kt][ct][2] = -x[2]; NS[kt][ct][3] = -x[3];
             }
-            const f4 x = *reinterpret_cast<const f4*>(final_z + (int64_t)n * KD + koff + kl + 4 * G);
-            nz[0] = -x[0]; nz[1] = -x[1]; nz[2] = -x[2]; nz[3] = -x[3];
+            const f4 x = *reinterpret_cast<const f4*>(final_z + (int64_t)n * KD + koff + kl0 + 16 * kt + 4 * G);
+            nz[kt][0] = -x[0]; nz[kt][1] = -x[1]; nz[kt][2] = -x[2]; nz[kt][3] = -x[3];
         }
         const h8 ones = h8_ones();
         // RAGGED: the chunk may have fewer than 64 steps (only the last chunk of the sequence, the
@@ -287,33 +289,46 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
             constexpr bool RAGGED = decltype(ragged_tag)::value;
             const int t0 = (n_chunks - i) * C;
             const Stage st = stage_of(i - 1);
-            // the state one chunk back: -S_prev = -S + K^T V, -z_prev = -z + K^T 1
-            h8 kf[2];        // K column fragments: K[j = 32js + 8G + e][k = kl + i]
+            // the state one chunk back: -S_prev = -S + K^T V, -z_prev = -z + K^T 1.  Every operand
+            // read from LDS serves both feature tiles of the wave.
+            h8 kf[2][2];     // K column fragments: K[j = 32js + 8G + e][k = kl0 + 16kt + i]
 #pragma unroll
-            for (int js = 0; js < 2; ++js) kf[js] = col8(st.Ks, LDK, js * 32, kl, lane);
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int js = 0; js < 2; ++js) kf[kt][js] = col8(st.Ks, LDK, js * 32, kl0 + 16 * kt, lane);
 #pragma unroll
             for (int js = 0; js < 2; ++js) {
+                h8 vc[NCT];
 #pragma unroll
-                for (int ct = 0; ct < NCT; ++ct)
-                    NS[ct] = mfma32(col8(st.Vs, LDV, js * 32, 16 * ct, lane), kf[js], NS[ct]);
-                nz = mfma32(kf[js], ones, nz);
+                for (int ct = 0; ct < NCT; ++ct) vc[ct] = col8(st.Vs, LDV, js * 32, 16 * ct, lane);
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct) NS[kt][ct] = mfma32(vc[ct], kf[kt][js], NS[kt][ct]);
+                    nz[kt] = mfma32(kf[kt][js], ones, nz[kt]);
+                }
             }
             // dQ^T tiles (m = k, n = i)
-            f4 yt[4];       // -(S_prev G^T)
+            f4 yt[2][4];       // -(S_prev G^T)
 #pragma unroll
-            for (int it = 0; it < 4; ++it) yt[it] = f4_zero();
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int it = 0; it < 4; ++it) yt[kt][it] = f4_zero();
 #pragma unroll
             for (int cs = 0; cs < DH / 32; ++cs) {
                 h8 bg[4];
 #pragma unroll
                 for (int it = 0; it < 4; ++it) bg[it] = row_split8(st.Gs, LDV, 16 * it + row, cs * 32, G);
                 __builtin_amdgcn_sched_barrier(0);
-                h8 hi, lo;
-                acc_to_operand(NS[2 * cs], NS[2 * cs + 1], hi, lo);
 #pragma unroll
-                for (int it = 0; it < 4; ++it) {
-                    yt[it] = mfma32(hi, bg[it], yt[it]);
-                    yt[it] = mfma32(lo, bg[it], yt[it]);
+                for (int kt = 0; kt < 2; ++kt) {
+                    h8 hi, lo;
+                    acc_to_operand(NS[kt][2 * cs], NS[kt][2 * cs + 1], hi, lo);
+#pragma unroll
+                    for (int it = 0; it < 4; ++it) {
+                        yt[kt][it] = mfma32(hi, bg[it], yt[kt][it]);
+                        yt[kt][it] = mfma32(lo, bg[it], yt[kt][it]);
+                    }
                 }
             }
             RFA_TICK_AT(11, 256);
@@ -323,13 +338,19 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
             for (int it = 0; it < 4; ++it) {
                 const int ii = 16 * it + row;
                 const float gzi = st.gzs[ii];
-                f4 acc;
+                const h8 p0 = row8(st.Ps, LDA, ii, 0, G);
+                h8 p1 = p0;
+                if (it >= 2) p1 = row8(st.Ps, LDA, ii, 32, G);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[e] = -(yt[it][e] + gzi * nz[e]);
-                acc = mfma32(kf[0], row8(st.Ps, LDA, ii, 0, G), acc);
-                if (it >= 2) acc = mfma32(kf[1], row8(st.Ps, LDA, ii, 32, G), acc);
-                if (!RAGGED || t0 + ii < T)
-                    *reinterpret_cast<h4*>(dqb + (int64_t)(t0 + ii) * k_stride + kl + 4 * G) = to_h4(acc);
+                for (int kt = 0; kt < 2; ++kt) {
+                    f4 acc;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e] = -(yt[kt][it][e] + gzi * nz[kt][e]);
+                    acc = mfma32(kf[kt][0], p0, acc);
+                    if (it >= 2) acc = mfma32(kf[kt][1], p1, acc);
+                    if (!RAGGED || t0 + ii < T)
+                        *reinterpret_cast<h4*>(dqb + (int64_t)(t0 + ii) * k_stride + kl0 + 16 * kt + 4 * G) = to_h4(acc);
+                }
             }
             RFA_TICK_AT(13, 256);
             wg_sync();
@@ -341,24 +362,36 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
         for (int i = 2; i <= n_chunks; ++i) chunk_body(std::false_type{}, i);
     } else {
         half_t* dkb = dk + (int64_t)n * KD + koff;
-        f4 RT[NCT], racc = f4_zero();
+        f4 RT[2][NCT], racc[2];
 #pragma unroll
-        for (int ct = 0; ct < NCT; ++ct) RT[ct] = f4_zero();
+        for (int kt = 0; kt < 2; ++kt) {
+            racc[kt] = f4_zero();
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct) RT[kt][ct] = f4_zero();
+        }
         auto chunk_body = [&](auto ragged_tag, int i) __attribute__((always_inline)) {
             constexpr bool RAGGED = decltype(ragged_tag)::value;
             const int t0 = (n_chunks - i) * C;
             const Stage st = stage_of(i - 1);
             // dK^T tiles (m = k, n = j), then R += G^T Q, r += Q^T gz
-            h8 qf[2];    // Q column fragments: Q[i = 32is + 8G + e][k = kl + lane i]
+            h8 qf[2][2];    // Q column fragments: Q[i = 32is + 8G + e][k = kl0 + 16kt + lane i]
 #pragma unroll
-            for (int is = 0; is < 2; ++is) qf[is] = col8(st.Qs, LDK, is * 32, kl, lane);
-            f4 dkacc[4];
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int is = 0; is < 2; ++is) qf[kt][is] = col8(st.Qs, LDK, is * 32, kl0 + 16 * kt, lane);
+            f4 dkacc[2][4];
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) {
-                f4 acc = racc;
-                if (jt < 2) acc = mfma32(qf[0], col8(st.Ps, LDA, 0, 16 * jt, lane), acc);
-                acc = mfma32(qf[1], col8(st.Ps, LDA, 32, 16 * jt, lane), acc);
-                dkacc[jt] = acc;
+                const h8 pc1 = col8(st.Ps, LDA, 32, 16 * jt, lane);
+                h8 pc0 = pc1;
+                if (jt < 2) pc0 = col8(st.Ps, LDA, 0, 16 * jt, lane);
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+                    f4 acc = racc[kt];
+                    if (jt < 2) acc = mfma32(qf[kt][0], pc0, acc);
+                    acc = mfma32(qf[kt][1], pc1, acc);
+                    dkacc[kt][jt] = acc;
+                }
             }
 #pragma unroll
             for (int cs = 0; cs < DH / 32; ++cs) {
@@ -366,31 +399,41 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) bvv[jt] = row_split8(st.Vs, LDV, 16 * jt + row, cs * 32, G);
                 __builtin_amdgcn_sched_barrier(0);
-                h8 hi, lo;
-                acc_to_operand(RT[2 * cs], RT[2 * cs + 1], hi, lo);
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt) {
-                    dkacc[jt] = mfma32(hi, bvv[jt], dkacc[jt]);
-                    dkacc[jt] = mfma32(lo, bvv[jt], dkacc[jt]);
+                for (int kt = 0; kt < 2; ++kt) {
+                    h8 hi, lo;
+                    acc_to_operand(RT[kt][2 * cs], RT[kt][2 * cs + 1], hi, lo);
+#pragma unroll
+                    for (int jt = 0; jt < 4; ++jt) {
+                        dkacc[kt][jt] = mfma32(hi, bvv[jt], dkacc[kt][jt]);
+                        dkacc[kt][jt] = mfma32(lo, bvv[jt], dkacc[kt][jt]);
+                    }
                 }
             }
             wg_sync();
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) {
                 const int jj = 16 * jt + row;
-                if (!RAGGED || t0 + jj < T)
-                    *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + kl + 4 * G) = to_h4(dkacc[jt]);
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+                    if (!RAGGED || t0 + jj < T)
+                        *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + kl0 + 16 * kt + 4 * G) = to_h4(dkacc[kt][jt]);
             }
 #pragma unroll
             for (int is = 0; is < 2; ++is) {
                 h8 ghi, glo;
                 f8_to_operand(*reinterpret_cast<const f4*>(st.gzs + is * 32 + 8 * G),
                               *reinterpret_cast<const f4*>(st.gzs + is * 32 + 8 * G + 4), ghi, glo);
-                racc = mfma32(qf[is], ghi, racc);
-                racc = mfma32(qf[is], glo, racc);
+                h8 gc[NCT];
 #pragma unroll
-                for (int ct = 0; ct < NCT; ++ct)
-                    RT[ct] = mfma32(col8(st.Gs, LDV, is * 32, 16 * ct, lane), qf[is], RT[ct]);
+                for (int ct = 0; ct < NCT; ++ct) gc[ct] = col8(st.Gs, LDV, is * 32, 16 * ct, lane);
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+                    racc[kt] = mfma32(qf[kt][is], ghi, racc[kt]);
+                    racc[kt] = mfma32(qf[kt][is], glo, racc[kt]);
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct) RT[kt][ct] = mfma32(gc[ct], qf[kt][is], RT[kt][ct]);
+                }
             }
             wg_sync();
         };
@@ -422,10 +465,11 @@ __device__ __forceinline__ void sliced_bwd_dv(
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int grp = w >> 2, wc = w & 3;
+    const int grp = w >> 2, wc = w & 3;         // loader: column block of the A^T tiles
     const int tid = threadIdx.x & (NT - 1);
     const int row = lane & 15, G = lane >> 4;
-    const int cl = 16 * wc;                     // first column of this wave, local to the slice array
+    const int jh = (w >> 1) & 1;                // product waves 4..7: half of the chunk's rows ...
+    const int cl0 = 32 * (w & 1);               // ... and first of this wave's 32 columns, local to the slice array
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
     const int n_chunks = (T + C - 1) / C;
     RFA_TICK_INIT();
@@ -528,28 +572,36 @@ __device__ __forceinline__ void sliced_bwd_dv(
         wg_sync();
         wg_sync();
     } else {
-        const int jh = grp - 1;
         half_t* dvb = dv + (int64_t)n * DH + coff;
-        f4 RR[NKT];
+        f4 RR[2][NKT];
 #pragma unroll
-        for (int kt = 0; kt < NKT; ++kt) RR[kt] = f4_zero();
+        for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt) RR[cc][kt] = f4_zero();
         auto chunk_body = [&](auto ragged_tag, int i) __attribute__((always_inline)) {
             constexpr bool RAGGED = decltype(ragged_tag)::value;
             const int t0 = (n_chunks - i) * C;
             const Stage st = stage_of(i - 1);
-            // dV^T tiles (m = c, n = j) for j tiles 2jh, 2jh + 1, then R += Q^T G^
-            h8 gf[2];     // G^ column fragments: G^[i = 32is + 8G + e][c = cl + lane i]
+            // dV^T tiles (m = c, n = j) for j tiles 2jh, 2jh + 1, then R += Q^T G^; every operand
+            // read from LDS serves both column tiles of the wave
+            h8 gf[2][2];     // G^ column fragments: G^[i = 32is + 8G + e][c = cl0 + 16cc + lane i]
 #pragma unroll
-            for (int is = 0; is < 2; ++is) gf[is] = col8(st.Gs, LDG, is * 32, cl, lane);
-            f4 dvacc[2];
+            for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+                for (int is = 0; is < 2; ++is) gf[cc][is] = col8(st.Gs, LDG, is * 32, cl0 + 16 * cc, lane);
+            f4 dvacc[2][2];
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int jr = 16 * (2 * jh + u) + row;
                 // rows i < 32 of A^T only reach the first two j tiles: their operand is all zero
-                // for the other group, and multiplying by zeros keeps both groups on one code path
-                f4 acc = mfma32(gf[0], row8(st.ATs, LDA, jr, 0, G), f4_zero());
-                acc = mfma32(gf[1], row8(st.ATs, LDA, jr, 32, G), acc);
-                dvacc[u] = acc;
+                // for the other half, and multiplying by zeros keeps both halves on one code path
+                const h8 a0 = row8(st.ATs, LDA, jr, 0, G), a1 = row8(st.ATs, LDA, jr, 32, G);
+#pragma unroll
+                for (int cc = 0; cc < 2; ++cc) {
+                    f4 acc = mfma32(gf[cc][0], a0, f4_zero());
+                    acc = mfma32(gf[cc][1], a1, acc);
+                    dvacc[cc][u] = acc;
+                }
             }
 #pragma unroll
             for (int ks = 0; ks < KD / 32; ++ks) {
@@ -557,12 +609,15 @@ __device__ __forceinline__ void sliced_bwd_dv(
 #pragma unroll
                 for (int u = 0; u < 2; ++u) bkk[u] = row_split8(st.Ks, LDQ, 16 * (2 * jh + u) + row, ks * 32, G);
                 __builtin_amdgcn_sched_barrier(0);
-                h8 hi, lo;
-                acc_to_operand(RR[2 * ks], RR[2 * ks + 1], hi, lo);
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    dvacc[u] = mfma32(hi, bkk[u], dvacc[u]);
-                    dvacc[u] = mfma32(lo, bkk[u], dvacc[u]);
+                for (int cc = 0; cc < 2; ++cc) {
+                    h8 hi, lo;
+                    acc_to_operand(RR[cc][2 * ks], RR[cc][2 * ks + 1], hi, lo);
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        dvacc[cc][u] = mfma32(hi, bkk[u], dvacc[cc][u]);
+                        dvacc[cc][u] = mfma32(lo, bkk[u], dvacc[cc][u]);
+                    }
                 }
             }
             RFA_TICK_AT(11, 256);
@@ -571,14 +626,19 @@ __device__ __forceinline__ void sliced_bwd_dv(
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int jj = 16 * (2 * jh + u) + row;
-                if (!RAGGED || t0 + jj < T)
-                    *reinterpret_cast<h4*>(dvb + (int64_t)(t0 + jj) * v_stride + cl + 4 * G) = to_h4(dvacc[u]);
+#pragma unroll
+                for (int cc = 0; cc < 2; ++cc)
+                    if (!RAGGED || t0 + jj < T)
+                        *reinterpret_cast<h4*>(dvb + (int64_t)(t0 + jj) * v_stride + cl0 + 16 * cc + 4 * G) = to_h4(dvacc[cc][u]);
             }
 #pragma unroll
             for (int is = 0; is < 2; ++is)
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt)
-                    RR[kt] = mfma32(col8(st.Qs, LDQ, is * 32, 16 * kt, lane), gf[is], RR[kt]);
+                for (int kt = 0; kt < NKT; ++kt) {
+                    const h8 qc = col8(st.Qs, LDQ, is * 32, 16 * kt, lane);
+#pragma unroll
+                    for (int cc = 0; cc < 2; ++cc) RR[cc][kt] = mfma32(qc, gf[cc][is], RR[cc][kt]);
+                }
             RFA_TICK_AT(13, 256);
             wg_sync();
             RFA_TICK_AT(14, 256);
