@@ -181,6 +181,19 @@ __device__ __forceinline__ void acc_to_operand(const f4& t0, const f4& t1, h8& h
     }
 }
 
+// Two accumulator tiles as one fp16 operand in the same (split) slot order, rounded to nearest.
+// For products that only *use* a carried fp32 state: the state itself stays fp32 in its
+// accumulator, so the rounding is that of any other fp16 operand and does not build up over steps.
+__device__ __forceinline__ h8 acc_to_operand_rn(const f4& t0, const f4& t1) {
+    h8 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        r[e] = (half_t)t0[e];
+        r[4 + e] = (half_t)t1[e];
+    }
+    return r;
+}
+
 __device__ __forceinline__ h4 to_h4(const f4& x) {
     h4 r;
     r[0] = (half_t)x[0]; r[1] = (half_t)x[1]; r[2] = (half_t)x[2]; r[3] = (half_t)x[3];

@@ -322,13 +322,9 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt) {
-                    h8 hi, lo;
-                    acc_to_operand(NS[kt][2 * cs], NS[kt][2 * cs + 1], hi, lo);
+                    const h8 sh = acc_to_operand_rn(NS[kt][2 * cs], NS[kt][2 * cs + 1]);
 #pragma unroll
-                    for (int it = 0; it < 4; ++it) {
-                        yt[kt][it] = mfma32(hi, bg[it], yt[kt][it]);
-                        yt[kt][it] = mfma32(lo, bg[it], yt[kt][it]);
-                    }
+                    for (int it = 0; it < 4; ++it) yt[kt][it] = mfma32(sh, bg[it], yt[kt][it]);
                 }
             }
             RFA_TICK_AT(11, 256);
@@ -401,13 +397,9 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt) {
-                    h8 hi, lo;
-                    acc_to_operand(RT[kt][2 * cs], RT[kt][2 * cs + 1], hi, lo);
+                    const h8 rh = acc_to_operand_rn(RT[kt][2 * cs], RT[kt][2 * cs + 1]);
 #pragma unroll
-                    for (int jt = 0; jt < 4; ++jt) {
-                        dkacc[kt][jt] = mfma32(hi, bvv[jt], dkacc[kt][jt]);
-                        dkacc[kt][jt] = mfma32(lo, bvv[jt], dkacc[kt][jt]);
-                    }
+                    for (int jt = 0; jt < 4; ++jt) dkacc[kt][jt] = mfma32(rh, bvv[jt], dkacc[kt][jt]);
                 }
             }
             wg_sync();
@@ -611,13 +603,9 @@ __device__ __forceinline__ void sliced_bwd_dv(
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int cc = 0; cc < 2; ++cc) {
-                    h8 hi, lo;
-                    acc_to_operand(RR[cc][2 * ks], RR[cc][2 * ks + 1], hi, lo);
+                    const h8 rh = acc_to_operand_rn(RR[cc][2 * ks], RR[cc][2 * ks + 1]);
 #pragma unroll
-                    for (int u = 0; u < 2; ++u) {
-                        dvacc[cc][u] = mfma32(hi, bkk[u], dvacc[cc][u]);
-                        dvacc[cc][u] = mfma32(lo, bkk[u], dvacc[cc][u]);
-                    }
+                    for (int u = 0; u < 2; ++u) dvacc[cc][u] = mfma32(rh, bkk[u], dvacc[cc][u]);
                 }
             }
             RFA_TICK_AT(11, 256);
