@@ -712,16 +712,13 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
 #pragma unroll
                     for (int i4 = 0; i4 < 4; ++i4) bq[i4] = row_split8(Qs, LDQ, 16 * i4 + row, ks * 32, G);
                     __builtin_amdgcn_sched_barrier(0);
-                    h8 hi[NCT], lo[NCT];
+                    h8 sh[NCT];
 #pragma unroll
-                    for (int ct = 0; ct < NCT; ++ct) acc_to_operand(S[2 * ks][ct], S[2 * ks + 1][ct], hi[ct], lo[ct]);
+                    for (int ct = 0; ct < NCT; ++ct) sh[ct] = acc_to_operand_rn(S[2 * ks][ct], S[2 * ks + 1][ct]);
 #pragma unroll
-                    for (int i4 = 0; i4 < 4; ++i4) {
+                    for (int i4 = 0; i4 < 4; ++i4)
 #pragma unroll
-                        for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(hi[ct], bq[i4], acc[i4][ct]);
-#pragma unroll
-                        for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(lo[ct], bq[i4], acc[i4][ct]);
-                    }
+                        for (int ct = 0; ct < NCT; ++ct) acc[i4][ct] = mfma32(sh[ct], bq[i4], acc[i4][ct]);
                 }
                 RFA_TICK_AT(11, 256);
 #pragma unroll
