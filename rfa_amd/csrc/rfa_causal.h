@@ -401,15 +401,13 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
 #pragma unroll
                 for (int it = 0; it < 4; ++it) bq[it] = row_split8(Qs, LDQ, 16 * it + row, ks * 32, G);
                 __builtin_amdgcn_sched_barrier(0);
-                h8 hi[NCT], lo[NCT];
+                h8 hi[NCT];
 #pragma unroll
-                for (int ct = 0; ct < NCT; ++ct) acc_to_operand(S[2 * ks][ct], S[2 * ks + 1][ct], hi[ct], lo[ct]);
+                for (int ct = 0; ct < NCT; ++ct) hi[ct] = acc_to_operand_rn(S[2 * ks][ct], S[2 * ks + 1][ct]);
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
 #pragma unroll
                     for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = mfma32(hi[ct], bq[it], acc[it][ct]);
-#pragma unroll
-                    for (int ct = 0; ct < NCT; ++ct) acc[it][ct] = mfma32(lo[ct], bq[it], acc[it][ct]);
                 }
             }
             RFA_TICK(7);
@@ -938,15 +936,13 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
 #pragma unroll
                 for (int it = 0; it < 4; ++it) bg[it] = row_split8(Gs, LDV, 16 * it + row, cs * 32, G);
                 __builtin_amdgcn_sched_barrier(0);
-                h8 hi[NKT], lo[NKT];
+                h8 hi[NKT];
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt) acc_to_operand(ST[2 * cs][kt], ST[2 * cs + 1][kt], hi[kt], lo[kt]);
+                for (int kt = 0; kt < NKT; ++kt) hi[kt] = acc_to_operand_rn(ST[2 * cs][kt], ST[2 * cs + 1][kt]);
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
 #pragma unroll
                     for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(hi[kt], bg[it], yt[kt][it]);
-#pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(lo[kt], bg[it], yt[kt][it]);
                 }
             }
             float e2[4] = {0.f, 0.f, 0.f, 0.f};
@@ -1305,15 +1301,13 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
 #pragma unroll
                 for (int it = 0; it < 4; ++it) bg[it] = row_split8(Gs, LDV, 16 * it + row, cs * 32, G);
                 __builtin_amdgcn_sched_barrier(0);
-                h8 hi[NKT], lo[NKT];
+                h8 hi[NKT];
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt) acc_to_operand(ST[2 * cs][kt], ST[2 * cs + 1][kt], hi[kt], lo[kt]);
+                for (int kt = 0; kt < NKT; ++kt) hi[kt] = acc_to_operand_rn(ST[2 * cs][kt], ST[2 * cs + 1][kt]);
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
 #pragma unroll
                     for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(hi[kt], bg[it], yt[kt][it]);
-#pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) yt[kt][it] = mfma32(lo[kt], bg[it], yt[kt][it]);
                 }
             }
         }
@@ -1684,15 +1678,13 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) bvv[jt] = row_split8(Vs, LDV, 16 * jt + row, cs * 32, G);
                 __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
-                h8 hi[NKT], lo[NKT];
+                h8 hi[NKT];
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt) acc_to_operand<CAUSAL>(RT[2 * cs][kt], RT[2 * cs + 1][kt], hi[kt], lo[kt]);
+                for (int kt = 0; kt < NKT; ++kt) hi[kt] = acc_to_operand_rn(RT[2 * cs][kt], RT[2 * cs + 1][kt]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
 #pragma unroll
                     for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(hi[kt], bvv[jt], dkacc[kt][jt]);
-#pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(lo[kt], bvv[jt], dkacc[kt][jt]);
                 }
             }
 #pragma unroll
@@ -1728,15 +1720,13 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) bkk[jt] = row_split8(Ks, LDQ, 16 * jt + row, ks * 32, G);
                 __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
-                h8 hi[NCT2], lo[NCT2];
+                h8 hi[NCT2];
 #pragma unroll
-                for (int ct = 0; ct < NCT2; ++ct) acc_to_operand<CAUSAL>(RR[2 * ks][ct], RR[2 * ks + 1][ct], hi[ct], lo[ct]);
+                for (int ct = 0; ct < NCT2; ++ct) hi[ct] = acc_to_operand_rn(RR[2 * ks][ct], RR[2 * ks + 1][ct]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
 #pragma unroll
                     for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(hi[ct], bkk[jt], dvacc[ct][jt]);
-#pragma unroll
-                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(lo[ct], bkk[jt], dvacc[ct][jt]);
                 }
             }
 #pragma unroll
@@ -1941,15 +1931,13 @@ __device__ __forceinline__ void dkdv_role_dk(
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) bvv[jt] = row_split8(Vs, LDV, 16 * jt + row, cs * 32, G);
                 __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
-                h8 hi[NKT], lo[NKT];
+                h8 hi[NKT];
 #pragma unroll
-                for (int kt = 0; kt < NKT; ++kt) acc_to_operand(RT[2 * cs][kt], RT[2 * cs + 1][kt], hi[kt], lo[kt]);
+                for (int kt = 0; kt < NKT; ++kt) hi[kt] = acc_to_operand_rn(RT[2 * cs][kt], RT[2 * cs + 1][kt]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
 #pragma unroll
                     for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(hi[kt], bvv[jt], dkacc[kt][jt]);
-#pragma unroll
-                    for (int kt = 0; kt < NKT; ++kt) dkacc[kt][jt] = mfma32(lo[kt], bvv[jt], dkacc[kt][jt]);
                 }
             }
 #pragma unroll
@@ -2109,15 +2097,13 @@ __device__ __forceinline__ void dkdv_role_dv(
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) bkk[jt] = row_split8(Ks, LDQ, 16 * jt + row, ks * 32, G);
                 __builtin_amdgcn_sched_barrier(0);     // keep the reads ahead of the conversion
-                h8 hi[NCT2], lo[NCT2];
+                h8 hi[NCT2];
 #pragma unroll
-                for (int ct = 0; ct < NCT2; ++ct) acc_to_operand(RR[2 * ks][ct], RR[2 * ks + 1][ct], hi[ct], lo[ct]);
+                for (int ct = 0; ct < NCT2; ++ct) hi[ct] = acc_to_operand_rn(RR[2 * ks][ct], RR[2 * ks + 1][ct]);
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
 #pragma unroll
                     for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(hi[ct], bkk[jt], dvacc[ct][jt]);
-#pragma unroll
-                    for (int ct = 0; ct < NCT2; ++ct) dvacc[ct][jt] = mfma32(lo[ct], bkk[jt], dvacc[ct][jt]);
                 }
             }
 #pragma unroll

@@ -160,27 +160,6 @@ __device__ __forceinline__ void f8_to_operand(const f4& a, const f4& b, h8& hi, 
     }
 }
 
-// Two fp32 accumulator tiles -> one fp16 operand pair (hi + lo carries ~22 bits),
-// split slot order (see header comment).  MIX = false spells the residual as a plain
-// subtraction (same bits, twice the VALU instructions): the non-causal dK/dV sweep allocates
-// 54 fewer registers with it and runs 3 % faster.
-template <bool MIX = true>
-__device__ __forceinline__ void acc_to_operand(const f4& t0, const f4& t1, h8& hi, h8& lo) {
-    if constexpr (MIX) {
-        f8_to_operand(t0, t1, hi, lo);
-    } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const half_t h0 = (half_t)t0[e];
-            const half_t h1 = (half_t)t1[e];
-            hi[e] = h0;
-            hi[4 + e] = h1;
-            lo[e] = (half_t)(t0[e] - (float)h0);
-            lo[4 + e] = (half_t)(t1[e] - (float)h1);
-        }
-    }
-}
-
 // Two accumulator tiles as one fp16 operand in the same (split) slot order, rounded to nearest.
 // For products that only *use* a carried fp32 state: the state itself stays fp32 in its
 // accumulator, so the rounding is that of any other fp16 operand and does not build up over steps.
