@@ -165,15 +165,21 @@ struct ScanPlan {
 //                    in state slices (rfa_sliced.h), one launch, every chunk read once
 enum SavedLayout { LAYOUT_SEGMENTS = 0, LAYOUT_FINAL = 1 };
 
-bool sliced_supported(int K, int d) { return (K == 64 || K == 128) && d == 64; }
+bool sliced_supported(int K, int d) { return (K == 64 || K == 128) && (d == 64 || d == 128); }
 
-// The sliced backward has N * (K / 64 + d / 64) workgroups that never wait for each other: taken
-// when they cover most of the compute units ("sliced" knob: 0 never, 1 whenever a kernel exists).
+// The sliced backward has N * (K / 64 + d / 64) workgroups that never wait for each other, each
+// walking a whole sequence.  Taken when they cover enough of the compute units ("sliced" knob: 0
+// never, 1 whenever a kernel exists).  Measured against the two time-segmented sweeps at T = 1024:
+// d = 64, K = 128 wins from 120 workgroups on (N = 40: 34.8 vs 37.3 us, N = 64: 34 vs 43, N = 512:
+// 262 vs 285); d = 128 wins with K = 128 at 256 workgroups (60 vs 67 us) and loses with K = 64 at
+// 192 (54 vs 50 us).
 int choose_saved_layout(int64_t N, int K, int d) {
     if (!sliced_supported(K, d)) return LAYOUT_SEGMENTS;
     const int knob = tune::get(tune::SLICED);
     if (knob >= 0) return knob ? LAYOUT_FINAL : LAYOUT_SEGMENTS;
-    return N * (K / rfa::kSliceWidth + d / rfa::kSliceWidth) * 10 >= (int64_t)device_cus() * 6 ? LAYOUT_FINAL : LAYOUT_SEGMENTS;
+    const int64_t wgs = N * (K / rfa::kSliceWidth + d / rfa::kSliceWidth), cus = device_cus();
+    if (d == 64) return wgs * 100 >= cus * 45 ? LAYOUT_FINAL : LAYOUT_SEGMENTS;
+    return K == 128 && wgs * 10 >= cus * 9 ? LAYOUT_FINAL : LAYOUT_SEGMENTS;
 }
 
 // Whether the consumers read one pre-scanned state instead of adding up the segment totals
@@ -458,7 +464,7 @@ int launch_sliced_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa
                            const rfa::half_t* out, rfa::half_t* dq, rfa::half_t* dk, rfa::half_t* dv, int T, int N,
                            const ScanPlan& pf, const int* savedHdr, const float* finalS, const float* finalZ,
                            const float* savedDen, hipStream_t st) {
-    if constexpr (KD <= 128 && DH == 64) {
+    if constexpr (KD <= 128 && DH <= 128) {
         using Cfg = rfa::SlicedBwdCfg<KD, DH>;
         auto kern = rfa::k_sliced_bwd<KD, DH>;
         if (int rc = set_lds(kern, Cfg::kLds)) return rc;

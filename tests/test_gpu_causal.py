@@ -285,7 +285,7 @@ def test_saved_buffer_carries_the_plan_of_its_forward(knobs):
 
 
 SLICED_SHAPES = [
-    # T, B, H, d, D: both feature widths the sliced backward exists for (d = 64), ragged tails, one step, sequence
+    # T, B, H, d, D: the feature and value widths the sliced backward exists for, ragged tails, one step, sequence
     # counts that are no multiple of the 8 XCDs, a long sequence (many backward steps of the state)
     (128, 2, 4, 64, 64),
     (1, 1, 1, 64, 64),
@@ -296,6 +296,10 @@ SLICED_SHAPES = [
     (192, 1, 2, 64, 32),     # K = 64: one feature slice
     (70, 65, 8, 64, 64),     # N = 520
     (4100, 1, 2, 64, 64),    # 65 chunks
+    (200, 2, 3, 128, 64),    # d = 128: two value slices
+    (130, 1, 5, 128, 32),
+    (1, 2, 1, 128, 64),
+    (1100, 1, 2, 128, 64),
 ]
 
 
