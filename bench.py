@@ -28,12 +28,12 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the bench configuration, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
 # passes summarised in profiles/bench_cfg2_hbm_traffic.md (counters scaled on the 512 MiB copy).
 MEASURED_TRAFFIC_BYTES = {
-    "k_segment_state": 25430665,
-    "k_causal_fwd": 61162601,
+    "k_segment_state": 25424532,
+    "k_causal_fwd": 61191361,
     "k_causal_bwd_dq": 92586196,       # the two-sweep backward (tuning knob sliced = 0)
     "k_causal_bwd_dkdv": 86253280,
-    "k_sliced_bwd": 105340904,
-    "k_decode_step": 68884930,
+    "k_sliced_bwd": 105368350,
+    "k_decode_step": 68884833,
 }
 
 
