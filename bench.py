@@ -185,6 +185,7 @@ def main():
         "config": {"workload": "configs[1]: RFA causal self-attention fwd+bwd, seq 1024, batch 8, 8 heads, "
                                "head_dim 64, proj_dim 64 (phi width 128), feature-level boundary RFA.apply",
                    "T": T, "B": B, "H": H, "head_dim": d, "proj_dim": D, "segments": nseg,
+                   "backward": "one launch by state slices" if "k_sliced_bwd" in kern_us else "two sweeps over time segments",
                    "arithmetic": "fp16 operands and outputs, fp32 accumulation and state"},
         "parity": parity, "roofline": roofline, "cpu_baseline": cpu_baseline,
     }
