@@ -191,18 +191,24 @@ def _random_cases(count, seed):
 
 
 @pytest.mark.parametrize("T,B,H,d,D,seed", _random_cases(16, 424242))
-def test_seeded_random_shapes(T, B, H, d, D, seed):
+def test_seeded_random_shapes(T, B, H, d, D, seed, knobs):
     """Sixteen shapes drawn once from a fixed seed (lengths 1..699, 1..3 batch entries and heads, every
-    supported width pair): output, saved-pair and plain-pair gradients against the oracle."""
+    supported width pair): output, saved-pair gradients in both layouts of the saved buffer (time
+    segments; final state with the one-launch backward where it exists) and plain-pair gradients
+    against the oracle."""
     from rfa_amd import rfa_hip
     cpu = _features(T, B, H, d, D, seed)
     pq, pk, v, g = (t.cuda() for t in cpu)
     print(f"causal random T={T} B={B} H={H} d={d} D={D}", flush=True)
     ref = _oracle_fwd(*cpu[:3])
     want = _oracle_bwd(*cpu)
-    out, saved = rfa_hip.forward_save(pq, pk, v)
-    assert (out.float().cpu() - ref).abs().max().item() <= OUT_ATOL
-    for pair in (rfa_hip.backward_saved(pq, pk, v, g, out, saved), rfa_hip.backward(pq, pk, v, g)):
+    pairs = [rfa_hip.backward(pq, pk, v, g)]
+    for sliced in (0, 1):
+        knobs(sliced=sliced)
+        out, saved = rfa_hip.forward_save(pq, pk, v)
+        assert (out.float().cpu() - ref).abs().max().item() <= OUT_ATOL
+        pairs.append(rfa_hip.backward_saved(pq, pk, v, g, out, saved))
+    for pair in pairs:
         for name, a, b in zip(("dq", "dk", "dv"), pair, want):
             assert torch.isfinite(a).all(), name
             assert _rel(a.float().cpu(), b) <= GRAD_RTOL, (name, _rel(a.float().cpu(), b))
