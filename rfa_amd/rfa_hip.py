@@ -615,14 +615,25 @@ _BOUND = ("supported", "feature_map_supported", "selftest_layout", "forward", "b
 _CTYPES_IMPL = {name: globals()[name] for name in _BOUND}
 _active = "ctypes"
 
-try:
-    from . import _rfa_hip_ext as _ext      # built by rfa_amd.build.build_ext
-except ImportError:
-    _ext = None
+_ext = None
+
+
+def _resolve_ext():
+    """Imports the torch binding if it is there.  Retried on every query while it is missing, so a
+    process that imported this package before the binding was built (the build entry point does)
+    finds it afterwards."""
+    global _ext
+    if _ext is None:
+        import importlib
+        try:
+            _ext = importlib.import_module(__package__ + "._rfa_hip_ext")   # built by rfa_amd.build.build_ext
+        except ImportError:
+            _ext = None
+    return _ext
 
 
 def ext_available() -> bool:
-    return _ext is not None
+    return _resolve_ext() is not None
 
 
 def binding() -> str:
@@ -633,7 +644,7 @@ def binding() -> str:
 def use_binding(name: str) -> None:
     global _active
     if name == "ext":
-        if _ext is None:
+        if _resolve_ext() is None:
             raise ImportError("the torch binding _rfa_hip_ext has not been built (python -m rfa_amd.build)")
         impl = {n: getattr(_ext, n) for n in _BOUND}
     elif name == "ctypes":
@@ -646,7 +657,7 @@ def use_binding(name: str) -> None:
 
 def _initial_binding() -> None:
     import os
-    want = os.environ.get("RFA_AMD_BINDING", "ext" if _ext is not None else "ctypes")
+    want = os.environ.get("RFA_AMD_BINDING", "ext" if _resolve_ext() is not None else "ctypes")
     use_binding(want)
 
 

@@ -219,3 +219,34 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "librfa_hip.so"))
     with pytest.raises(ImportError, match="rfa_amd.build"):
         _lib.load()
+
+
+def test_binding_built_after_the_package_was_imported_is_found(tmp_path):
+    """A clean tree has no _rfa_hip_ext.so when the package is first imported (the build entry point
+    imports the package to reach the build recipe).  Once the file is there, ext_available() and
+    use_binding('ext') must find it in the same process."""
+    import os
+    import shutil
+    import subprocess
+    import sys
+    from rfa_amd import build as B
+    if not (os.path.exists(B.EXT_PATH) and os.path.exists(B.LIB_PATH)):
+        pytest.skip("the torch binding has not been built")
+    pkg = tmp_path / "rfa_amd"
+    shutil.copytree(os.path.dirname(B.__file__), pkg,
+                    ignore=shutil.ignore_patterns("_rfa_hip_ext*.so", "__pycache__", "csrc"))
+    code = (
+        "import os, shutil, sys\n"
+        f"sys.path.insert(0, {str(tmp_path)!r})\n"
+        "os.environ.pop('RFA_AMD_BINDING', None)\n"
+        "import rfa_amd\n"
+        "from rfa_amd import rfa_hip\n"
+        f"assert rfa_amd.__file__.startswith({str(tmp_path)!r})\n"
+        "assert not rfa_hip.ext_available() and rfa_hip.binding() == 'ctypes'\n"
+        f"shutil.copy({B.EXT_PATH!r}, os.path.dirname(rfa_amd.__file__))\n"
+        "assert rfa_hip.ext_available()\n"
+        "rfa_hip.use_binding('ext')\n"
+        "assert rfa_hip.binding() == 'ext' and rfa_hip.forward.__module__.endswith('_rfa_hip_ext')\n"
+        "print('found')\n")
+    proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=str(tmp_path))
+    assert proc.returncode == 0 and "found" in proc.stdout, proc.stdout + proc.stderr
