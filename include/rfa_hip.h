@@ -86,7 +86,8 @@ int rfa_causal_forward(const void* q, const void* k, const void* v, void* out, i
  * rfa_causal_forward_workspace_bytes exceed the array return RFA_ERR_WORKSPACE.  All calls on one
  * GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads)
  * race; calls on one stream, one after the other, are fine (nothing in the array has to start
- * at zero: every total the scan reads is written earlier in the same call). */
+ * at zero: every total the scan reads is written earlier in the same call).  The first call on a
+ * device looks the array's address up and sets kernel attributes: make it outside graph capture. */
 size_t rfa_static_scratch_bytes(void);
 int rfa_causal_forward_noalloc(const void* q, const void* k, const void* v, void* out, int64_t T,
                                int64_t N, int K, int d, void* stream);
@@ -128,10 +129,11 @@ int rfa_causal_backward_saved(const void* q, const void* k, const void* v, const
  * wrote it (16 ints: magic, version, layout, K, d, segments, steps per segment, scanned-totals
  * flag, T and N as two ints each, zeros), written on the device by that call.
  * rfa_causal_backward_saved runs with the plan recorded on the host when a forward call of this
- * process last wrote the buffer (whatever the tuning knobs say by then) and returns
- * RFA_ERR_WORKSPACE if that call had another T, N, K or d.  For a buffer this process has no
- * record of, it assumes the current plan and its kernels compare the header with it on the
- * device: on a mismatch dq, dk, dv are filled with NaN rather than computed from totals laid out
+ * process last wrote a buffer at that address (whatever the tuning knobs say by then), provided
+ * that call had this call's T, N, K and d; for any other buffer (a copy, or an address the
+ * caller's allocator has since given to another buffer) it assumes the current plan.  In every
+ * case its kernels compare the header in the buffer with the plan they run, on the device: on a
+ * mismatch dq, dk, dv are filled with NaN rather than computed from totals laid out
  * for another plan.  rfa_causal_backward_saved_workspace_bytes is the workspace that call needs
  * for a given saved buffer (= rfa_causal_backward_workspace_bytes unless the knobs changed since
  * the forward).  rfa_causal_saved_describe copies the 16 header ints to host memory and waits
@@ -150,7 +152,9 @@ int rfa_causal_num_segments(int64_t T, int64_t N, int K, int d);
  *   "free_wg"  workgroups the cross-attention readout and state backward aim for
  *   "project_streaming"  1: rfa_project_feature_map uses its streaming kernel for every shape
  *   "sliced"  1/0: rfa_causal_forward_save writes the final-state layout, whose backward is one
- *             launch that walks whole sequences by state slices (K <= 128, d = 64 only) / the
+ *             launch that walks whole sequences by state slices (K <= 128; taken by itself at
+ *             d = 64 when the slices cover 45 % of the compute units, at d = 128 only with K = 128
+ *             and 90 %) / the
  *             segment-totals layout of the two-sweep backward
  * Initial values come from the environment variables RFA_HIP_<NAME>, read once per process and
  * never on the launch path.  No counterpart in the reference. */

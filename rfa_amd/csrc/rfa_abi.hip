@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <deque>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -238,17 +239,32 @@ rfa::PlanWords plan_words(int64_t T, int64_t N, int K, int d, const ScanPlan& p)
 }
 
 // What the last rfa_causal_forward_save wrote at each saved-buffer address, kept on the host so
-// that the backward call runs with that forward's plan whatever the knobs say by then.  A buffer
-// the table does not know (copied by the caller, written by another process) is taken to follow
-// the current plan; the backward kernels then check the header on the device.
+// that the backward call runs with that forward's plan whatever the knobs say by then.  The table
+// is a hint, never an authority: addresses come back from the caller's allocator for other
+// buffers, so a record may describe a buffer that no longer exists.  The backward kernels always
+// compare the header on the device with the plan they were launched for (NaN gradients on a
+// mismatch); a record of another shape than the call's is dropped and the call falls back to the
+// current plan, like a buffer the table does not know (copied by the caller, written by another
+// process).  The table holds the most recent kRegistryEntries forwards; the oldest go first.
 namespace registry {
+constexpr size_t kRegistryEntries = 4096;
 std::mutex mu;
 std::unordered_map<const void*, rfa::PlanWords> table;
+std::deque<const void*> order;       // addresses in the order they first entered the table
 
 void put(const void* saved, const rfa::PlanWords& w) {
     std::lock_guard<std::mutex> lk(mu);
-    if (table.size() >= 4096) table.clear();
-    table[saved] = w;
+    auto it = table.find(saved);
+    if (it != table.end()) {
+        it->second = w;
+        return;
+    }
+    while (table.size() >= kRegistryEntries && !order.empty()) {
+        table.erase(order.front());
+        order.pop_front();
+    }
+    table.emplace(saved, w);
+    order.push_back(saved);
 }
 
 bool get(const void* saved, rfa::PlanWords* w) {
@@ -257,6 +273,17 @@ bool get(const void* saved, rfa::PlanWords* w) {
     if (it == table.end()) return false;
     *w = it->second;
     return true;
+}
+
+// the address stays in `order`; put() tolerates entries whose record is already gone
+void drop(const void* saved) {
+    std::lock_guard<std::mutex> lk(mu);
+    table.erase(saved);
+}
+
+size_t size() {
+    std::lock_guard<std::mutex> lk(mu);
+    return table.size();
 }
 }  // namespace registry
 
@@ -963,21 +990,18 @@ size_t rfa_causal_saved_state_bytes(int64_t T, int64_t N, int K, int d) {
 }
 
 // The plan a backward call on `saved` runs with: the one recorded when a forward call of this
-// process last wrote that buffer, else the current one.  RFA_ERR_WORKSPACE if the recorded
-// forward had another shape.
-static int saved_plan(const char* fn, const void* saved, int64_t T, int64_t N, int K, int d, ScanPlan* p) {
+// process last wrote a buffer at that address, if that forward had this call's shape; else the
+// current one.  Either way the kernels check the plan against the header in the buffer itself.
+static int saved_plan(const void* saved, int64_t T, int64_t N, int K, int d, ScanPlan* p) {
     rfa::PlanWords w;
     if (saved && registry::get(saved, &w)) {
-        const rfa::PlanWords same = plan_words(T, N, K, d, ScanPlan{w.w[5], w.w[6], w.w[7], w.w[2]});
-        if (memcmp(&w, &same, sizeof(w)) != 0)
-            return fail(RFA_ERR_WORKSPACE,
-                        "%s: the saved buffer was written by a forward call of another shape (T=%lld N=%lld K=%d d=%d), "
-                        "this call has T=%lld N=%lld K=%d d=%d", fn,
-                        (long long)(((int64_t)w.w[9] << 32) | (uint32_t)w.w[8]),
-                        (long long)(((int64_t)w.w[11] << 32) | (uint32_t)w.w[10]), w.w[3], w.w[4], (long long)T,
-                        (long long)N, K, d);
-        *p = ScanPlan{w.w[5], w.w[6], w.w[7], w.w[2]};
-        return RFA_OK;
+        const ScanPlan rec{w.w[5], w.w[6], w.w[7], w.w[2]};
+        const rfa::PlanWords same = plan_words(T, N, K, d, rec);
+        if (memcmp(&w, &same, sizeof(w)) == 0) {
+            *p = rec;
+            return RFA_OK;
+        }
+        registry::drop(saved);      // the address now holds something else
     }
     *p = make_plan(T, N, K, d);
     return RFA_OK;
@@ -986,7 +1010,7 @@ static int saved_plan(const char* fn, const void* saved, int64_t T, int64_t N, i
 size_t rfa_causal_backward_saved_workspace_bytes(const void* saved, int64_t T, int64_t N, int K, int d) {
     if (T <= 0 || N <= 0 || !rfa_shape_supported(K, d)) return 0;
     ScanPlan p;
-    if (saved_plan("rfa_causal_backward_saved_workspace_bytes", saved, T, N, K, d, &p) != RFA_OK) return 0;
+    if (saved_plan(saved, T, N, K, d, &p) != RFA_OK) return 0;
     if (p.layout == LAYOUT_FINAL) return 0;
     return layout_workspace(T, N, K, d, p, true).total;
 }
@@ -1137,7 +1161,7 @@ static int causal_backward_impl(const void* q, const void* k, const void* v, con
     if (have_saved) {
         if (!saved || !aligned16(saved))
             return fail(RFA_ERR_WORKSPACE, "rfa_causal_backward_saved: NULL or misaligned saved-state buffer");
-        if (int rc = saved_plan("rfa_causal_backward_saved", saved, T, N, K, d, &p)) return rc;
+        if (int rc = saved_plan(saved, T, N, K, d, &p)) return rc;
         const SavedLayoutBytes sl = saved_layout(T, N, K, d, p);
         if (saved_bytes < sl.total)
             return fail(RFA_ERR_WORKSPACE, "rfa_causal_backward_saved: saved-state buffer of %zu bytes required, got %zu",

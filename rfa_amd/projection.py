@@ -29,12 +29,14 @@ def linear_param_grads(x2: Tensor, dys: Sequence[Tensor], has_bias: Sequence[boo
 class _ProjectHeads(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x: Tensor, w_feat: Optional[Tensor], scale: float, heads: int, want_phi: Tuple[bool, ...],
-                *params: Optional[Tensor]):
+                grad_mode: bool, *params: Optional[Tensor]):
         n = len(want_phi)
         weights, biases = list(params[0::2]), list(params[1::2])
         wf = None if w_feat is None else w_feat.contiguous()
         # y of a projection that goes through the feature map is only kept for the backward pass
-        keep_y = any(ctx.needs_input_grad)
+        # (needs_input_grad does not see grad mode -- under no_grad it still names the trainable
+        # parameters -- and inside forward() grad mode is always off: the caller passes its own)
+        keep_y = grad_mode and any(ctx.needs_input_grad)
         ys, phis = rfa_hip.project_feature_map(x.contiguous(), [w.contiguous() for w in weights], biases, list(want_phi),
                                                wf, heads, scale, keep_y)
         ctx.scale, ctx.heads, ctx.want_phi = scale, heads, want_phi
@@ -86,7 +88,7 @@ class _ProjectHeads(torch.autograd.Function):
             dx = dx.view(L, B, E)
         if dwf is not None:
             dwf = dwf.to(wf.dtype)
-        return (dx, dwf, None, None, None, *dparams)
+        return (dx, dwf, None, None, None, None, *dparams)
 
 
 def fused_projection_supported(x: Tensor, layers: Sequence[nn.Linear], heads: int,
@@ -120,7 +122,8 @@ def project_heads(x: Tensor, layers: Sequence[nn.Linear], want_phi: Sequence[boo
     params = []
     for layer in layers:
         params += [layer.weight, layer.bias]
-    return _ProjectHeads.apply(x, w_feat, scale, heads, tuple(bool(f) for f in want_phi), *params)
+    return _ProjectHeads.apply(x, w_feat, scale, heads, tuple(bool(f) for f in want_phi), torch.is_grad_enabled(),
+                               *params)
 
 
 class _LinearOut(torch.autograd.Function):

@@ -260,7 +260,7 @@ def test_saved_buffer_carries_the_plan_of_its_forward(knobs):
     """The forward writes its plan into the saved buffer and the library remembers it: a backward
     call runs with that plan whatever the knobs say by then; a buffer the library has no record
     of (here: a copy) whose header differs from the current plan yields NaN gradients, never
-    numbers computed from totals laid out for another plan; another shape is an error."""
+    numbers computed from totals laid out for another plan, and so does a call of another shape."""
     import ctypes
     from rfa_amd import _lib, rfa_hip
     T, B, H, d, D = 700, 1, 3, 64, 64
@@ -285,9 +285,70 @@ def test_saved_buffer_carries_the_plan_of_its_forward(knobs):
     knobs(nseg=4, prefix=0)                     # back on the forward's plan: the copy is as good as the original
     for name, a, b in zip(("dq", "dk", "dv"), rfa_hip.backward_saved(pq, pk, v, g, out, stray), want):
         assert _rel(a.float().cpu(), b) <= GRAD_RTOL, name
-    with pytest.raises(RuntimeError, match="another shape"):      # RfaHipError (ctypes) is a RuntimeError too
-        rfa_hip.backward_saved(pq[:640].contiguous(), pk[:640].contiguous(), v[:640].contiguous(), g[:640].contiguous(),
-                               out[:640].contiguous(), saved)
+    # another shape than the forward's: the record of this address does not apply, the call runs with the current
+    # plan and the kernels find a header written for T = 700
+    grads = rfa_hip.backward_saved(pq[:640].contiguous(), pk[:640].contiguous(), v[:640].contiguous(), g[:640].contiguous(),
+                                   out[:640].contiguous(), saved)
+    assert all(torch.isnan(t.float()).all() for t in grads)
+
+
+def _forward_save_into(saved, pq, pk, v):
+    """rfa_causal_forward_save into a buffer the test owns (the wrappers allocate their own)."""
+    from rfa_amd import _lib
+    lib = _lib.load()
+    T, N, K = pq.shape
+    d = v.shape[2]
+    out = torch.empty_like(v)
+    nbytes = lib.rfa_causal_forward_workspace_bytes(T, N, K, d)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device="cuda")
+    assert lib.rfa_causal_saved_state_bytes(T, N, K, d) <= saved.numel()
+    _lib.check(lib.rfa_causal_forward_save(pq.data_ptr(), pk.data_ptr(), v.data_ptr(), out.data_ptr(), saved.data_ptr(),
+                                           saved.numel(), T, N, K, d, ws.data_ptr(), nbytes,
+                                           torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("stale", ["other_plan", "other_shape"])
+def test_saved_buffer_at_an_address_the_library_has_a_stale_record_of(stale, knobs):
+    """The caller's allocator hands the address of a freed saved buffer to another one.  The library's
+    record of that address then describes a buffer that is gone.  A copy of a saved buffer of
+    another shape placed there gives correct gradients (the record is dropped, the current plan is
+    the copy's plan); one of the same shape and another plan gives NaN (the kernels compare the
+    header in the buffer with the plan they run) -- never numbers read through the wrong layout."""
+    from rfa_amd import rfa_hip
+    T, B, H, d, D = 700, 1, 3, 64, 64
+    cpu = _features(T, B, H, d, D, seed=5300)
+    pq, pk, v, g = (t.cuda() for t in cpu)
+    want = _oracle_bwd(*cpu)
+    nbytes = 1 << 23                               # one size for every buffer, so the allocator reuses the block
+    knobs(nseg=2, prefix=0, sliced=0)
+    if stale == "other_plan":
+        first = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        _forward_save_into(first, pq, pk, v)       # record: address -> (T, N, 2 segments)
+    else:
+        Ts = 300
+        cs = [t.cuda() for t in _features(Ts, B, H, d, D, seed=5301)]
+        first = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        _forward_save_into(first, cs[0], cs[1], cs[2])   # record: address -> (T = 300, ...)
+    address = first.data_ptr()
+    knobs(nseg=4, prefix=0, sliced=0)
+    other = torch.empty(nbytes + 512, dtype=torch.uint8, device="cuda")[:nbytes]    # another block
+    out = _forward_save_into(other, pq, pk, v)     # the buffer whose copy will land on the stale address
+    assert other.data_ptr() != address
+    del first
+    reused = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    if reused.data_ptr() != address:
+        pytest.skip("the allocator did not hand the freed block out again")
+    reused.copy_(other)
+    grads = rfa_hip.backward_saved(pq, pk, v, g, out, reused)
+    if stale == "other_plan":
+        assert all(torch.isnan(t.float()).all() for t in grads)
+        # the address is written by a forward again: the record follows
+        out2 = _forward_save_into(reused, pq, pk, v)
+        grads = rfa_hip.backward_saved(pq, pk, v, g, out2, reused)
+    for name, a, b in zip(("dq", "dk", "dv"), grads, want):
+        assert _rel(a.float().cpu(), b) <= GRAD_RTOL, name
 
 
 SLICED_SHAPES = [

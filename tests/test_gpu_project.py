@@ -87,9 +87,24 @@ def test_projection_without_keeping_y(streaming, knobs):
         lin = torch.nn.Linear(E, H * d).cuda().half()
         lin.weight.data.copy_(w); lin.bias.data.copy_(b)
         layers.append(lin)
-    with torch.no_grad():
-        outs = project_heads(x.cuda(), layers, (True, True, False), H, wf, O.SCALE)
+    # the modules' entry: trainable layers under no_grad must take the keep_y=False launch, and the keeping one
+    # (with the same bits) when a gradient can be asked for
+    seen = []
+    real = rfa_hip.project_feature_map
+
+    def spy(*a, **kw):
+        seen.append(a[7] if len(a) > 7 else kw.get("keep_y", True))
+        return real(*a, **kw)
+    rfa_hip.project_feature_map = spy
+    try:
+        with torch.no_grad():
+            outs = project_heads(x.cuda(), layers, (True, True, False), H, wf, O.SCALE)
+        kept = project_heads(x.cuda(), layers, (True, True, False), H, wf, O.SCALE)
+    finally:
+        rfa_hip.project_feature_map = real
+    assert seen == [False, True] and all(p.requires_grad for lin in layers for p in lin.parameters())
     assert torch.equal(outs[0], phis[0]) and torch.equal(outs[1], phis[1]) and torch.equal(outs[2], ys[2])
+    assert all(torch.equal(a, b) for a, b in zip(outs, kept)) and kept[0].requires_grad
     with pytest.raises(Exception, match="neither y nor phi"):
         from rfa_amd import _lib
         import ctypes

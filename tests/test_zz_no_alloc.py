@@ -34,10 +34,12 @@ def test_noalloc_forward_equals_workspace_forward_on_two_calls_in_a_row():
         got = torch.full_like(v, float("nan"))
         torch.cuda.synchronize()
         before = torch.cuda.memory_stats()["num_alloc_retries"], torch.cuda.memory_allocated()
+        free_before = torch.cuda.mem_get_info()[0]          # the driver's own count: sees a hipMalloc inside the library
         print(f"noalloc forward T={T} N={N} K={K} d={d}", flush=True)
         _lib.check(lib.rfa_causal_forward_noalloc(q.data_ptr(), k.data_ptr(), v.data_ptr(), got.data_ptr(), T, N, K, d, stream))
         torch.cuda.synchronize()
         assert (torch.cuda.memory_stats()["num_alloc_retries"], torch.cuda.memory_allocated()) == before
+        assert torch.cuda.mem_get_info()[0] == free_before
         assert torch.equal(got, want)
         if first:                                          # and against the oracle, once
             ref = O.causal_forward_chunked(q[:, :2].float().cpu(), k[:, :2].float().cpu(), v[:, :2].float().cpu())
@@ -50,3 +52,33 @@ def test_noalloc_forward_equals_workspace_forward_on_two_calls_in_a_row():
     assert rc == -5 and b"static scratch" in lib.rfa_last_error()
     # empty input: nothing to do
     assert lib.rfa_causal_forward_noalloc(None, None, None, None, 0, 4, 128, 64, stream) == 0
+
+
+def test_noalloc_forward_under_graph_capture_replays_the_eager_bits():
+    """The callers the entry point is for: a HIP graph captured after one warm-up call (the first call
+    on a device looks the static array's address up and sets kernel attributes, which must not
+    happen under capture).  Every replay, with eager work and synchronisation in between and new
+    input values in the same tensors, gives the bits of rfa_causal_forward on those values."""
+    from rfa_amd import _lib, rfa_hip
+    lib = _lib.load()
+    T, N, K, d = 1024, 64, 128, 64
+    q, k, v = _inputs(T, N, K, d, 3)
+    got = torch.empty_like(v)
+    _lib.check(lib.rfa_causal_forward_noalloc(q.data_ptr(), k.data_ptr(), v.data_ptr(), got.data_ptr(), T, N, K, d,
+                                              torch.cuda.current_stream().cuda_stream))      # warm-up, outside capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    print("noalloc forward: capture", flush=True)
+    with torch.cuda.graph(graph):
+        _lib.check(lib.rfa_causal_forward_noalloc(q.data_ptr(), k.data_ptr(), v.data_ptr(), got.data_ptr(), T, N, K, d,
+                                                  torch.cuda.current_stream().cuda_stream))
+    for rep in range(3):
+        q2, k2, v2 = _inputs(T, N, K, d, 10 + rep)
+        q.copy_(q2), k.copy_(k2), v.copy_(v2)
+        want = rfa_hip.forward(q, k, v)                    # eager work of the program between replays
+        got.fill_(float("nan"))
+        torch.cuda.synchronize()
+        print(f"noalloc forward: replay {rep}", flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), rep
