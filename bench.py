@@ -25,16 +25,31 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch at the bench configuration, from the rocprofv3 FETCH_SIZE / WRITE_SIZE
-# passes summarised in profiles/bench_cfg2_hbm_traffic.md (counters scaled on the 512 MiB copy).
-MEASURED_TRAFFIC_BYTES = {
-    "k_segment_state": 25424532,
-    "k_causal_fwd": 61191361,
-    "k_causal_bwd_dq": 92586196,       # the two-sweep backward (tuning knob sliced = 0)
-    "k_causal_bwd_dkdv": 86253280,
-    "k_sliced_bwd": 105368350,
-    "k_decode_step": 68884833,
-}
+TRAFFIC_PROFILE = os.path.join("profiles", "bench_cfg2_hbm_traffic.md")
+
+
+def _profile_traffic_bytes(*kernels):
+    """Measured HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE passes, counters scaled on
+    the 512 MiB copy) of the named kernels, summed, read from the table of the tracked profile
+    summary: `rfa::<name><...>` rows, first match per name.  None when a name has no row."""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as fh:
+            rows = [[c.strip() for c in ln.strip().strip("|").split("|")] for ln in fh if ln.startswith("| `rfa::")]
+    except OSError:
+        return None
+    total = 0.0
+    for name in kernels:
+        hit = next((r for r in rows if r[0].strip("`").startswith("rfa::" + name)), None)
+        if hit is None:
+            return None
+        total += float(hit[-1])
+    return int(round(total * 1e6))
+
+
+def _cpu_threads(torch):
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    return cores
 
 
 def _event_time_ms(torch, fn, iters):
@@ -139,7 +154,11 @@ def main():
     achieved = dom_bytes / (kern_us[dominant] * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
+                "traffic": _profile_traffic_bytes({"k_causal_fwd": "k_causal_fwd_pipe<128, 64>",
+                                                   "k_segment_state": "k_segment_state<128, 64, 4, true, false>",
+                                                   "k_sliced_bwd": "k_sliced_bwd<128, 64>"}.get(dominant, dominant + "<")),
+                "traffic_source": TRAFFIC_PROFILE + " (FETCH_SIZE + WRITE_SIZE of this kernel at this shape, a profile run "
+                                  "of this file, not measured in this run)",
                 "bytes_per_launch": dom_bytes, "avg_us": round(kern_us[dominant], 2),
                 "kernels_us": {n_: round(u, 2) for n_, u in kern_us.items()},
                 "step_algorithmic_bytes": 2176 * N * T,
@@ -148,9 +167,7 @@ def main():
     # ---------------------------------------------------------------- CPU baseline (oracle port)
     cpu_baseline = None
     if not args.no_cpu_baseline:
-        cores = os.cpu_count() or 1
-        cores = min(cores, 16)
-        torch.set_num_threads(cores)
+        cores = _cpu_threads(torch)
         bs = B                                                 # the whole batch: about 10 s of CPU work
         sq, sk = pq[:, :bs * H].float().cpu(), pk[:, :bs * H].float().cpu()
         sv, sg = vv[:, :bs * H].float().cpu(), gg[:, :bs * H].float().cpu()
@@ -191,7 +208,10 @@ def main():
     }
 
     if not args.no_extras:
-        result["extras"] = extras(torch, O, lib, _lib, rfa_hip, dev, stream, set(filter(None, args.skip.split(","))))
+        skip = set(filter(None, args.skip.split(",")))
+        if args.no_cpu_baseline:
+            skip.add("cpu")
+        result["extras"] = extras(torch, O, lib, _lib, rfa_hip, dev, stream, skip)
     print(json.dumps(result))
 
 
@@ -255,6 +275,35 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream, skip=()):
     want, _, _ = O.causal_forward_loop(fq, fk, vs[:8, :1, :2].float().cpu().reshape(8, 2, d),
                                        s0[:1, :2].cpu().reshape(2, K, d), z0[:1, :2].cpu().reshape(2, K))
     ex["decode"]["parity_max_abs"] = (outs[:8, :1, :2].float().cpu().reshape(8, 2, d) - want).abs().max().item()
+    dec_gbs = ex["decode"]["hbm_gbs"]
+    ex["decode"]["roofline"] = {"bound": "hbm", "kernel": "k_decode_step", "achieved": dec_gbs, "peak": HBM_PEAK_GBS,
+                                "unit": "GB/s", "frac": round(dec_gbs / HBM_PEAK_GBS, 4),
+                                "traffic": _profile_traffic_bytes("k_decode_step<128, 64, true>"),
+                                "traffic_source": TRAFFIC_PROFILE, "bytes_per_launch": step_bytes}
+    if "cpu" not in skip:
+        # the reference's decode loop (causal_attention.py:42-50) with its feature map, fp32 torch-CPU, whole batch,
+        # from the same prefilled state, on the first rows of the run
+        cores = _cpu_threads(torch)
+        n_cpu = 48
+        Wf = W.float().cpu()
+        cq_, ck_, cv_ = (t[:n_cpu].float().cpu() for t in (qs, ks, vs))
+        cs_, cz_ = s0.cpu().reshape(N, K, d).clone(), z0.cpu().reshape(N, K).clone()
+
+        def cpu_decode(steps_):
+            s_, z_ = cs_, cz_
+            for t in range(steps_):
+                fq_ = O.random_project(cq_[t:t + 1], Wf).reshape(N, K)
+                fk_ = O.random_project(ck_[t:t + 1], Wf).reshape(N, K)
+                _, s_, z_ = O.incremental_step(fq_, fk_, cv_[t].reshape(N, d), s_, z_)
+        cpu_decode(4)
+        t0 = time.perf_counter()
+        cpu_decode(n_cpu)
+        tcpu = (time.perf_counter() - t0) / n_cpu
+        ex["decode"]["cpu_baseline"] = {
+            "value": round(B / tcpu, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{n_cpu} of the {steps} steps (the first ones, whole batch of {B} x {H} heads) after 4 warm-up steps: "
+                      "feature maps of q, k and the loop-form step (causal_attention.py:42-50) in fp32 torch-CPU",
+            "us_per_step": round(1e6 * tcpu, 1), "speedup": round(ex["decode"]["tokens_per_s"] / (B / tcpu), 1)}
     del qs, ks, vs, outs
     if "decode_module" not in skip:
         # (3) through the API the reference exposes: one CausalAttention.forward(x[1], W, saved_state=state)
@@ -357,6 +406,35 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream, skip=()):
                                 "algorithmic_bytes": cross_bytes,
                                 "mfma_frac_of_2500_tflops": round(flops / (ms * 1e-3) / 1e12 / 2500.0, 4)}}
 
+    if "cpu" not in skip:
+        # the reference's einsum formulas (cross_attention.py:97-104, 266-269) and their closed-form gradients in fp32
+        # torch-CPU on the whole configuration
+        cores = _cpu_threads(torch)
+        cpk, cpq, cv_, cgo = (t.float().cpu() for t in (pk, pq, v, go))
+        cmask = pad.bool().cpu().t().contiguous()        # [S, B], True = pad
+
+        def cpu_cross():
+            s_, z_ = O.cross_state(cpk, cv_, cmask)
+            O.cross_readout(cpq, s_, z_)
+            _, ds_, dz_ = O.cross_readout_backward(cpq, s_, z_, cgo)
+            O.cross_state_backward(cpk, cv_, ds_, dz_, cmask)
+        cpu_cross()
+        ctimes = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            cpu_cross()
+            ctimes.append(time.perf_counter() - t0)
+        tcpu = min(ctimes)
+        ex["cross"]["cpu_baseline"] = {
+            "value": round(B * Tt / tcpu, 1), "unit": "tgt tokens/s", "cores": cores, "kind": "port",
+            "sample": "the whole configuration (32 x 8 sequences), state + readout + both backward formulas in fp32 "
+                      "torch-CPU, 1 warm-up, best of 3",
+            "ms_per_step": round(1e3 * tcpu, 2), "speedup": round(ex["cross"]["tgt_tokens_per_s"] / (B * Tt / tcpu), 1)}
+    ex["cross"]["roofline"]["traffic"] = _profile_traffic_bytes(
+        "k_segment_state<128, 64, 4, false, true>", "k_causal_fwd<128, 64, 4, false>", "k_causal_bwd_dq<128, 64, 8, false>",
+        "k_causal_bwd_dkdv<128, 64, 4, false, false>")
+    ex["cross"]["roofline"]["traffic_source"] = TRAFFIC_PROFILE + " (sum of the four kernels)"
+
     # ---- long-context causal fwd+bwd (config 5): seq 16384, batch 2, 16 heads, head_dim 128, proj_dim 128
     T5, B5, H5, d5, D5 = 16384, 2, 16, 128, 128
     N5, K5 = B5 * H5, 2 * D5
@@ -386,8 +464,12 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream, skip=()):
     ms = _event_time_ms(torch, long_step, 20)
     ns = 2                                                  # parity on two sequences (chunked-exact oracle)
     sl = lambda t: t[:, :ns].float().cpu()
-    ref5 = O.causal_forward_chunked(sl(pq5), sl(pk5), sl(v5))
-    rq5, rk5, rv5 = O.causal_backward_chunked(sl(pq5), sl(pk5), sl(v5), sl(go5))
+    cores = _cpu_threads(torch)
+    c5 = [sl(t) for t in (pq5, pk5, v5, go5)]
+    t0 = time.perf_counter()
+    ref5 = O.causal_forward_chunked(*c5[:3])
+    rq5, rk5, rv5 = O.causal_backward_chunked(*c5)
+    tcpu5 = time.perf_counter() - t0
     rel = lambda a, b: ((a - b).norm() / b.norm()).item()
     bytes5 = (2 * K5 * 2 + 2 * d5 * 2 + 2 * K5 * 2 + 2 * d5 * 2 + 2 * K5 * 2 + d5 * 2) * N5 * T5   # 4352 B per (head, token)
     ex["long_context"] = {"workload": "configs[4]: seq 16384, batch 2, 16 heads, head_dim 128, proj_dim 128 (phi width 256), "
@@ -396,6 +478,18 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream, skip=()):
                           "algorithmic_bytes": bytes5, "frac_of_hbm": round(bytes5 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                           "parity": {"out_max_abs": (sl(o5) - ref5).abs().max().item(), "dq_rel": rel(sl(dq5), rq5),
                                      "dk_rel": rel(sl(dk5), rk5), "dv_rel": rel(sl(dv5), rv5)}}
+    gbs5 = bytes5 / (ms * 1e-3) / 1e9
+    ex["long_context"]["roofline"] = {
+        "bound": "hbm", "achieved": round(gbs5, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs5 / HBM_PEAK_GBS, 4),
+        "traffic": _profile_traffic_bytes("k_segment_state<256, 128, 8, true, false>", "k_totals_scan<false>",
+                                          "k_causal_fwd<256, 128, 8, true>", "k_causal_bwd_dq_saved<128, 128, 8, 8, 256>",
+                                          "k_totals_scan<true>", "k_causal_bwd_dkdv_roles<256, 128, 8>"),
+        "traffic_source": TRAFFIC_PROFILE + " (sum of the step's kernels)", "bytes_per_step": bytes5}
+    ex["long_context"]["cpu_baseline"] = {
+        "value": round(ns * T5 / H5 / tcpu5, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+        "sample": f"{ns} of the {N5} sequences (T={T5}), forward + backward in the oracle's chunked form (the cumulative-sum "
+                  "form would need 64 GiB) in fp32 torch-CPU, one run (the parity check of this section)",
+        "seconds": round(tcpu5, 2), "speedup": round(ex["long_context"]["tokens_per_s"] / (ns * T5 / H5 / tcpu5), 1)}
     del pq5, pk5, v5, go5, o5, dq5, dk5, dv5, ws5, sv5
 
     # ---- feature map (config 2 shape): phi forward + backward for q
