@@ -176,6 +176,8 @@ bool sliced_supported(int K, int d) { return (K == 64 || K == 128) && (d == 64 |
 // 192 (54 vs 50 us).
 int choose_saved_layout(int64_t N, int K, int d) {
     if (!sliced_supported(K, d)) return LAYOUT_SEGMENTS;
+    // its loader addresses the 64 rows of a chunk with 32-bit byte offsets
+    if ((int64_t)rfa::kChunk * N * (K > d ? K : d) * 2 >= ((int64_t)1 << 32)) return LAYOUT_SEGMENTS;
     const int knob = tune::get(tune::SLICED);
     if (knob >= 0) return knob ? LAYOUT_FINAL : LAYOUT_SEGMENTS;
     const int64_t wgs = N * (K / rfa::kSliceWidth + d / rfa::kSliceWidth), cus = device_cus();
@@ -493,10 +495,13 @@ int launch_sliced_backward(const rfa::half_t* q, const rfa::half_t* k, const rfa
                            const float* savedDen, hipStream_t st) {
     if constexpr (KD <= 128 && DH <= 128) {
         using Cfg = rfa::SlicedBwdCfg<KD, DH>;
-        auto kern = rfa::k_sliced_bwd<KD, DH>;
+        auto kern = rfa::k_sliced_bwd<KD, DH, rfa::kSliceWidth>;
         if (int rc = set_lds(kern, Cfg::kLds)) return rc;
+        // the loader group addresses the 64 rows of a chunk with 32-bit byte offsets
+        if ((int64_t)rfa::kChunk * N * (KD > DH ? KD : DH) * 2 >= ((int64_t)1 << 32))
+            return fail(RFA_ERR_BAD_SHAPE, "sliced backward: 64 time steps of a tensor span 4 GiB or more (N=%d)", N);
         const int64_t grid = (int64_t)rfa::kXcds * ((N + rfa::kXcds - 1) / rfa::kXcds) * (Cfg::NA + Cfg::NB);
-        RFA_LAUNCH(CAUSAL_BWD_SLICED, kern, dim3((unsigned)grid), dim3(rfa::kSlicedThreads), Cfg::kLds, st, q, k, v, g, out,
+        RFA_LAUNCH(CAUSAL_BWD_SLICED, kern, dim3((unsigned)grid), dim3(Cfg::kThreads), Cfg::kLds, st, q, k, v, g, out,
                    savedDen, finalS, finalZ, dq, dk, dv, T, N, savedHdr, plan_words(T, N, KD, DH, pf));
         RFA_HIP_TRY(hipGetLastError());
         return RFA_OK;
@@ -960,6 +965,13 @@ size_t rfa_causal_backward_workspace_bytes(int64_t T, int64_t N, int K, int d) {
     return layout_workspace(T, N, K, d, make_plan(T, N, K, d), true).total;
 }
 
+// RFA_ONLY_KD=<K>,<d> (a development build: python -m rfa_amd.build --only K,d): kernels of one
+// shape only, every other shape falls through to RFA_ERR_UNSUPPORTED; compiles in a fraction of
+// the time.  Never defined in the library the package ships.
+#ifdef RFA_ONLY_K
+#define RFA_DISPATCH_KD(K, d, CALL) \
+    if (K == RFA_ONLY_K && d == RFA_ONLY_D) { return CALL(RFA_ONLY_K, RFA_ONLY_D); }
+#else
 #define RFA_DISPATCH_KD(K, d, CALL)                                   \
     if (K == 64 && d == 64) { return CALL(64, 64); }                  \
     if (K == 128 && d == 64) { return CALL(128, 64); }                \
@@ -967,6 +979,7 @@ size_t rfa_causal_backward_workspace_bytes(int64_t T, int64_t N, int K, int d) {
     if (K == 64 && d == 128) { return CALL(64, 128); }                \
     if (K == 128 && d == 128) { return CALL(128, 128); }              \
     if (K == 256 && d == 128) { return CALL(256, 128); }
+#endif
 
 // The saved buffer: a 256-byte header (rfa::PlanWords: the plan of the forward that wrote the
 // buffer), then S and z -- the segment totals (S in fragment order) or, with LAYOUT_FINAL, the

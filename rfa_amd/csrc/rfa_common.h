@@ -14,6 +14,7 @@
 //                         slots 4..7 <-> m = 4G+e of tile t+1;
 //     the other operand is then read with the same slot order (row_split8).
 #pragma once
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -173,6 +174,14 @@ __device__ __forceinline__ h8 acc_to_operand_rn(const f4& t0, const f4& t1) {
     return r;
 }
 
+// two floats rounded to nearest into one register of two halves (a in the low half)
+__device__ __forceinline__ unsigned pack_h2(float a, float b) {
+    typedef _Float16 hh2 __attribute__((ext_vector_type(2)));
+    hh2 r;
+    r[0] = (half_t)a; r[1] = (half_t)b;
+    return __builtin_bit_cast(unsigned, r);
+}
+
 __device__ __forceinline__ h4 to_h4(const f4& x) {
     h4 r;
     r[0] = (half_t)x[0]; r[1] = (half_t)x[1]; r[2] = (half_t)x[2]; r[3] = (half_t)x[3];
@@ -316,6 +325,62 @@ __device__ __forceinline__ void chunk_r2s(const ChunkRegs<F, NT>& r, half_t* Xs,
     }
 }
 
+// 1 / x for x >= 1 (denominators): the hardware approximation and one Newton step, 3 vector
+// instructions where the correctly rounded quotient takes about ten; the result differs from
+// it by at most one unit in the last place, far below the fp16 rounding of whatever it scales.
+__device__ __forceinline__ float rcp_nr(float x) {
+    const float y = __builtin_amdgcn_rcpf(x);
+    return __builtin_fmaf(__builtin_fmaf(-x, y, 1.0f), y, y);
+}
+
+// Eight halves times one fp32 factor, each product formed in fp32 and rounded once to fp16:
+// the mixed-precision multiply-add reads the half in place and writes the rounded half, one
+// instruction per element (convert, multiply, convert and pack take 2.5).
+__device__ __forceinline__ uint4 scale_h8(uint4 x, float f) {
+    uint4 y;
+    const unsigned in[4] = {x.x, x.y, x.z, x.w};
+    unsigned out[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        unsigned r;
+        asm("v_fma_mixlo_f16 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(in[i]), "v"(f));
+        asm("v_fma_mixhi_f16 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(r) : "v"(in[i]), "v"(f));
+        out[i] = r;
+    }
+    y.x = out[0]; y.y = out[1]; y.z = out[2]; y.w = out[3];
+    return y;
+}
+
+// dot product of two rows of eight halves, accumulated in fp32 (v_dot2_f32_f16: 4 instructions)
+__device__ __forceinline__ float dot_h8(uint4 a, uint4 b) {
+    typedef _Float16 hh2 __attribute__((ext_vector_type(2)));
+    const unsigned ua[4] = {a.x, a.y, a.z, a.w}, ub[4] = {b.x, b.y, b.z, b.w};
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(hh2, ua[i]), __builtin_bit_cast(hh2, ub[i]), acc, false);
+    return acc;
+}
+
+// Sum of x over groups of W adjacent lanes (W = 4, 8 or 16, groups aligned to W), result in every
+// lane of the group: data-parallel-primitive moves inside the vector unit (quad permutes, then the
+// mirror of a half row / of a row, which for lanes that already hold their quad's / half row's
+// sum fetches the other one), no trip through the LDS crossbar.  Same pairing of the additions
+// as a butterfly over lane ^ 1, ^ 2, ^ 4, ^ 8.
+template <int W>
+__device__ __forceinline__ float sum_adjacent(float x) {
+    static_assert(W == 4 || W == 8 || W == 16, "group width");
+    auto dpp = [](float v, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value,
+                                                                     0xf, 0xf, true));
+    };
+    x += dpp(x, std::integral_constant<int, 0xB1>{});                       // quad_perm [1, 0, 3, 2]
+    x += dpp(x, std::integral_constant<int, 0x4E>{});                       // quad_perm [2, 3, 0, 1]
+    if constexpr (W >= 8) x += dpp(x, std::integral_constant<int, 0x141>{});    // row_half_mirror
+    if constexpr (W >= 16) x += dpp(x, std::integral_constant<int, 0x140>{});   // row_mirror
+    return x;
+}
+
 // same, each row multiplied by scale[piece] (fp32) before the store
 template <int F, int NT = kThreads>
 __device__ __forceinline__ void chunk_r2s_scaled(const ChunkRegs<F, NT>& r, const float* scale,
@@ -326,12 +391,7 @@ __device__ __forceinline__ void chunk_r2s_scaled(const ChunkRegs<F, NT>& r, cons
         const int p = tid + NT * it;
         const int row = p / PPR, c8 = p % PPR;
         const float sc = row < r.rows ? scale[it] : 0.f;
-        union { uint4 u; h8 h; } x;
-        x.u = r.v[it];
-        h8 y;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)x.h[e] * sc);
-        *reinterpret_cast<h8*>(Xs + row * ld + c8 * 8) = y;
+        *reinterpret_cast<uint4*>(Xs + row * ld + c8 * 8) = scale_h8(r.v[it], sc);
     }
 }
 

@@ -26,12 +26,17 @@
 //     dK = P^T Q + V R_next^T + 1 r_next^T     (R_next, r_next: sums over later chunks)
 //     dV = A^T G^ + K R_next
 //
-// A workgroup is a pipeline of 12 waves, three per SIMD.  Waves 0-3 (loader group) bring chunk c
-// from HBM into LDS and form its masked tile matrix (P or A^T); waves 4-7 and 8-11 work on chunk
-// c + 1 (the one staged an iteration earlier): dQ and dK in the feature-slice role, the two
-// halves of the dV rows in the value-slice role.  The groups meet at two workgroup barriers per
-// chunk; the chunk arrays and the tile matrix are double buffered.  Only the loader group issues
-// loads and only the others issue stores, so neither kind waits for the other.
+// A workgroup is a pipeline of 8 waves, two per SIMD.  Waves 0-3 (loader group) bring chunk c from
+// HBM into LDS and form its masked tile matrix (P or A^T); waves 4-7 work on chunk c + 1 (the one
+// staged an iteration earlier), each on 32 features or 32 value columns: waves 4, 5 dQ and waves
+// 6, 7 dK in the feature-slice role, the two halves of the dV rows in the value-slice role.  The
+// groups meet at two workgroup barriers per chunk; the chunk arrays and the tile matrix are
+// double buffered.  Only the loader group issues loads and only the others issue stores, so
+// neither kind waits for the other.  What bounds the kernel is instruction issue and dependent
+// latency with two waves per SIMD, not bytes: the loader's per-element work (row scaling, row
+// dot products, masks) is therefore written with the fewest vector instructions that give the
+// same rounding (mixed-precision multiply-add, two-element dot products, lane permutes inside
+// the vector unit), and addresses are a wave-uniform base plus one 32-bit offset per lane.
 #pragma once
 #include <type_traits>
 
@@ -51,44 +56,63 @@ __device__ __forceinline__ void seq_role_of_block(int b, int wps, int& n, int& r
     n = kXcds * (l / wps) + xcd;
 }
 
-template <int KD, int DH>
+// threads per workgroup for feature slices of SW: the loader group and SW / 32 product waves each for dQ and dK
+constexpr int sliced_threads(int SW) { return 256 + 64 * 2 * (SW / 32); }
+
+template <int KD, int DH, int SW = kSliceWidth>
 struct SlicedBwdCfg {
-    static constexpr int C = kChunk, KSL = kSliceWidth, CSL = kSliceWidth;
+    static_assert(SW % 64 == 0 && KD % SW == 0, "feature slice width");
+    static constexpr int C = kChunk, KSL = SW, CSL = kSliceWidth;
     static constexpr int NA = KD / KSL;             // dQ/dK workgroups per sequence
     static constexpr int NB = DH / CSL;             // dV workgroups per sequence
-    static constexpr int LDS_ = KSL + lds_pad(KSL); // row stride of a 64-wide slice array
+    static constexpr int NPW = KSL / 32;            // product waves per output (dQ, dK) of the feature-slice role
+    static constexpr int kThreads = sliced_threads(SW);   // >= the 512 of the dV role
+    static constexpr int LDS_ = KSL + lds_pad(KSL); // row stride of a feature-slice array
+    static constexpr int LDG_ = CSL + lds_pad(CSL); // row stride of a value-slice array
     static constexpr int LDQ = KD + lds_pad(KD);
     static constexpr int LDV = DH + lds_pad(DH);
     static constexpr int LDA = C + 8;
     // dQ/dK role, per stage: Q slice | K slice | V | G^ | P | gz
     static constexpr size_t kStageA = (size_t)(2 * C * LDS_ + 2 * C * LDV + C * LDA) * 2 + C * 4;
     // dV role, per stage: Q | K | G^ slice | A^T
-    static constexpr size_t kStageB = (size_t)(2 * C * LDQ + C * LDS_ + C * LDA) * 2;
+    static constexpr size_t kStageB = (size_t)(2 * C * LDQ + C * LDG_ + C * LDA) * 2;
     static constexpr size_t kLds = 2 * (kStageA > kStageB ? kStageA : kStageB);
     static_assert(kStageA % 16 == 0 && kStageB % 16 == 0, "stage alignment");
 };
 
 __device__ __forceinline__ void wg_sync() { __syncthreads(); }
 
-// 64 rows x F halves of a full chunk: thread-private row pointers (set up once) plus the
-// chunk's offset; no clamping, no address arithmetic beyond one 64-bit add per piece
+// store through a wave-uniform base (scalar registers, scalar address arithmetic) plus one 32-bit
+// byte offset per lane that is set up once: no vector arithmetic per store
+template <typename V>
+__device__ __forceinline__ void store_lane(half_t* uniform_base, unsigned lane_off_bytes, const V& value) {
+    *reinterpret_cast<V*>(reinterpret_cast<char*>(uniform_base) + lane_off_bytes) = value;
+}
+
+// 64 rows x F halves of a full chunk.  The address of a piece is a base that is the same for the
+// whole wave (tensor + sequence + chunk + piece index * rows per pass: scalar registers and scalar
+// arithmetic) plus one 32-bit byte offset per lane, set up once: a load costs no vector
+// arithmetic and the row addresses take one register per tensor.  64 rows of a tensor must span
+// less than 4 GiB (the launcher checks).
 template <int F>
 struct RowPtrs {
     static constexpr int kPieces = ChunkRegs<F, kGroupThreads>::kPieces;
-    const half_t* p[kPieces];
-    __device__ __forceinline__ void init(const half_t* base, int64_t row_stride, int tid) {
-        constexpr int PPR = F / 8;
-#pragma unroll
-        for (int it = 0; it < kPieces; ++it) {
-            const int pc = tid + kGroupThreads * it;
-            p[it] = base + (int64_t)(pc / PPR) * row_stride + (pc % PPR) * 8;
-        }
+    static constexpr int PPR = F / 8;                       // 16-byte pieces per row
+    static constexpr int kRowsPerPass = kGroupThreads / PPR;
+    const char* base;       // wave-uniform
+    int64_t pass_bytes;     // wave-uniform: kRowsPerPass rows
+    unsigned lane_off;
+    __device__ __forceinline__ void init(const half_t* tensor, int64_t row_stride, int tid) {
+        base = reinterpret_cast<const char*>(tensor);
+        pass_bytes = (int64_t)kRowsPerPass * row_stride * 2;
+        lane_off = (unsigned)(tid / PPR) * (unsigned)(row_stride * 2) + (unsigned)(tid % PPR) * 16u;
     }
     __device__ __forceinline__ void load_full(ChunkRegs<F, kGroupThreads>& r, int64_t chunk_off) const {
         r.rows = kChunk;
+        const char* b = base + chunk_off * 2;
 #pragma unroll
         for (int it = 0; it < kPieces; ++it) {
-            r.v[it] = *reinterpret_cast<const uint4*>(p[it] + chunk_off);
+            r.v[it] = *reinterpret_cast<const uint4*>(b + it * pass_bytes + lane_off);
             r.drop[it] = 0;
         }
     }
@@ -102,26 +126,28 @@ struct RowPtrs {
 //             carried negated so that the MFMA can step them backwards by adding K^T V.
 //   dK group: same features; RT[ct] = R^T tile, r as a tile.
 // ---------------------------------------------------------------------------
-template <int KD, int DH>
+template <int KD, int DH, int SW>
 __device__ __forceinline__ void sliced_bwd_dqdk(
     unsigned char* smem, int n, int koff, const half_t* __restrict__ q, const half_t* __restrict__ k,
     const half_t* __restrict__ v, const half_t* __restrict__ g, const half_t* __restrict__ o,
     const float* __restrict__ den_raw, half_t* __restrict__ dq, half_t* __restrict__ dk,
     const float* __restrict__ final_s, const float* __restrict__ final_z, int T, int N) {
-    using Cfg = SlicedBwdCfg<KD, DH>;
-    constexpr int NT = kGroupThreads, C = Cfg::C, KSL = Cfg::KSL;
+    using Cfg = SlicedBwdCfg<KD, DH, SW>;
+    constexpr int NT = kGroupThreads, C = Cfg::C, KSL = Cfg::KSL, NPW = Cfg::NPW;
     constexpr int LDK = Cfg::LDS_, LDV = Cfg::LDV, LDA = Cfg::LDA;
+    constexpr int kDqTick = 256, kDkTick = 256 + 64 * NPW;     // first thread of the dQ / dK waves
     constexpr int NCT = DH / 16;
     constexpr int PPR = DH / 8, VP = ChunkRegs<DH, NT>::kPieces;
     constexpr size_t kStage = Cfg::kLds / 2;
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int grp = w < 4 ? 0 : 1 + ((w - 4) >> 1);     // loader | dQ waves 4, 5 | dK waves 6, 7
+    const int grp = w < 4 ? 0 : 1 + (w - 4) / NPW;      // loader | NPW dQ waves | NPW dK waves
     const int wf = w & 3;                       // loader: row block of the P tiles
     const int tid = threadIdx.x & (NT - 1);     // thread inside the loader group
     const int row = lane & 15, G = lane >> 4;
-    const int kl0 = 32 * (w & 1);               // product waves: first of this wave's 32 features, local to the slice arrays
+    const int kl0 = 32 * ((w - 4) % NPW);       // product waves: first of this wave's 32 features, local to the slice arrays
+    const unsigned out_lane_off = (unsigned)row * (unsigned)(N * KD * 2) + 8u * G;   // bytes: row `row` of a 16-step tile, 4 halves from 4G
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
     const int n_chunks = (T + C - 1) / C;
     RFA_TICK_INIT();
@@ -162,6 +188,15 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
             float dn[VP];
         };
         RowSet s0, s1;
+        // which halves of this lane's P elements lie on or below the diagonal: element (i = 16wf + row,
+        // j = 16jt + 4G + e) is kept when j <= i
+        uint2 tril_mask[4];
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt) {
+            auto keep = [&](int e) { return (16 * jt + 4 * G + e <= 16 * wf + row) ? 0xffffu : 0u; };
+            tril_mask[jt].x = keep(0) | (keep(1) << 16);
+            tril_mask[jt].y = keep(2) | (keep(3) << 16);
+        }
         // the last chunk of the sequence may be short: clamped row addresses
         auto prefetch_ragged = [&](RowSet& r, int c) __attribute__((always_inline)) {
             const int t0 = c * C, rows = T - t0;
@@ -199,21 +234,11 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
             for (int it = 0; it < VP; ++it) {
                 const int pc = tid + NT * it;
                 const int r_ = pc / PPR, c8 = pc % PPR;
-                union { uint4 u; h8 h; } xg, xo;
-                xg.u = r.rg.v[it];
-                xo.u = r.ro.v[it];
-                float dot = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) dot += (float)xg.h[e] * (float)xo.h[e];
-#pragma unroll
-                for (int m = 1; m < PPR; m <<= 1) dot += __shfl_xor(dot, m, 64);
+                const float dot = sum_adjacent<PPR>(dot_h8(r.rg.v[it], r.ro.v[it]));
                 const bool valid = r_ < r.rg.rows;
-                const float inv = valid ? 1.0f / fmaxf(r.dn[it], 1.0f) : 0.f;
+                const float inv = valid ? rcp_nr(fmaxf(r.dn[it], 1.0f)) : 0.f;
                 const float gzv = (valid && r.dn[it] > 1.0f) ? -dot * inv : 0.f;
-                h8 y;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)xg.h[e] * inv);
-                *reinterpret_cast<h8*>(st.Gs + r_ * LDV + c8 * 8) = y;
+                *reinterpret_cast<uint4*>(st.Gs + r_ * LDV + c8 * 8) = scale_h8(r.rg.v[it], inv);
                 if (c8 == 0) st.gzs[r_] = gzv;
             }
             RFA_TICK_AT(1, 0);
@@ -228,9 +253,12 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
             {
                 const int ii = 16 * wf + row;
                 const float gzi = st.gzs[ii];
+                // gz enters as the accumulator the products start from (column i of X^T is this lane)
+                f4 gz4;
+                gz4[0] = gzi; gz4[1] = gzi; gz4[2] = gzi; gz4[3] = gzi;
                 f4 xt[4];
 #pragma unroll
-                for (int jt = 0; jt < 4; ++jt) xt[jt] = f4_zero();
+                for (int jt = 0; jt < 4; ++jt) xt[jt] = gz4;
 #pragma unroll
                 for (int cs = 0; cs < DH / 32; ++cs) {
                     const h8 bg = row8(st.Gs, LDV, ii, cs * 32, G);
@@ -239,13 +267,11 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
                 }
 #pragma unroll
                 for (int jt = 0; jt < 4; ++jt) {
-                    h4 pv_;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int j = 16 * jt + 4 * G + e;
-                        pv_[e] = (j <= ii) ? (half_t)(xt[jt][e] + gzi) : (half_t)0.f;
-                    }
-                    *reinterpret_cast<h4*>(st.Ps + ii * LDA + 16 * jt + 4 * G) = pv_;
+                    // rounded pairs, then the halves above the diagonal cleared by a mask that is set up once
+                    uint2 pv_;
+                    pv_.x = pack_h2(xt[jt][0], xt[jt][1]) & tril_mask[jt].x;
+                    pv_.y = pack_h2(xt[jt][2], xt[jt][3]) & tril_mask[jt].y;
+                    *reinterpret_cast<uint2*>(st.Ps + ii * LDA + 16 * jt + 4 * G) = pv_;
                 }
             }
             RFA_TICK_AT(4, 0);
@@ -327,9 +353,9 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
                     for (int it = 0; it < 4; ++it) yt[kt][it] = mfma32(sh, bg[it], yt[kt][it]);
                 }
             }
-            RFA_TICK_AT(11, 256);
+            RFA_TICK_AT(11, kDqTick);
             wg_sync();
-            RFA_TICK_AT(12, 256);
+            RFA_TICK_AT(12, kDqTick);
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const int ii = 16 * it + row;
@@ -345,12 +371,12 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
                     acc = mfma32(kf[kt][0], p0, acc);
                     if (it >= 2) acc = mfma32(kf[kt][1], p1, acc);
                     if (!RAGGED || t0 + ii < T)
-                        *reinterpret_cast<h4*>(dqb + (int64_t)(t0 + ii) * k_stride + kl0 + 16 * kt + 4 * G) = to_h4(acc);
+                        store_lane(dqb + (int64_t)(t0 + 16 * it) * k_stride + kl0 + 16 * kt, out_lane_off, to_h4(acc));
                 }
             }
-            RFA_TICK_AT(13, 256);
+            RFA_TICK_AT(13, kDqTick);
             wg_sync();
-            RFA_TICK_AT(14, 256);
+            RFA_TICK_AT(14, kDqTick);
         };
         wg_sync();      // the first iteration: the loader group stages the last chunk
         wg_sync();
@@ -409,7 +435,7 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt)
                     if (!RAGGED || t0 + jj < T)
-                        *reinterpret_cast<h4*>(dkb + (int64_t)(t0 + jj) * k_stride + kl0 + 16 * kt + 4 * G) = to_h4(dkacc[kt][jt]);
+                        store_lane(dkb + (int64_t)(t0 + 16 * jt) * k_stride + kl0 + 16 * kt, out_lane_off, to_h4(dkacc[kt][jt]));
             }
 #pragma unroll
             for (int is = 0; is < 2; ++is) {
@@ -444,24 +470,26 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
 //             (k = 16kt + 4G + e, c = cw + i), all KD feature rows, is kept by both waves of a
 //             column tile (the same updates in the same order: identical bits).
 // ---------------------------------------------------------------------------
-template <int KD, int DH>
+template <int KD, int DH, int SW>
 __device__ __forceinline__ void sliced_bwd_dv(
     unsigned char* smem, int n, int coff, const half_t* __restrict__ q, const half_t* __restrict__ k,
     const half_t* __restrict__ g, const float* __restrict__ den_raw, half_t* __restrict__ dv, int T, int N) {
-    using Cfg = SlicedBwdCfg<KD, DH>;
+    using Cfg = SlicedBwdCfg<KD, DH, SW>;
     constexpr int NT = kGroupThreads, C = Cfg::C, CSL = Cfg::CSL;
-    constexpr int LDQ = Cfg::LDQ, LDG = Cfg::LDS_, LDA = Cfg::LDA;
+    constexpr int LDQ = Cfg::LDQ, LDG = Cfg::LDG_, LDA = Cfg::LDA;
     constexpr int NKT = KD / 16;
     constexpr int PPR = CSL / 8, VP = ChunkRegs<CSL, NT>::kPieces;
     constexpr size_t kStage = Cfg::kLds / 2;
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (w >= 8) return;                         // the role has 8 waves; the launch may carry more for the other role
     const int grp = w >> 2, wc = w & 3;         // loader: column block of the A^T tiles
     const int tid = threadIdx.x & (NT - 1);
     const int row = lane & 15, G = lane >> 4;
     const int jh = (w >> 1) & 1;                // product waves 4..7: half of the chunk's rows ...
     const int cl0 = 32 * (w & 1);               // ... and first of this wave's 32 columns, local to the slice array
+    const unsigned out_lane_off = (unsigned)row * (unsigned)(N * DH * 2) + 8u * G;
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
     const int n_chunks = (T + C - 1) / C;
     RFA_TICK_INIT();
@@ -491,6 +519,14 @@ __device__ __forceinline__ void sliced_bwd_dv(
             float den[VP];
         };
         RowSet s0, s1;
+        // which halves of this lane's A^T elements are kept: element (j = 16wc + row, i = 16it + 4G + e) when i >= j
+        uint2 tril_mask[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            auto keep = [&](int e) { return (16 * it + 4 * G + e >= 16 * wc + row) ? 0xffffu : 0u; };
+            tril_mask[it].x = keep(0) | (keep(1) << 16);
+            tril_mask[it].y = keep(2) | (keep(3) << 16);
+        }
         auto prefetch_ragged = [&](RowSet& r, int c) __attribute__((always_inline)) {
             const int t0 = c * C, rows = T - t0;
             chunk_g2r<KD, NT>(r.rk, kb + (int64_t)t0 * k_stride, k_stride, rows, tid);
@@ -516,7 +552,7 @@ __device__ __forceinline__ void sliced_bwd_dv(
             chunk_r2s<KD, NT>(r.rq, st.Qs, LDQ, tid);
             float inv_den[VP];
 #pragma unroll
-            for (int it = 0; it < VP; ++it) inv_den[it] = 1.0f / fmaxf(r.den[it], 1.0f);
+            for (int it = 0; it < VP; ++it) inv_den[it] = rcp_nr(fmaxf(r.den[it], 1.0f));
             chunk_r2s_scaled<CSL, NT>(r.rg, inv_den, st.Gs, LDG, tid);
             RFA_TICK_AT(1, 0);
             wg_sync();
@@ -538,13 +574,10 @@ __device__ __forceinline__ void sliced_bwd_dv(
                 }
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
-                    h4 av;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int ii = 16 * it + 4 * G + e;
-                        av[e] = (ii >= j) ? (half_t)a_[it][e] : (half_t)0.f;
-                    }
-                    *reinterpret_cast<h4*>(st.ATs + j * LDA + 16 * it + 4 * G) = av;
+                    uint2 av;
+                    av.x = pack_h2(a_[it][0], a_[it][1]) & tril_mask[it].x;
+                    av.y = pack_h2(a_[it][2], a_[it][3]) & tril_mask[it].y;
+                    *reinterpret_cast<uint2*>(st.ATs + j * LDA + 16 * it + 4 * G) = av;
                 }
             }
             RFA_TICK_AT(4, 0);
@@ -617,7 +650,7 @@ __device__ __forceinline__ void sliced_bwd_dv(
 #pragma unroll
                 for (int cc = 0; cc < 2; ++cc)
                     if (!RAGGED || t0 + jj < T)
-                        *reinterpret_cast<h4*>(dvb + (int64_t)(t0 + jj) * v_stride + cl0 + 16 * cc + 4 * G) = to_h4(dvacc[cc][u]);
+                        store_lane(dvb + (int64_t)(t0 + 16 * (2 * jh + u)) * v_stride + cl0 + 16 * cc, out_lane_off, to_h4(dvacc[cc][u]));
             }
 #pragma unroll
             for (int is = 0; is < 2; ++is)
@@ -638,31 +671,31 @@ __device__ __forceinline__ void sliced_bwd_dv(
     }
 }
 
-// grid = kXcds * ceil(N / kXcds) * (NA + NB); kSlicedThreads threads.  hdr_in / plan: see plan_matches.
-template <int KD, int DH>
-__global__ __launch_bounds__(kSlicedThreads) void k_sliced_bwd(
+// grid = kXcds * ceil(N / kXcds) * (NA + NB); Cfg::kThreads threads.  hdr_in / plan: see plan_matches.
+template <int KD, int DH, int SW>
+__global__ __launch_bounds__(sliced_threads(SW)) void k_sliced_bwd(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     const half_t* __restrict__ g, const half_t* __restrict__ o, const float* __restrict__ den_raw,
     const float* __restrict__ final_s, const float* __restrict__ final_z, half_t* __restrict__ dq,
     half_t* __restrict__ dk, half_t* __restrict__ dv, int T, int N, const int* __restrict__ hdr_in, PlanWords plan) {
-    using Cfg = SlicedBwdCfg<KD, DH>;
+    using Cfg = SlicedBwdCfg<KD, DH, SW>;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     int n, role;
     seq_role_of_block(blockIdx.x, Cfg::NA + Cfg::NB, n, role);
     if (n >= N) return;
     if (!plan_matches(hdr_in, plan)) {
         if (role < Cfg::NA) {
-            poison_rows<kSliceWidth>(dq + (int64_t)n * KD + role * kSliceWidth, (int64_t)N * KD, 0, T);
-            poison_rows<kSliceWidth>(dk + (int64_t)n * KD + role * kSliceWidth, (int64_t)N * KD, 0, T);
+            poison_rows<SW>(dq + (int64_t)n * KD + role * SW, (int64_t)N * KD, 0, T);
+            poison_rows<SW>(dk + (int64_t)n * KD + role * SW, (int64_t)N * KD, 0, T);
         } else {
             poison_rows<kSliceWidth>(dv + (int64_t)n * DH + (role - Cfg::NA) * kSliceWidth, (int64_t)N * DH, 0, T);
         }
         return;
     }
     if (role < Cfg::NA)
-        sliced_bwd_dqdk<KD, DH>(smem_raw, n, role * kSliceWidth, q, k, v, g, o, den_raw, dq, dk, final_s, final_z, T, N);
+        sliced_bwd_dqdk<KD, DH, SW>(smem_raw, n, role * SW, q, k, v, g, o, den_raw, dq, dk, final_s, final_z, T, N);
     else
-        sliced_bwd_dv<KD, DH>(smem_raw, n, (role - Cfg::NA) * kSliceWidth, q, k, g, den_raw, dv, T, N);
+        sliced_bwd_dv<KD, DH, SW>(smem_raw, n, (role - Cfg::NA) * kSliceWidth, q, k, g, den_raw, dv, T, N);
 }
 
 }  // namespace rfa
