@@ -156,6 +156,12 @@ int rfa_causal_num_segments(int64_t T, int64_t N, int K, int d);
  *             d = 64 when the slices cover 45 % of the compute units, at d = 128 only with K = 128
  *             and 90 %) / the
  *             segment-totals layout of the two-sweep backward
+ *   "recompute"  1/0: the forward with K <= 128 runs as one launch without segment totals (every
+ *             workgroup rebuilds the state at its segment's first step from the k, v rows before
+ *             it; segments of unequal length) whenever no backward wants the totals / never.
+ *             Unset: for up to 4 segments.  Its output has the bits of the one-segment scan.
+ *   "prefix_cost"  cost of a rebuilt 64-step block in percent of a scanned one (default 12): moves
+ *             the cut of that forward into segments
  * Initial values come from the environment variables RFA_HIP_<NAME>, read once per process and
  * never on the launch path.  No counterpart in the reference. */
 int rfa_tuning_set(const char* name, int value);

@@ -1,7 +1,9 @@
 """Builds librfa_hip.so (the C-ABI kernel library) for gfx950 with hipcc, and
 _rfa_hip_ext.so, the PyTorch C++ binding of that library (host code only, g++).
 
-Usage:  python -m rfa_amd.build [--verbose] [--resource-usage] [--no-ext]
+Usage:  python -m rfa_amd.build [--verbose] [--resource-usage] [--no-ext] [--only K,d -o PATH]
+(--only builds a development library with the scan kernels of one (feature width, head dim) only,
+in a fraction of the time, into PATH; the package never loads it by itself.)
 Both are written next to this file; rfa_amd._lib loads the first with ctypes, rfa_amd.rfa_hip
 imports the second when it is there.
 """
@@ -38,9 +40,9 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose: bool = False, extra_flags=()) -> str:
+def build(verbose: bool = False, extra_flags=(), out_path: str = LIB_PATH) -> str:
     cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags,
-           *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB_PATH]
+           *[os.path.join(CSRC, s) for s in SOURCES], "-o", out_path]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -49,7 +51,7 @@ def build(verbose: bool = False, extra_flags=()) -> str:
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
-    return LIB_PATH
+    return out_path
 
 
 EXT_NAME = "_rfa_hip_ext"
@@ -86,6 +88,13 @@ def build_ext(verbose: bool = False) -> str:
 if __name__ == "__main__":
     extra = ["-Rpass-analysis=kernel-resource-usage"] if "--resource-usage" in sys.argv else []
     verbose = True if extra else ("--verbose" in sys.argv or "-v" in sys.argv)
+    if "--only" in sys.argv:
+        kd = sys.argv[sys.argv.index("--only") + 1].split(",")
+        if "-o" not in sys.argv:
+            sys.exit("--only needs -o PATH: a one-shape library must not replace the package's own")
+        print(build(verbose=verbose, extra_flags=[*extra, f"-DRFA_ONLY_K={int(kd[0])}", f"-DRFA_ONLY_D={int(kd[1])}"],
+                    out_path=sys.argv[sys.argv.index("-o") + 1]))
+        sys.exit(0)
     print(build(verbose=verbose, extra_flags=extra))
     if "--no-ext" not in sys.argv and not extra:
         print(build_ext(verbose=verbose))

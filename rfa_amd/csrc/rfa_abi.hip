@@ -98,10 +98,11 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // every code path at small sizes.  -1 = the heuristic.  The environment is read once, when the
 // first knob is looked up, never on the launch path; rfa_tuning_set changes a knob afterwards.
 namespace tune {
-enum Key { NSEG, PREFIX, NSEG_SAME, FREE_WG, PROJECT_STREAMING, SLICED, COUNT };
-const char* const kNames[COUNT] = {"nseg", "prefix", "nseg_same", "free_wg", "project_streaming", "sliced"};
+enum Key { NSEG, PREFIX, NSEG_SAME, FREE_WG, PROJECT_STREAMING, SLICED, RECOMPUTE, PREFIX_COST, COUNT };
+const char* const kNames[COUNT] = {"nseg", "prefix", "nseg_same", "free_wg", "project_streaming", "sliced", "recompute", "prefix_cost"};
 const char* const kEnv[COUNT] = {"RFA_HIP_NSEG", "RFA_HIP_PREFIX", "RFA_HIP_NSEG_SAME", "RFA_HIP_FREE_WG",
-                                 "RFA_HIP_PROJECT_STREAMING", "RFA_HIP_SLICED"};
+                                 "RFA_HIP_PROJECT_STREAMING", "RFA_HIP_SLICED", "RFA_HIP_RECOMPUTE",
+                                 "RFA_HIP_PREFIX_COST"};
 std::atomic<int> value[COUNT];
 std::once_flag once;
 
@@ -337,10 +338,41 @@ void launch_totals_scan(float* a, int64_t Ma, float* b, int64_t Mb, int N, int n
                dim3(rfa::kThreads), 0, st, a, Ma, b, Mb, nseg);
 }
 
+// The forward without segment totals (k_causal_fwd_pipe<.., RECOMPUTE>): every workgroup rebuilds
+// the state at its segment's first step from the k, v rows before it.  A prefix chunk costs
+// about an eighth of a scan chunk ("prefix_cost" knob, percent; measured at T = 1024, N = 64:
+// 10 and 15 give 18.8 us, 20 to 30 give 19.0 to 19.2), so segment s gets
+// u - cost * first[s] chunks, with u the smallest figure whose segments cover the sequence:
+// prefix plus scan then take every workgroup about equally long.  Pays while a sequence has few
+// segments (the last one streams nearly the whole sequence): up to 4 ("recompute" knob: 0 never,
+// 1 whenever the kernel exists).  False if no such cut exists.
+bool recompute_bounds(int64_t T, int nseg, rfa::SegBounds* b) {
+    const int knob = tune::get(tune::RECOMPUTE);
+    if (knob == 0 || nseg < 2 || nseg > rfa::kMaxSegments || (knob < 0 && nseg > 4)) return false;
+    const int nch = (int)((T + rfa::kChunk - 1) / rfa::kChunk);
+    const int cost_knob = tune::get(tune::PREFIX_COST);
+    const double cost = (cost_knob >= 0 ? cost_knob : 12) / 100.0;
+    for (double u = (double)nch / nseg; u <= nch; u += 0.25) {
+        b->first[0] = 0;
+        for (int s_ = 0; s_ < nseg; ++s_) {
+            int len = (int)(u - cost * b->first[s_] + 1e-9);
+            if (len < 1) len = 1;
+            b->first[s_ + 1] = b->first[s_] + len;
+        }
+        if (b->first[nseg] < nch) continue;
+        if (b->first[nseg - 1] >= nch) return false;        // the cut leaves a segment empty
+        b->first[nseg] = nch;
+        for (int s_ = nseg + 1; s_ <= rfa::kMaxSegments; ++s_) b->first[s_] = nch;
+        return true;
+    }
+    return false;
+}
+
 template <int KD, int DH>
 int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, rfa::half_t* out,
                    int T, int N, const ScanPlan& p, char* ws, const Workspace& wl, int* savedHdr, float* savedS,
-                   float* savedZ, float* savedDen, float* final_s, float* final_z, hipStream_t st) {
+                   float* savedZ, float* savedDen, float* final_s, float* final_z, bool allow_recompute,
+                   hipStream_t st) {
     // the two-stage pipelined forward needs both chunk buffers in LDS: K <= 128
     constexpr bool PIPE = rfa::FwdPipeCfg<KD, DH>::kLds <= 160 * 1024;
     constexpr int NW = PIPE ? 4 : causal_waves(KD, DH);
@@ -348,6 +380,24 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
     using Cfg = rfa::CausalCfg<KD, DH, NW>;
     // with a saved buffer the segment totals are written there directly (S in the forward's
     // fragment order, which the saved-pair backward reads as is)
+    const rfa::PlanWords pw = plan_words(T, N, KD, DH, p);
+    if constexpr (PIPE) {
+        // nobody else reads the totals (the saved pair of this layout keeps only the final state):
+        // one launch that needs none
+        rfa::SegBounds bounds{};
+        if (allow_recompute && !savedS && recompute_bounds(T, p.nseg, &bounds) &&
+            (int64_t)rfa::kChunk * N * KD * 2 < ((int64_t)1 << 32)) {
+            auto kern = rfa::k_causal_fwd_pipe<KD, DH, true>;
+            if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
+            RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(512), rfa::FwdPipeCfg<KD, DH>::kLds, st, q, k, v, out,
+                       (const float*)nullptr, (const float*)nullptr, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, 0,
+                       savedHdr, pw, bounds);
+            RFA_HIP_TRY(hipGetLastError());
+            return RFA_OK;
+        }
+    }
+    if (p.nseg > 1 && !ws && !savedS)
+        return fail(RFA_ERR_WORKSPACE, "rfa_causal_forward: this shape needs a workspace for its segment totals");
     float* wsS = savedS ? savedS : reinterpret_cast<float*>(ws + wl.S);
     float* wsZ = savedZ ? savedZ : reinterpret_cast<float*>(ws + wl.Z);
     if (p.nseg > 1) {
@@ -357,12 +407,12 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
                            k, v, (const uint8_t*)nullptr, 1, wsS, wsZ, (float*)nullptr, T, N, p.nseg, p.nseg - 1, p.seg_len);
     }
     if (p.prefixed) launch_totals_scan<false>(wsS, (int64_t)KD * DH, wsZ, KD, N, p.nseg, st);
-    const rfa::PlanWords pw = plan_words(T, N, KD, DH, p);
     if constexpr (PIPE) {
-        auto kern = rfa::k_causal_fwd_pipe<KD, DH>;
+        auto kern = rfa::k_causal_fwd_pipe<KD, DH, false>;
         if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(512), rfa::FwdPipeCfg<KD, DH>::kLds, st, q, k, v, out,
-                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, p.prefixed, savedHdr, pw);
+                           wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, p.prefixed, savedHdr, pw,
+                           rfa::SegBounds{});
     } else {
         auto kern = rfa::k_causal_fwd<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
@@ -1038,7 +1088,8 @@ int rfa_causal_saved_describe(const void* saved, int32_t* words16, void* stream)
 
 static int causal_forward_impl(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
                                int K, int d, void* saved, size_t saved_bytes, bool want_saved, float* final_s,
-                               float* final_z, void* workspace, size_t workspace_bytes, void* stream);
+                               float* final_z, void* workspace, size_t workspace_bytes, void* stream,
+                               bool allow_recompute = true);
 
 int rfa_causal_forward(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
                        int K, int d, void* workspace, size_t workspace_bytes, void* stream) {
@@ -1060,9 +1111,10 @@ int rfa_causal_forward_noalloc(const void* q, const void* k, const void* v, void
     unsigned char* ptr = nullptr;       // this device's copy of the static array
     if (int rc = static_scratch_address(&ptr)) return rc;
     // every slot of the segment totals that the scan reads is written by the totals pass of the same
-    // call first, so what an earlier call left in the array does not matter
+    // call first, so what an earlier call left in the array does not matter.  (This entry point
+    // always takes the form with segment totals: the array is what it exists for.)
     return causal_forward_impl(q, k, v, out, T, N, K, d, nullptr, 0, false, nullptr, nullptr, ptr, kStaticScratchBytes,
-                               stream);
+                               stream, false);
 }
 
 int rfa_causal_prefill(const void* q, const void* k, const void* v, void* out, float* s, float* z, int64_t T,
@@ -1089,7 +1141,8 @@ int rfa_causal_forward_save(const void* q, const void* k, const void* v, void* o
 
 static int causal_forward_impl(const void* q, const void* k, const void* v, void* out, int64_t T, int64_t N,
                                int K, int d, void* saved, size_t saved_bytes, bool want_saved, float* final_s,
-                               float* final_z, void* workspace, size_t workspace_bytes, void* stream) {
+                               float* final_z, void* workspace, size_t workspace_bytes, void* stream,
+                               bool allow_recompute) {
     if (int rc = check_causal_dims(T, N, K, d)) return rc;
     if (T == 0 || N == 0) return RFA_OK;
     const ScanPlan p = make_plan(T, N, K, d);
@@ -1130,7 +1183,7 @@ static int causal_forward_impl(const void* q, const void* k, const void* v, void
     auto* oh = static_cast<rfa::half_t*>(out);
     char* ws = static_cast<char*>(workspace);
     if (want_saved) registry::put(saved, plan_words(T, N, K, d, p));
-#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedHdr, savedS, savedZ, savedDen, final_s, final_z, st)
+#define RFA_CALL_FWD(KD, DH) launch_forward<KD, DH>(qh, kh, vh, oh, (int)T, (int)N, p, ws, wl, savedHdr, savedS, savedZ, savedDen, final_s, final_z, allow_recompute, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL_FWD)
 #undef RFA_CALL_FWD
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");

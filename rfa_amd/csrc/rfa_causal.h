@@ -493,12 +493,23 @@ __device__ __forceinline__ void wg_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
-template <int KD, int DH>
+//
+// RECOMPUTE: no segment totals.  A workgroup first rebuilds the state at its segment's first step
+// by streaming the k, v rows of everything before it through the same state update (one barrier
+// and about a fifth of a scan chunk's time per 64 steps: the rows come out of the L2 of the XCD
+// that holds all segments of the sequence), then scans.  Segments are cut so that prefix plus
+// scan take every workgroup about equally long (SegBounds: later segments are shorter).  One
+// launch, no workspace; pays while a sequence has few segments.
+struct SegBounds {
+    int first[17];      // segment s covers chunks [first[s], first[s + 1])
+};
+
+template <int KD, int DH, bool RECOMPUTE = false>
 __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
     float* __restrict__ den_out, float* __restrict__ final_s, float* __restrict__ final_z, int T, int N,
-    int nseg, int seg_len, int prefixed, int* __restrict__ hdr_out, PlanWords plan) {
+    int nseg, int seg_len, int prefixed, int* __restrict__ hdr_out, PlanWords plan, SegBounds bounds) {
     plan_write(hdr_out, plan);
     using Cfg = FwdPipeCfg<KD, DH>;
     constexpr int NT = 256;      // threads per group
@@ -516,19 +527,28 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
     const int row = lane & 15, G = lane >> 4;
     int n, seg;
     seq_seg_of_block(blockIdx.x, N, nseg, n, seg);
-    const int t_begin = seg * seg_len;
-    const int t_end = min(T, t_begin + seg_len);
+    const int t_begin = RECOMPUTE ? bounds.first[seg] * C : seg * seg_len;
+    const int t_end = min(T, RECOMPUTE ? bounds.first[seg + 1] * C : t_begin + seg_len);
     const int n_chunks = t_end > t_begin ? (t_end - t_begin + C - 1) / C : 0;
+    const int n_prefix = (RECOMPUTE && n_chunks > 0) ? bounds.first[seg] : 0;     // full chunks before the segment
     const int64_t k_stride = (int64_t)N * KD, v_stride = (int64_t)N * DH;
 
     RFA_TICK_INIT();
-    // Both branches run n_chunks + 1 iterations with exactly two barriers each.
+    // Both branches run n_prefix iterations with one barrier each and one more barrier (RECOMPUTE),
+    // then n_chunks + 1 iterations with exactly two barriers each.
     if (tile_group) {
         const half_t* qb = q + (int64_t)n * KD;
         const half_t* kb = k + (int64_t)n * KD;
         const half_t* vb = v + (int64_t)n * DH;
         ChunkRegs<KD, NT> rq, rk;
         ChunkRegs<DH, NT> rv;
+        // full chunks: wave-uniform base plus one lane offset per tensor; only the last chunk of the
+        // sequence can be short and takes the clamped row addresses
+        RowPtrs<KD, NT> pq_, pk_;
+        RowPtrs<DH, NT> pv_;
+        pq_.init(qb, k_stride, tid);
+        pk_.init(kb, k_stride, tid);
+        pv_.init(vb, v_stride, tid);
         if (n_chunks > 0) {
             chunk_g2r<KD, NT>(rq, qb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
             chunk_g2r<KD, NT>(rk, kb + (int64_t)t_begin * k_stride, k_stride, t_end - t_begin, tid);
@@ -537,7 +557,47 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
         f4 zacc[NKTW];      // z for feature tiles kt = w*NKTW + a, element k = 16kt + 4G + e
 #pragma unroll
         for (int a = 0; a < NKTW; ++a) zacc[a] = f4_zero();
-        {
+        const h8 ones = h8_ones();
+        if constexpr (RECOMPUTE) {
+            // the k, v rows of the chunks before the segment, three chunks in flight
+            ChunkRegs<KD, NT> xk[3];
+            ChunkRegs<DH, NT> xv[3];
+            auto request = [&](auto set, int c) __attribute__((always_inline)) {
+                constexpr int S_ = decltype(set)::value;
+                const int64_t t0 = (int64_t)min(c, max(n_prefix - 1, 0)) * C;     // past the prefix: any valid chunk, never used
+                pk_.load_full(xk[S_], t0 * k_stride);
+                pv_.load_full(xv[S_], t0 * v_stride);
+            };
+            auto step = [&](auto set, int jc) __attribute__((always_inline)) {
+                constexpr int S_ = decltype(set)::value;
+                unsigned char* base = smem_raw + (jc & 1) * Cfg::kBufBytes;
+                half_t* Ks = reinterpret_cast<half_t*>(base) + C * LDQ;
+                half_t* Vs = Ks + C * LDQ;
+                chunk_r2s<KD, NT>(xk[S_], Ks, LDQ, tid);
+                chunk_r2s<DH, NT>(xv[S_], Vs, LDV, tid);
+                wg_barrier();
+                request(set, jc + 3);
+#pragma unroll
+                for (int a = 0; a < NKTW; ++a)
+#pragma unroll
+                    for (int js = 0; js < 2; ++js)
+                        zacc[a] = mfma32(col8(Ks, LDQ, js * 32, 16 * (w * NKTW + a), lane), ones, zacc[a]);
+            };
+            using I0 = std::integral_constant<int, 0>;
+            using I1 = std::integral_constant<int, 1>;
+            using I2 = std::integral_constant<int, 2>;
+            if (n_prefix > 0) {
+                request(I0{}, 0);
+                request(I1{}, 1);
+                request(I2{}, 2);
+            }
+            for (int jc = 0; jc < n_prefix; jc += 3) {
+                step(I0{}, jc);
+                if (jc + 1 < n_prefix) step(I1{}, jc + 1);
+                if (jc + 2 < n_prefix) step(I2{}, jc + 2);
+            }
+            wg_barrier();       // the state group has read the last prefix chunk
+        } else {
             struct ZSlot { f4 z[NKTW]; };
             sum_slots<4, ZSlot>(prefixed ? seg : 0, prefixed ? seg + 1 : seg,
                 [&](int s, ZSlot& t) {
@@ -550,7 +610,6 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
                     for (int a = 0; a < NKTW; ++a) zacc[a] += keep * t.z[a];
                 });
         }
-        const h8 ones = h8_ones();
         RFA_TICK_AT(0, 0);
         for (int it = 0; it <= n_chunks; ++it) {
             unsigned char* base = smem_raw + (it & 1) * Cfg::kBufBytes;
@@ -574,10 +633,9 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
             RFA_TICK_AT(2, 0);
             if (live) {
                 const int t0 = t_begin + it * C;
-                if (it + 1 < n_chunks) {
-                    const int rows = t_end - t0 - C;
-                    chunk_g2r<KD, NT>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-                }
+                const int rows_next = t_end - t0 - C;
+                if (rows_next >= C) pq_.load_full(rq, (int64_t)(t0 + C) * k_stride);
+                else if (rows_next > 0) chunk_g2r<KD, NT>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows_next, tid);
                 RFA_TICK_AT(3, 0);
                 // rows i in [16w, 16w+16) of A as A^T tiles (m=j, n=i), all four j tiles
                 f4 at[4];
@@ -589,10 +647,12 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
 #pragma unroll
                     for (int a = 0; a < 4; ++a) at[a] = mfma32(row8(Ks, LDQ, 16 * a + row, ks * 32, G), bq, at[a]);
                 }
-                if (it + 1 < n_chunks) {      // second part of the next chunk's rows
-                    const int rows = t_end - t0 - C;
-                    chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows, tid);
-                    chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows, tid);
+                if (rows_next >= C) {         // second part of the next chunk's rows
+                    pk_.load_full(rk, (int64_t)(t0 + C) * k_stride);
+                    pv_.load_full(rv, (int64_t)(t0 + C) * v_stride);
+                } else if (rows_next > 0) {
+                    chunk_g2r<KD, NT>(rk, kb + (int64_t)(t0 + C) * k_stride, k_stride, rows_next, tid);
+                    chunk_g2r<DH, NT>(rv, vb + (int64_t)(t0 + C) * v_stride, v_stride, rows_next, tid);
                 }
                 float part = 0.f;
 #pragma unroll
@@ -645,12 +705,33 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
         }
     } else {
         half_t* ob = out + (int64_t)n * DH;
+        const unsigned out_lane_off = (unsigned)row * (unsigned)(N * DH * 2) + 8u * G;   // bytes: row of a 16-step tile, 4 halves from 4G
         f4 S[NKT][NCT];
 #pragma unroll
         for (int a = 0; a < NKT; ++a)
 #pragma unroll
             for (int b = 0; b < NCT; ++b) S[a][b] = f4_zero();
-        {
+        if constexpr (RECOMPUTE) {
+            for (int jc = 0; jc < n_prefix; ++jc) {
+                wg_barrier();
+                const half_t* Ks = reinterpret_cast<const half_t*>(smem_raw + (jc & 1) * Cfg::kBufBytes) + C * LDQ;
+                const half_t* Vs = Ks + C * LDQ;
+                h8 av[NCT][2];
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                    for (int js = 0; js < 2; ++js) av[ct][js] = col8(Vs, LDV, js * 32, w * DS + 16 * ct, lane);
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                    for (int js = 0; js < 2; ++js) {
+                        h8 ak = col8(Ks, LDQ, js * 32, 16 * kt, lane);
+#pragma unroll
+                        for (int ct = 0; ct < NCT; ++ct) S[kt][ct] = mfma32(ak, av[ct][js], S[kt][ct]);
+                    }
+            }
+            wg_barrier();
+        } else {
             struct SSlot { f4 s[NKT][NCT]; };
             constexpr int GRP = (NKT * NCT <= 8) ? 3 : 1;     // 32 registers per slot at K = 128, d = 64
             sum_slots<GRP, SSlot>(prefixed ? seg : 0, prefixed ? seg + 1 : seg,
@@ -722,13 +803,13 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
                     const int i = 16 * i4 + row;
-                    const float inv = 1.0f / fmaxf(dens[i], 1.0f);
+                    const float inv = rcp_nr(fmaxf(dens[i], 1.0f));
                     if (t0 + i < t_end) {
 #pragma unroll
                         for (int ct = 0; ct < NCT; ++ct) {
                             f4 o = acc[i4][ct];
                             o[0] *= inv; o[1] *= inv; o[2] *= inv; o[3] *= inv;
-                            *reinterpret_cast<h4*>(ob + (int64_t)(t0 + i) * v_stride + w * DS + 16 * ct + 4 * G) = to_h4(o);
+                            store_lane(ob + (int64_t)(t0 + 16 * i4) * v_stride + w * DS + 16 * ct, out_lane_off, to_h4(o));
                         }
                     }
                 }

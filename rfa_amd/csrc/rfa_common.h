@@ -299,6 +299,42 @@ __device__ __forceinline__ void chunk_g2r(ChunkRegs<F, NT>& r, const half_t* __r
     }
 }
 
+// 64 rows x F halves of a full chunk.  The address of a piece is a base that is the same for the
+// whole wave (tensor + sequence + chunk + piece index * rows per pass: scalar registers and scalar
+// arithmetic) plus one 32-bit byte offset per lane, set up once: a load costs no vector
+// arithmetic and the row addresses take one register per tensor.  64 rows of a tensor must span
+// less than 4 GiB (the launchers check).
+template <int F, int NT = kThreads>
+struct RowPtrs {
+    static constexpr int kPieces = ChunkRegs<F, NT>::kPieces;
+    static constexpr int PPR = F / 8;                       // 16-byte pieces per row
+    static constexpr int kRowsPerPass = NT / PPR;
+    const char* base;       // wave-uniform
+    int64_t pass_bytes;     // wave-uniform: kRowsPerPass rows
+    unsigned lane_off;
+    __device__ __forceinline__ void init(const half_t* tensor, int64_t row_stride, int tid) {
+        base = reinterpret_cast<const char*>(tensor);
+        pass_bytes = (int64_t)kRowsPerPass * row_stride * 2;
+        lane_off = (unsigned)(tid / PPR) * (unsigned)(row_stride * 2) + (unsigned)(tid % PPR) * 16u;
+    }
+    __device__ __forceinline__ void load_full(ChunkRegs<F, NT>& r, int64_t chunk_off) const {
+        r.rows = kChunk;
+        const char* b = base + chunk_off * 2;
+#pragma unroll
+        for (int it = 0; it < kPieces; ++it) {
+            r.v[it] = *reinterpret_cast<const uint4*>(b + it * pass_bytes + lane_off);
+            r.drop[it] = 0;
+        }
+    }
+};
+
+// store through a wave-uniform base (scalar registers, scalar address arithmetic) plus one 32-bit
+// byte offset per lane that is set up once: no vector arithmetic per store
+template <typename V>
+__device__ __forceinline__ void store_lane(half_t* uniform_base, unsigned lane_off_bytes, const V& value) {
+    *reinterpret_cast<V*>(reinterpret_cast<char*>(uniform_base) + lane_off_bytes) = value;
+}
+
 // mark the rows whose mask byte is non-zero (mask already offset to the chunk's first
 // step); they are written to LDS as zeros.  Call after chunk_g2r.
 template <int F, int NT = kThreads>

@@ -82,42 +82,6 @@ struct SlicedBwdCfg {
 
 __device__ __forceinline__ void wg_sync() { __syncthreads(); }
 
-// store through a wave-uniform base (scalar registers, scalar address arithmetic) plus one 32-bit
-// byte offset per lane that is set up once: no vector arithmetic per store
-template <typename V>
-__device__ __forceinline__ void store_lane(half_t* uniform_base, unsigned lane_off_bytes, const V& value) {
-    *reinterpret_cast<V*>(reinterpret_cast<char*>(uniform_base) + lane_off_bytes) = value;
-}
-
-// 64 rows x F halves of a full chunk.  The address of a piece is a base that is the same for the
-// whole wave (tensor + sequence + chunk + piece index * rows per pass: scalar registers and scalar
-// arithmetic) plus one 32-bit byte offset per lane, set up once: a load costs no vector
-// arithmetic and the row addresses take one register per tensor.  64 rows of a tensor must span
-// less than 4 GiB (the launcher checks).
-template <int F>
-struct RowPtrs {
-    static constexpr int kPieces = ChunkRegs<F, kGroupThreads>::kPieces;
-    static constexpr int PPR = F / 8;                       // 16-byte pieces per row
-    static constexpr int kRowsPerPass = kGroupThreads / PPR;
-    const char* base;       // wave-uniform
-    int64_t pass_bytes;     // wave-uniform: kRowsPerPass rows
-    unsigned lane_off;
-    __device__ __forceinline__ void init(const half_t* tensor, int64_t row_stride, int tid) {
-        base = reinterpret_cast<const char*>(tensor);
-        pass_bytes = (int64_t)kRowsPerPass * row_stride * 2;
-        lane_off = (unsigned)(tid / PPR) * (unsigned)(row_stride * 2) + (unsigned)(tid % PPR) * 16u;
-    }
-    __device__ __forceinline__ void load_full(ChunkRegs<F, kGroupThreads>& r, int64_t chunk_off) const {
-        r.rows = kChunk;
-        const char* b = base + chunk_off * 2;
-#pragma unroll
-        for (int it = 0; it < kPieces; ++it) {
-            r.v[it] = *reinterpret_cast<const uint4*>(b + it * pass_bytes + lane_off);
-            r.drop[it] = 0;
-        }
-    }
-};
-
 // ---------------------------------------------------------------------------
 // dQ, dK for features [koff, koff + 64) of one sequence.
 //   loader group: stages Q, K slices, V, G^ = G / den and gz, then P = tril(G^ V^T + gz 1^T)
@@ -173,8 +137,8 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
         const half_t* vb = v + (int64_t)n * DH;
         const half_t* gb = g + (int64_t)n * DH;
         const half_t* ob = o + (int64_t)n * DH;
-        RowPtrs<KSL> pq, pk;
-        RowPtrs<DH> pv, pg, po;
+        RowPtrs<KSL, NT> pq, pk;
+        RowPtrs<DH, NT> pv, pg, po;
         pq.init(qb, k_stride, tid);
         pk.init(kb, k_stride, tid);
         pv.init(vb, v_stride, tid);
@@ -508,8 +472,8 @@ __device__ __forceinline__ void sliced_bwd_dv(
         const half_t* qb = q + (int64_t)n * KD;
         const half_t* kb = k + (int64_t)n * KD;
         const half_t* gb = g + (int64_t)n * DH + coff;
-        RowPtrs<KD> pq, pk;
-        RowPtrs<CSL> pg;
+        RowPtrs<KD, NT> pq, pk;
+        RowPtrs<CSL, NT> pg;
         pq.init(qb, k_stride, tid);
         pk.init(kb, k_stride, tid);
         pg.init(gb, v_stride, tid);

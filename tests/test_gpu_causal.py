@@ -138,7 +138,9 @@ def test_every_segment_count_gives_the_same_answer(nseg, scanned, knobs):
     consumers to add up the segment totals themselves ("0") or to read totals that a scan
     kernel turned into running sums first ("1"); unset, five segments or more take the scan."""
     from rfa_amd import rfa_hip
-    knobs(nseg=nseg, prefix=-1 if scanned is None else int(scanned))
+    # recompute=0: every forward of this test takes its state from segment totals (the form without
+    # totals has its own test below)
+    knobs(nseg=nseg, prefix=-1 if scanned is None else int(scanned), recompute=0)
     T, B, H, d, D = 700, 1, 3, 64, 64
     cpu = _features(T, B, H, d, D, seed=5000)
     pq, pk, v, g = (t.cuda() for t in cpu)
@@ -155,6 +157,38 @@ def test_every_segment_count_gives_the_same_answer(nseg, scanned, knobs):
     assert torch.equal(o2, out)
     _, s_ref, z_ref = O.causal_forward_loop(cpu[0].float(), cpu[1].float(), cpu[2].float())
     assert _rel(s.cpu(), s_ref) < 1e-5 and _rel(z.cpu(), z_ref) < 1e-5
+
+
+@pytest.mark.parametrize("T,B,H,d,D,nseg,cost,cut", [
+    (700, 1, 3, 64, 64, 2, -1, True), (700, 1, 3, 64, 64, 3, -1, True), (700, 1, 3, 64, 64, 4, 50, True),
+    (1024, 2, 3, 64, 64, 4, -1, True), (641, 1, 2, 64, 64, 11, 0, True), (3000, 1, 2, 64, 32, 12, 3, True),
+    (3000, 1, 2, 64, 32, 16, 5, False),      # no cut into 16 non-empty segments at this cost: the form with totals runs
+    (520, 1, 2, 128, 64, 3, -1, True), (130, 1, 5, 64, 64, 2, 90, True), (65, 1, 1, 64, 64, 2, -1, True)])
+def test_forward_without_segment_totals(T, B, H, d, D, nseg, cost, cut, knobs):
+    """The forward whose workgroups rebuild the state at their segment's first step from the k, v rows
+    before it (no totals pass, unequal segments; taken by itself for up to 4 segments, "recompute"
+    = 1 forces it for any count, "prefix_cost" moves the cut).  Output, prefill state and the
+    denominators handed to the sliced backward meet the oracle; the state is accumulated chunk
+    by chunk in time order whatever the cut, so the output has the bits of the one-segment scan."""
+    from rfa_amd import rfa_hip
+    cpu = _features(T, B, H, d, D, seed=5400 + T)
+    pq, pk, v, g = (t.cuda() for t in cpu)
+    ref = _oracle_fwd(*cpu[:3])
+    knobs(nseg=1, recompute=0)
+    one = rfa_hip.forward(pq, pk, v)
+    knobs(nseg=nseg, recompute=1, prefix_cost=cost, sliced=1)
+    print(f"forward without totals T={T} N={B * H} K={2 * D} d={d} nseg={nseg} cost={cost}", flush=True)
+    out = rfa_hip.forward(pq, pk, v)
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_ATOL
+    assert torch.equal(out, one) == cut
+    o2, s, z = rfa_hip.prefill(pq, pk, v)
+    assert torch.equal(o2, out)
+    _, s_ref, z_ref = O.causal_forward_loop(cpu[0].float(), cpu[1].float(), cpu[2].float())
+    assert _rel(s.cpu(), s_ref) < 1e-5 and _rel(z.cpu(), z_ref) < 1e-5
+    o3, saved = rfa_hip.forward_save(pq, pk, v)        # final-state layout: the same launch, plus den_raw and S_T, z_T
+    assert torch.equal(o3, out)
+    for name, a, b in zip(("dq", "dk", "dv"), rfa_hip.backward_saved(pq, pk, v, g, o3, saved), _oracle_bwd(*cpu)):
+        assert _rel(a.float().cpu(), b) <= GRAD_RTOL, name
 
 
 @pytest.mark.parametrize("nseg,same", [(8, False), (4, False), (6, False), (8, True), (5, False)])

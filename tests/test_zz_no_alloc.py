@@ -20,9 +20,10 @@ def _inputs(T, N, K, d, seed):
     return pq, pk, v.cuda().view(T, N, d)
 
 
-def test_noalloc_forward_equals_workspace_forward_on_two_calls_in_a_row():
+def test_noalloc_forward_equals_workspace_forward_on_two_calls_in_a_row(knobs):
     from rfa_amd import _lib, rfa_hip
     lib = _lib.load()
+    knobs(recompute=0)      # the existing entry point in the form this one always takes: state from segment totals
     stream = torch.cuda.current_stream().cuda_stream
     assert lib.rfa_static_scratch_bytes() == 16 << 20
     first = True
@@ -54,13 +55,14 @@ def test_noalloc_forward_equals_workspace_forward_on_two_calls_in_a_row():
     assert lib.rfa_causal_forward_noalloc(None, None, None, None, 0, 4, 128, 64, stream) == 0
 
 
-def test_noalloc_forward_under_graph_capture_replays_the_eager_bits():
+def test_noalloc_forward_under_graph_capture_replays_the_eager_bits(knobs):
     """The callers the entry point is for: a HIP graph captured after one warm-up call (the first call
     on a device looks the static array's address up and sets kernel attributes, which must not
     happen under capture).  Every replay, with eager work and synchronisation in between and new
     input values in the same tensors, gives the bits of rfa_causal_forward on those values."""
     from rfa_amd import _lib, rfa_hip
     lib = _lib.load()
+    knobs(recompute=0)
     T, N, K, d = 1024, 64, 128, 64
     q, k, v = _inputs(T, N, K, d, 3)
     got = torch.empty_like(v)
