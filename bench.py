@@ -507,9 +507,14 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream, skip=()):
     for _ in range(5):
         f(); b()
     tf, tb = _event_time_ms(torch, f, 100), _event_time_ms(torch, b, 100)
+    x_b, phi_b = torch.randn(T, B, H, d, generator=g).half().to(dev), torch.empty_like(gp)
+    fp_ = lambda: _lib.check(lib.rfa_feature_map_forward_pair(p(x), p(x_b), p(W), p(phi), p(phi_b), R, H, D, d, O.SCALE, stream))
+    for _ in range(5):
+        fp_()
+    tfp = _event_time_ms(torch, fp_, 100)
     rows = R * H
     ex["feature_map"] = {"workload": "phi of [1024, 8, 8, 64] -> [.., 128]; back-to-back launches through the C ABI",
-                         "fwd_us": round(1e3 * tf, 2), "bwd_us": round(1e3 * tb, 2),
+                         "fwd_us": round(1e3 * tf, 2), "bwd_us": round(1e3 * tb, 2), "fwd_pair_us": round(1e3 * tfp, 2),
                          "fwd_hbm_gbs": round(rows * (d + 2 * D) * 2 / (tf * 1e-3) / 1e9, 1),
                          "bwd_hbm_gbs": round(rows * (2 * d + 2 * D) * 2 / (tb * 1e-3) / 1e9, 1)}
     # ---- raw boundary (config 2): q, k, v [T, B, H, d] in, dq, dk, dv out -- the feature maps of q
@@ -532,8 +537,7 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream, skip=()):
     sv2 = torch.empty(max(sb2, 1), dtype=torch.uint8, device=dev)
 
     def raw_step():
-        _lib.check(lib.rfa_feature_map_forward(p(q2), p(W), p(pq2), R, H, D, d, O.SCALE, stream))
-        _lib.check(lib.rfa_feature_map_forward(p(k2), p(W), p(pk2), R, H, D, d, O.SCALE, stream))
+        _lib.check(lib.rfa_feature_map_forward_pair(p(q2), p(k2), p(W), p(pq2), p(pk2), R, H, D, d, O.SCALE, stream))
         _lib.check(lib.rfa_causal_forward_save(p(pq2), p(pk2), p(v2), p(o2), p(sv2), sb2, T, N2, K2, d, p(ws2), fb2, stream))
         _lib.check(lib.rfa_causal_backward_saved(p(pq2), p(pk2), p(v2), p(g2), p(o2), p(sv2), sb2, p(dpq), p(dpk), p(dv2),
                                                  T, N2, K2, d, p(ws2), bb2, stream))
@@ -543,7 +547,8 @@ def extras(torch, O, lib, _lib, rfa_hip, dev, stream, skip=()):
         raw_step()
     traw = _event_time_ms(torch, raw_step, 100)
     raw_bytes = 22 * d * N2 * T
-    ex["raw_boundary"] = {"workload": "configs[1] from raw q, k, v to dq, dk, dv: phi(q), phi(k), causal fwd+bwd, phi backward",
+    ex["raw_boundary"] = {"workload": "configs[1] from raw q, k, v to dq, dk, dv: phi(q) and phi(k) in one launch, causal "
+                                      "fwd+bwd, phi backward pair",
                           "us_per_step": round(1e3 * traw, 2), "tokens_per_s": round(B * T / (traw * 1e-3), 1),
                           "algorithmic_bytes": raw_bytes,
                           "frac_of_hbm": round(raw_bytes / (traw * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}

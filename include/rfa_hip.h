@@ -196,6 +196,11 @@ int rfa_build_random_matrices_backward(const void* w, const void* sigma, const v
                                        void* dsigma, void* dw, int H, int D, int d, void* stream);
 int rfa_feature_map_forward(const void* x, const void* w, void* phi, int64_t R, int H, int D, int d,
                             float scale, void* stream);
+/* phi(x0) and phi(x1) through the same w in one launch: the q and k projections of a module
+ * (causal_attention.py:241-248 calls random_project twice).  Same results as two
+ * rfa_feature_map_forward calls. */
+int rfa_feature_map_forward_pair(const void* x0, const void* x1, const void* w, void* phi0, void* phi1,
+                                 int64_t R, int H, int D, int d, float scale, void* stream);
 size_t rfa_feature_map_backward_workspace_bytes(int64_t R, int H, int D, int d);
 int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi, void* dx, float* dw,
                              int64_t R, int H, int D, int d, float scale, void* workspace,

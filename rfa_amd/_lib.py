@@ -54,6 +54,7 @@ SIGNATURES = {
     "rfa_build_random_matrices": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_void_p]),
     "rfa_build_random_matrices_backward": (c_int, [c_void_p] * 3 + [c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "rfa_feature_map_forward": (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int, c_int, c_float, c_void_p]),
+    "rfa_feature_map_forward_pair": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_float, c_void_p]),
     "rfa_feature_map_backward_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int]),
     "rfa_feature_map_backward": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p]),
     "rfa_feature_map_backward_pair_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int]),

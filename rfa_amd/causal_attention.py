@@ -20,7 +20,7 @@ from torch.nn import Parameter
 from . import rfa_hip
 from .projection import fused_projection_supported, linear_out, project_heads
 from .rfa import RFA
-from .utils import (EPS, SCALE, build_random_matrices, random_project,
+from .utils import (EPS, SCALE, build_random_matrices, random_project, random_project_pair,
                     upgrade_state_dict_named)
 
 
@@ -225,8 +225,7 @@ class CausalAttention(nn.Module):
             if s is None and tgt_len > 1:
                 # prefill: one pass of the training kernels over the prompt, final state kept
                 with torch.no_grad():
-                    phi_q = random_project(x=q, random_matrices=w)
-                    phi_k = random_project(x=k, random_matrices=w)
+                    phi_q, phi_k = random_project_pair(x0=q, x1=k, random_matrices=w)
                     pad = _drop_scalar_mask(key_padding_mask)
                     if pad is not None:
                         phi_k = phi_k.masked_fill(pad.to(torch.bool).transpose(0, 1)[:, :, None, None], 0.0)
@@ -259,8 +258,7 @@ class CausalAttention(nn.Module):
             attn = attn.to(x.dtype).view(tgt_len, bsz, embed_dim)
             saved_state["prev_s"], saved_state["prev_z"] = s, z
         else:
-            phi_q = random_project(x=q, random_matrices=w)
-            phi_k = random_project(x=k, random_matrices=w)
+            phi_q, phi_k = random_project_pair(x0=q, x1=k, random_matrices=w)
             if self.cuda_causal_rfa:
                 attn = cuda_causal_rfa(phi_q=phi_q, phi_k=phi_k, v=v, key_padding_mask=key_padding_mask)
             else:

@@ -784,12 +784,13 @@ int feature_bwd_blocks(int64_t R, int H) {
 }
 
 template <int D, int DH>
-int launch_feature_fwd(const rfa::half_t* x, const rfa::half_t* w, rfa::half_t* phi, int R, int H, float scale,
-                       hipStream_t st) {
+int launch_feature_fwd(const rfa::half_t* x, const rfa::half_t* w, rfa::half_t* phi, const rfa::half_t* x1,
+                       rfa::half_t* phi1, int R, int H, float scale, hipStream_t st) {
     using Cfg = rfa::FeatureCfg<D, DH>;
     auto kern = rfa::k_feature_map_fwd<D, DH>;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
-    RFA_LAUNCH(FEATURE_FWD, kern, dim3((R + 63) / 64, H), dim3(rfa::kThreads), Cfg::kFwdLds, st, x, w, phi, R, H, scale);
+    RFA_LAUNCH(FEATURE_FWD, kern, dim3((R + 63) / 64, H, x1 ? 2 : 1), dim3(rfa::kThreads), Cfg::kFwdLds, st, x, w, phi, x1,
+               phi1, R, H, scale);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -1580,7 +1581,25 @@ int rfa_feature_map_forward(const void* x, const void* w, void* phi, int64_t R, 
     auto* xh = static_cast<const rfa::half_t*>(x);
     auto* wh = static_cast<const rfa::half_t*>(w);
     auto* ph = static_cast<rfa::half_t*>(phi);
-#define RFA_CALL(DD, DH) launch_feature_fwd<DD, DH>(xh, wh, ph, (int)R, H, scale, st)
+#define RFA_CALL(DD, DH) launch_feature_fwd<DD, DH>(xh, wh, ph, nullptr, nullptr, (int)R, H, scale, st)
+    RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+int rfa_feature_map_forward_pair(const void* x0, const void* x1, const void* w, void* phi0, void* phi1, int64_t R,
+                                 int H, int D, int d, float scale, void* stream) {
+    if (int rc = check_feature_dims("rfa_feature_map_forward_pair", R, H, D, d)) return rc;
+    if (R == 0) return RFA_OK;
+    if (!x0 || !x1 || !w || !phi0 || !phi1)
+        return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_forward_pair: NULL tensor pointer");
+    if (!aligned16(x0) || !aligned16(x1) || !aligned16(w) || !aligned16(phi0) || !aligned16(phi1))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_feature_map_forward_pair: tensors must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define RFA_CALL(DD, DH)                                                                                         \
+    launch_feature_fwd<DD, DH>(static_cast<const rfa::half_t*>(x0), static_cast<const rfa::half_t*>(w),           \
+                               static_cast<rfa::half_t*>(phi0), static_cast<const rfa::half_t*>(x1),              \
+                               static_cast<rfa::half_t*>(phi1), (int)R, H, scale, st)
     RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");

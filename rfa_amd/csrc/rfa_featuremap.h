@@ -97,11 +97,16 @@ __device__ __forceinline__ void load_w_to_lds(half_t* Ws, const half_t* __restri
     }
 }
 
-// grid = (ceil(R / 64), H); wave w handles rows [64*bx + 16w, +16).
+// grid = (ceil(R / 64), H, 1 or 2); wave w handles rows [64*bx + 16w, +16).  gridDim.z = 2 maps two
+// tensors through the same W' in one launch (q and k of a module): workgroups with
+// blockIdx.z = 1 take x1 / phi1.
 template <int D, int DH>
 __global__ __launch_bounds__(kThreads) void k_feature_map_fwd(
-    const half_t* __restrict__ x, const half_t* __restrict__ w, half_t* __restrict__ phi, int R, int H,
-    float scale) {
+    const half_t* __restrict__ x0, const half_t* __restrict__ w, half_t* __restrict__ phi0,
+    const half_t* __restrict__ x1, half_t* __restrict__ phi1, int R, int H, float scale) {
+    const bool second = blockIdx.z != 0;
+    const half_t* __restrict__ x = second ? x1 : x0;
+    half_t* __restrict__ phi = second ? phi1 : phi0;
     using Cfg = FeatureCfg<D, DH>;
     constexpr int LDW = Cfg::LDW, LDP = Cfg::LDP;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_fwd(
         for (int e = 0; e < 8; ++e) ss += (float)xb[cs][e] * (float)xb[cs][e];
     }
     ss = sum_over_groups(ss);
-    const float inv = 1.0f / (sqrtf(ss) + 1e-3f);
+    const float inv = rcp_nr(sqrtf(ss) + 1e-3f);
     __syncthreads();
 
 #pragma unroll

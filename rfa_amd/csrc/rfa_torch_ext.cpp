@@ -196,6 +196,21 @@ Tensor feature_map_forward(const Tensor& x, const Tensor& w, double scale) {
     return phi;
 }
 
+std::tuple<Tensor, Tensor> feature_map_forward_pair(const Tensor& x0, const Tensor& x1, const Tensor& w, double scale) {
+    check_feature_args(x0, w);
+    check_feature_args(x1, w);
+    TORCH_CHECK(x0.sizes() == x1.sizes() && x0.device() == x1.device(), "x0 ", x0.sizes(), " and x1 ", x1.sizes(),
+                " must have one shape and device");
+    const int64_t L = x0.size(0), B = x0.size(1);
+    const int H = (int)x0.size(2), d = (int)x0.size(3), D = (int)w.size(1);
+    Tensor phi0 = torch::empty({L, B, H, 2 * D}, x0.options());
+    Tensor phi1 = torch::empty_like(phi0);
+    Launch l(x0);
+    check_rc(rfa_feature_map_forward_pair(ptr(x0), ptr(x1), ptr(w), ptr(phi0), ptr(phi1), L * B, H, D, d, (float)scale,
+                                          l.stream));
+    return {phi0, phi1};
+}
+
 std::tuple<Tensor, Tensor> feature_map_backward(const Tensor& x, const Tensor& w, const Tensor& grad_phi, double scale) {
     check_feature_args(x, w);
     const int64_t L = x.size(0), B = x.size(1);
@@ -515,6 +530,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("build_random_matrices_backward", &build_random_matrices_backward, py::arg("w"), py::arg("sigma"),
           py::arg("grad_out"), py::arg("tau"), py::arg("want_dsigma"), py::arg("want_dw"));
     m.def("feature_map_forward", &feature_map_forward, py::arg("x"), py::arg("w"), py::arg("scale"));
+    m.def("feature_map_forward_pair", &feature_map_forward_pair, py::arg("x0"), py::arg("x1"), py::arg("w"), py::arg("scale"));
     m.def("feature_map_backward", &feature_map_backward, py::arg("x"), py::arg("w"), py::arg("grad_phi"), py::arg("scale"));
     m.def("feature_map_backward_pair", &feature_map_backward_pair, py::arg("x0"), py::arg("x1"), py::arg("w"),
           py::arg("grad_phi0"), py::arg("grad_phi1"), py::arg("scale"));

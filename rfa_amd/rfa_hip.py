@@ -265,6 +265,23 @@ def feature_map_forward(x: Tensor, w: Tensor, scale: float) -> Tensor:
     return phi
 
 
+def feature_map_forward_pair(x0: Tensor, x1: Tensor, w: Tensor, scale: float):
+    """(phi(x0), phi(x1)) through the same w in one launch; x0, x1 fp16 of one shape [L, B, H, d]."""
+    _check_feature_args(x0, w)
+    _check_feature_args(x1, w)
+    _require(x0.shape == x1.shape and x0.device == x1.device, ValueError,
+             lambda: f"x0 {tuple(x0.shape)} and x1 {tuple(x1.shape)} must have one shape and device")
+    L, B, H, d = x0.shape
+    D = w.shape[1]
+    phi0 = torch.empty((L, B, H, 2 * D), dtype=torch.float16, device=x0.device)
+    phi1 = torch.empty_like(phi0)
+    with _on_device(x0.device):
+        _lib.check(_lib.load().rfa_feature_map_forward_pair(
+            x0.data_ptr(), x1.data_ptr(), w.data_ptr(), phi0.data_ptr(), phi1.data_ptr(), L * B, H, D, d, float(scale),
+            _stream_ptr(x0.device)))
+    return phi0, phi1
+
+
 def project_feature_map(x: Tensor, weights, biases, want_phi, w: Optional[Tensor], heads: int, scale: float,
                         keep_y: bool = True):
     """Linear projections of x to heads, with the feature map applied to some of them, in one launch.
@@ -609,6 +626,7 @@ def masked_backward(phi_q: Tensor, phi_k: Tensor, v: Tensor, grad_attn: Tensor, 
 # ---------------------------------------------------------------------------
 _BOUND = ("supported", "feature_map_supported", "selftest_layout", "forward", "backward", "prefill", "forward_save",
           "backward_saved", "build_random_matrices", "build_random_matrices_backward", "feature_map_forward",
+          "feature_map_forward_pair",
           "feature_map_backward", "feature_map_backward_pair", "project_feature_map", "linear_weight_grad", "cross_state",
           "cross_state_backward", "cross_readout", "cross_readout_backward", "incremental", "incremental_fused",
           "masked_forward", "masked_backward")
@@ -626,9 +644,17 @@ def _resolve_ext():
     if _ext is None:
         import importlib
         try:
-            _ext = importlib.import_module(__package__ + "._rfa_hip_ext")   # built by rfa_amd.build.build_ext
+            mod = importlib.import_module(__package__ + "._rfa_hip_ext")   # built by rfa_amd.build.build_ext
         except ImportError:
-            _ext = None
+            mod = None
+        if mod is not None and not all(hasattr(mod, n) for n in _BOUND):
+            # built from older sources than this file (the build itself imports the package first):
+            # unusable until rebuilt, and a rebuilt file needs a fresh process to be loaded
+            import warnings
+            warnings.warn("rfa_amd._rfa_hip_ext is older than rfa_hip.py (missing entry points); using the ctypes "
+                          "binding -- rebuild with `python -m rfa_amd.build`", RuntimeWarning)
+            mod = None
+        _ext = mod
     return _ext
 
 

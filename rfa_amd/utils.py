@@ -128,6 +128,38 @@ class _FeatureMap(torch.autograd.Function):
         return dx.to(ctx.in_dtypes[0]), dw.to(ctx.in_dtypes[1]), None
 
 
+class _FeatureMapPair(torch.autograd.Function):
+    """phi of two tensors of one shape through the same matrices: one launch forward, one backward
+    (with one reduction for the sum of both dW')."""
+
+    @staticmethod
+    def forward(ctx, x0: Tensor, x1: Tensor, w: Tensor, scale: float):
+        ctx.in_dtypes = (x0.dtype, x1.dtype, w.dtype)
+        ctx.scale = scale
+        x0h, x1h = x0.to(torch.float16).contiguous(), x1.to(torch.float16).contiguous()
+        wh = w.to(torch.float16).contiguous()
+        ctx.save_for_backward(x0h, x1h, wh)
+        phi0, phi1 = rfa_hip.feature_map_forward_pair(x0h, x1h, wh, scale)
+        return phi0.to(x0.dtype), phi1.to(x1.dtype)
+
+    @staticmethod
+    def backward(ctx, g0: Tensor, g1: Tensor):
+        x0h, x1h, wh = ctx.saved_tensors
+        dx0, dx1, dw = rfa_hip.feature_map_backward_pair(x0h, x1h, wh, g0.to(torch.float16).contiguous(),
+                                                         g1.to(torch.float16).contiguous(), ctx.scale)
+        return dx0.to(ctx.in_dtypes[0]), dx1.to(ctx.in_dtypes[1]), dw.to(ctx.in_dtypes[2]), None
+
+
+def random_project_pair(*, x0: Tensor, x1: Tensor, random_matrices: Tensor, scale: float = SCALE):
+    """(random_project(x=x0, ...), random_project(x=x1, ...)) for two tensors of one shape that go
+    through the same matrices -- the q and k of causal_attention.py:241-248 -- in one launch each
+    way.  Same values and gradients as the two calls."""
+    if x0.shape != x1.shape or x0.device != x1.device:
+        return (random_project(x=x0, random_matrices=random_matrices, scale=scale),
+                random_project(x=x1, random_matrices=random_matrices, scale=scale))
+    return _FeatureMapPair.apply(x0, x1, random_matrices, scale)
+
+
 def random_project(*, x: Tensor, random_matrices: Tensor, scale: float = SCALE) -> Tensor:
     """phi(x) = scale * [sin(W x^), cos(W x^)] (reference utils.py:105-120).
 

@@ -43,6 +43,30 @@ def test_feature_map_forward(L, B, H, d, D):
 
 
 @pytest.mark.parametrize("L,B,H,d,D", FEATURE_SHAPES)
+def test_feature_map_forward_pair(L, B, H, d, D):
+    """phi(q) and phi(k) in one launch: the bits of the two single launches; through
+    random_project_pair also the gradients of the two random_project calls (dW' summed)."""
+    from rfa_amd import rfa_hip
+    from rfa_amd.utils import random_project, random_project_pair
+    x0 = (_randn(L, B, H, d, seed=30 + L) * 1.7).half().cuda()
+    x1 = (_randn(L, B, H, d, seed=31 + L) * 0.6).half().cuda()
+    w = (_randn(H, D, d, seed=32) * 0.9).half().cuda()
+    print(f"phi fwd pair L={L} B={B} H={H} d={d} D={D}", flush=True)
+    p0, p1 = rfa_hip.feature_map_forward_pair(x0, x1, w, O.SCALE)
+    assert torch.equal(p0, rfa_hip.feature_map_forward(x0, w, O.SCALE))
+    assert torch.equal(p1, rfa_hip.feature_map_forward(x1, w, O.SCALE))
+    g0, g1 = _randn(L, B, H, 2 * D, seed=33).half().cuda(), _randn(L, B, H, 2 * D, seed=34).half().cuda()
+    a0, a1, aw = (t.clone().requires_grad_(True) for t in (x0, x1, w))
+    q0, q1 = random_project_pair(x0=a0, x1=a1, random_matrices=aw)
+    torch.autograd.backward([q0, q1], [g0, g1])
+    b0, b1, bw = (t.clone().requires_grad_(True) for t in (x0, x1, w))
+    torch.autograd.backward([random_project(x=b0, random_matrices=bw), random_project(x=b1, random_matrices=bw)], [g0, g1])
+    assert torch.equal(q0, p0) and torch.equal(q1, p1)
+    assert torch.equal(a0.grad, b0.grad) and torch.equal(a1.grad, b1.grad)
+    assert _rel(aw.grad.float().cpu(), bw.grad.float().cpu()) <= 2e-3     # one fp32 sum rounded once instead of two rounded sums added
+
+
+@pytest.mark.parametrize("L,B,H,d,D", FEATURE_SHAPES)
 def test_feature_map_backward(L, B, H, d, D):
     from rfa_amd import rfa_hip
     x = (_randn(L, B, H, d, seed=20 + L) * 1.3).half()
