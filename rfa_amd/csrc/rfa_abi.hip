@@ -98,11 +98,11 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // every code path at small sizes.  -1 = the heuristic.  The environment is read once, when the
 // first knob is looked up, never on the launch path; rfa_tuning_set changes a knob afterwards.
 namespace tune {
-enum Key { NSEG, PREFIX, NSEG_SAME, FREE_WG, PROJECT_STREAMING, SLICED, RECOMPUTE, PREFIX_COST, COUNT };
-const char* const kNames[COUNT] = {"nseg", "prefix", "nseg_same", "free_wg", "project_streaming", "sliced", "recompute", "prefix_cost"};
+enum Key { NSEG, PREFIX, NSEG_SAME, FREE_WG, PROJECT_STREAMING, SLICED, RECOMPUTE, PREFIX_COST, FEATURE_WG, COUNT };
+const char* const kNames[COUNT] = {"nseg", "prefix", "nseg_same", "free_wg", "project_streaming", "sliced", "recompute", "prefix_cost", "feature_wg"};
 const char* const kEnv[COUNT] = {"RFA_HIP_NSEG", "RFA_HIP_PREFIX", "RFA_HIP_NSEG_SAME", "RFA_HIP_FREE_WG",
                                  "RFA_HIP_PROJECT_STREAMING", "RFA_HIP_SLICED", "RFA_HIP_RECOMPUTE",
-                                 "RFA_HIP_PREFIX_COST"};
+                                 "RFA_HIP_PREFIX_COST", "RFA_HIP_FEATURE_WG"};
 std::atomic<int> value[COUNT];
 std::once_flag once;
 
@@ -775,9 +775,11 @@ WGradPlan make_wgrad_plan(int64_t R, int Eo, int Ei, int np) {
 }
 
 // ---- feature map launchers ---------------------------------------------------------
-int feature_bwd_blocks(int64_t R, int H) {
+int feature_bwd_blocks(int64_t R, int H, int ntens = 1) {
     const int64_t nrb = (R + 63) / 64;
-    int64_t nblk = (512 + H - 1) / H;   // about two workgroups per CU; few partial sums to reduce
+    int64_t target = 512;               // about two workgroups per CU; few partial sums to reduce
+    if (tune::get(tune::FEATURE_WG) >= 1) target = tune::get(tune::FEATURE_WG);
+    int64_t nblk = (target + (int64_t)H * ntens - 1) / ((int64_t)H * ntens);
     if (nblk > nrb) nblk = nrb;
     if (nblk < 1) nblk = 1;
     return (int)nblk;
@@ -800,8 +802,8 @@ int launch_feature_bwd(const rfa::half_t* x, const rfa::half_t* w, const rfa::ha
                        const rfa::half_t* x1, const rfa::half_t* gphi1, rfa::half_t* dx1,
                        float* dw, float* part, int R, int H, float scale, hipStream_t st) {
     using Cfg = rfa::FeatureCfg<D, DH>;
-    const int nblk = feature_bwd_blocks(R, H);
     const int ntens = x1 ? 2 : 1;       // two tensors through the same w: one launch, one reduction
+    const int nblk = feature_bwd_blocks(R, H, ntens);
     auto kern = rfa::k_feature_map_bwd<D, DH>;
     if (int rc = set_lds(kern, Cfg::kBwdLds)) return rc;
     RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H, ntens), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, x1, gphi1,
