@@ -336,6 +336,14 @@ int rfa_incremental_out(const void* phi_q, const void* phi_k, const void* v, con
 int rfa_incremental_fused_out(const void* q, const void* k, const void* v, const void* w, float scale,
                               const float* s_in, const float* z_in, float* s_out, float* z_out, void* out,
                               int64_t steps, int64_t B, int H, int D, int d, void* stream);
+/* The same step for callers whose q, k and v come out of ONE projection (a Linear layer whose
+ * weight stacks q_proj, k_proj, v_proj of causal_attention.py:228-247: one small-M GEMM per token
+ * instead of three): qkv fp16 [steps, B, 3, H, d], i.e. rows of 3 * H * d with q, k, v in their
+ * thirds.  State read from s_in, z_in and written to s_out, z_out, which may be the same
+ * buffers (in place).  Same results as rfa_incremental_fused(_out) on the three thirds. */
+int rfa_incremental_qkv(const void* qkv, const void* w, float scale, const float* s_in, const float* z_in,
+                        float* s_out, float* z_out, void* out, int64_t steps, int64_t B, int H, int D, int d,
+                        void* stream);
 
 /* ---------------------------------------------------------------------------
  * Per-kernel timing (no counterpart in the reference; used by bench.py).

@@ -78,6 +78,7 @@ SIGNATURES = {
     "rfa_incremental_fused": (c_int, [c_void_p] * 4 + [c_float] + [c_void_p] * 3 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
     "rfa_incremental_out": (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int, c_int, c_void_p]),
     "rfa_incremental_fused_out": (c_int, [c_void_p] * 4 + [c_float] + [c_void_p] * 5 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
+    "rfa_incremental_qkv": (c_int, [c_void_p] * 2 + [c_float] + [c_void_p] * 5 + [c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
 }
 
 _lib = None

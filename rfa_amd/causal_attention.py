@@ -14,6 +14,7 @@ import math
 from typing import Dict, Optional
 
 import torch
+import torch.nn.functional as F
 from torch import Tensor, nn
 from torch.nn import Parameter
 
@@ -190,6 +191,51 @@ class CausalAttention(nn.Module):
     def _heads(self, t: Tensor, tgt_len: int, bsz: int) -> Tensor:
         return t.contiguous().view(tgt_len, bsz, self.num_heads, self.head_dim)
 
+    # ---- inference-time caches ------------------------------------------------------------------
+    # Decoding calls forward once per token with the same parameters: what depends on the parameters
+    # alone is then kept between calls (only while autograd is off), keyed by the storage address
+    # and version counter of every tensor it was made from, so an optimizer step, load_state_dict
+    # or another random_matrices tensor makes it anew.
+    @staticmethod
+    def _tensor_key(t: Optional[Tensor]):
+        return None if t is None else (t.data_ptr(), t._version, t.dtype, tuple(t.shape), str(t.device))
+
+    def _cached(self, name: str, key, make):
+        cache = self.__dict__.setdefault("_inference_cache", {})
+        hit = cache.get(name)
+        if hit is None or hit[0] != key:
+            hit = (key, make())
+            cache[name] = hit
+        return hit[1]
+
+    def _scaled_matrices(self, random_matrices: Tensor) -> Tensor:
+        sigma = self.sigma if self.reparam_proj else None
+        make = lambda: build_random_matrices(random_matrices=random_matrices, tau=self.tau, sigma=sigma,
+                                             reparam_proj=self.reparam_proj)
+        if torch.is_grad_enabled():
+            return make()
+        key = (self._tensor_key(random_matrices), self._tensor_key(sigma), self.tau, self.reparam_proj)
+        return self._cached("w", key, make)
+
+    def _stacked_qkv(self):
+        """(weight [3E, E], bias [3E] or None) of one Linear layer that computes q_proj, k_proj and v_proj at once."""
+        layers = (self.q_proj, self.k_proj, self.v_proj)
+        key = tuple(self._tensor_key(t) for layer in layers for t in (layer.weight, layer.bias))
+
+        def make():
+            weight = torch.cat([layer.weight.detach() for layer in layers], 0).contiguous()
+            biases = [layer.bias for layer in layers]
+            bias = None if any(b is None for b in biases) else torch.cat([b.detach() for b in biases], 0).contiguous()
+            return weight, bias
+        return self._cached("qkv", key, make)
+
+    def _packed_decode_ok(self, x: Tensor) -> bool:
+        layers = (self.q_proj, self.k_proj, self.v_proj)
+        with_bias = [layer.bias is not None for layer in layers]
+        return (not torch.is_grad_enabled() and x.is_cuda and x.dtype == torch.float16
+                and all(layer.weight.dtype == torch.float16 for layer in layers)
+                and (all(with_bias) or not any(with_bias)))
+
     def forward(self, x: Tensor, random_matrices: Tensor, key_padding_mask: Optional[Tensor] = None,
                 attn_mask: Optional[Tensor] = None,
                 saved_state: Optional[Dict[str, Optional[Tensor]]] = None) -> Tensor:
@@ -203,9 +249,25 @@ class CausalAttention(nn.Module):
         """
         tgt_len, bsz, embed_dim = x.size()
         assert embed_dim == self.embed_dim
-        w = build_random_matrices(random_matrices=random_matrices, tau=self.tau,
-                                  sigma=self.sigma if self.reparam_proj else None,
-                                  reparam_proj=self.reparam_proj)
+        w = self._scaled_matrices(random_matrices)
+        if saved_state is not None and saved_state.get("prev_s") is not None and self._packed_decode_ok(x):
+            # a decoding step without autograd: q, k, v of the token(s) from one stacked projection (one
+            # small-M GEMM instead of three), and feature map + state update + readout in one kernel per step
+            feat = 2 * self.proj_dim
+            s_in, z_in = saved_state["prev_s"], saved_state["prev_z"]
+            assert z_in is not None
+            s = s_in.to(torch.float32).contiguous()
+            z = z_in.to(torch.float32).contiguous()
+            s_out = z_out = None
+            if not self.decode_inplace and (s is s_in or z is z_in):
+                s_out, z_out = torch.empty_like(s), torch.empty_like(z)
+            weight, bias = self._stacked_qkv()
+            rows = F.linear(x, weight, bias).view(tgt_len, bsz, 3, self.num_heads, self.head_dim)
+            attn = rfa_hip.incremental_qkv(rows, w.to(torch.float16).contiguous(), SCALE, s, z, s_out, z_out)
+            if s_out is not None:
+                s, z = s_out, z_out
+            saved_state["prev_s"], saved_state["prev_z"] = s, z
+            return linear_out(attn.view(tgt_len, bsz, embed_dim), self.out_proj)
         qkv = (self.q_proj, self.k_proj, self.v_proj)
         if self.fuse_projections and saved_state is None and fused_projection_supported(x, qkv, self.num_heads, w):
             # the three projections, the view to heads and phi of q and k in one launch

@@ -684,11 +684,16 @@ int launch_masked_bwd(const rfa::half_t* q, const rfa::half_t* k, const rfa::hal
 }
 
 // ---- decode launchers --------------------------------------------------------------
+// packed: q, k, v are the three thirds of rows of width 3 * H * DH (the output of one projection
+// whose weight stacks the three); otherwise separate contiguous tensors
 template <int KD, int DH, bool FUSED>
 int launch_decode(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t* v, const rfa::half_t* w,
                   float scale, int H, const float* s_in, const float* z_in, float* s, float* z, rfa::half_t* out,
-                  int64_t steps, int64_t N, hipStream_t st) {
-    const int64_t qk_step = FUSED ? N * DH : N * KD;
+                  int64_t steps, int64_t N, bool packed, hipStream_t st) {
+    const int64_t B = N / H;
+    const int64_t qk_bstride = packed ? (int64_t)3 * H * DH : (int64_t)H * (FUSED ? DH : KD);
+    const int64_t v_bstride = packed ? (int64_t)3 * H * DH : (int64_t)H * DH;
+    const int64_t qk_step = B * qk_bstride, v_step = B * v_bstride;
     // A step's q, k, v rows sit between its state loads and its state stores (the feature map
     // needs them first).  In a decoder they were written a moment ago; in a multi-step call they
     // are read for the first time, and that memory latency is then on every workgroup's critical
@@ -698,12 +703,17 @@ int launch_decode(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t*
     for (int64_t t = 0; t < steps; ++t) {
         if (steps > 1 && t % kTouchSteps == 0) {
             const int64_t m = (steps - t < kTouchSteps) ? steps - t : kTouchSteps;
-            RFA_LAUNCH(DECODE_TOUCH, rfa::k_touch_rows, dim3(256), dim3(rfa::kThreads), 0, st,
-                       reinterpret_cast<const uint4*>(q + t * qk_step), reinterpret_cast<const uint4*>(k + t * qk_step),
-                       reinterpret_cast<const uint4*>(v + t * N * DH), m * qk_step / 8, m * qk_step / 8, m * N * DH / 8);
+            if (packed)
+                RFA_LAUNCH(DECODE_TOUCH, rfa::k_touch_rows, dim3(256), dim3(rfa::kThreads), 0, st,
+                           reinterpret_cast<const uint4*>(q + t * qk_step), (const uint4*)nullptr, (const uint4*)nullptr,
+                           m * qk_step / 8, (int64_t)0, (int64_t)0);
+            else
+                RFA_LAUNCH(DECODE_TOUCH, rfa::k_touch_rows, dim3(256), dim3(rfa::kThreads), 0, st,
+                           reinterpret_cast<const uint4*>(q + t * qk_step), reinterpret_cast<const uint4*>(k + t * qk_step),
+                           reinterpret_cast<const uint4*>(v + t * v_step), m * qk_step / 8, m * qk_step / 8, m * v_step / 8);
         }
         RFA_LAUNCH(DECODE_STEP, (rfa::k_decode_step<KD, DH, FUSED>), dim3((unsigned)N), dim3(rfa::kThreads), 0, st,
-                           q + t * qk_step, k + t * qk_step, v + t * N * DH, w, scale, H,
+                           q + t * qk_step, k + t * qk_step, v + t * v_step, w, scale, H, qk_bstride, v_bstride,
                            t == 0 ? s_in : (const float*)s, t == 0 ? z_in : (const float*)z, s, z, out + t * N * DH);
     }
     RFA_HIP_TRY(hipGetLastError());
@@ -1457,7 +1467,7 @@ static int incremental_impl(const char* fn, const void* phi_q, const void* phi_k
     auto* kh = static_cast<const rfa::half_t*>(phi_k);
     auto* vh = static_cast<const rfa::half_t*>(v);
     auto* oh = static_cast<rfa::half_t*>(out);
-#define RFA_CALL(KD, DH) launch_decode<KD, DH, false>(qh, kh, vh, nullptr, 0.f, 1, s_in, z_in, s, z, oh, steps, N, st)
+#define RFA_CALL(KD, DH) launch_decode<KD, DH, false>(qh, kh, vh, nullptr, 0.f, 1, s_in, z_in, s, z, oh, steps, N, false, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
@@ -1475,7 +1485,7 @@ int rfa_incremental_out(const void* phi_q, const void* phi_k, const void* v, con
 
 static int incremental_fused_impl(const char* fn, const void* q, const void* k, const void* v, const void* w, float scale,
                                   const float* s_in, const float* z_in, float* s, float* z, void* out, int64_t steps,
-                                  int64_t B, int H, int D, int d, void* stream) {
+                                  int64_t B, int H, int D, int d, void* stream, bool packed = false) {
     if (int rc = check_cross_dims(fn, steps, B, H, 2 * D, d)) return rc;
     const int64_t N = B * H;
     if (steps == 0 || N == 0) return RFA_OK;
@@ -1490,7 +1500,7 @@ static int incremental_fused_impl(const char* fn, const void* q, const void* k, 
     auto* wh = static_cast<const rfa::half_t*>(w);
     auto* oh = static_cast<rfa::half_t*>(out);
     const int K = 2 * D;
-#define RFA_CALL(KD, DH) launch_decode<KD, DH, true>(qh, kh, vh, wh, scale, H, s_in, z_in, s, z, oh, steps, N, st)
+#define RFA_CALL(KD, DH) launch_decode<KD, DH, true>(qh, kh, vh, wh, scale, H, s_in, z_in, s, z, oh, steps, N, packed, st)
     RFA_DISPATCH_KD(K, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");
@@ -1506,6 +1516,16 @@ int rfa_incremental_fused_out(const void* q, const void* k, const void* v, const
                               int64_t steps, int64_t B, int H, int D, int d, void* stream) {
     return incremental_fused_impl("rfa_incremental_fused_out", q, k, v, w, scale, s_in, z_in, s_out, z_out, out, steps,
                                   B, H, D, d, stream);
+}
+
+int rfa_incremental_qkv(const void* qkv, const void* w, float scale, const float* s_in, const float* z_in,
+                        float* s_out, float* z_out, void* out, int64_t steps, int64_t B, int H, int D, int d,
+                        void* stream) {
+    if (H <= 0 || d <= 0) return fail(RFA_ERR_BAD_SHAPE, "rfa_incremental_qkv: bad sizes H=%d d=%d", H, d);
+    const rfa::half_t* base = static_cast<const rfa::half_t*>(qkv);
+    const int64_t E = (int64_t)H * d;
+    return incremental_fused_impl("rfa_incremental_qkv", base, base ? base + E : nullptr, base ? base + 2 * E : nullptr, w,
+                                  scale, s_in, z_in, s_out, z_out, out, steps, B, H, D, d, stream, true);
 }
 
 // ---- random matrices ----------------------------------------------------------------

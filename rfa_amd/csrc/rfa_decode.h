@@ -54,7 +54,7 @@ __device__ __forceinline__ void decode_feature_map(float* phi_q, float* phi_k,
 #pragma unroll
     for (int o = 1; o < TPP; o <<= 1) dot += __shfl_xor(dot, o, 64);
     if (part == 0) {
-        const float u = dot / (sqrtf(ss) + 1e-3f);
+        const float u = dot * rcp_nr(sqrtf(ss) + 1e-3f);
         float s_, c_;
         fast_sincos(u, s_, c_);
         float* dst = (vec == 0 ? phi_q : phi_k);
@@ -64,13 +64,15 @@ __device__ __forceinline__ void decode_feature_map(float* phi_q, float* phi_k,
 }
 
 // grid = N = bsz * heads.  FUSED: q, k are raw [N, DH] rows and w is [H, D, DH];
-// otherwise q, k are feature rows [N, KD] and w is unused.
-// s_in/s_out ([N, KD, DH] fp32) and z_in/z_out ([N, KD] fp32) may alias.
+// otherwise q, k are feature rows [N, KD] and w is unused.  The rows of batch entry b, head h
+// start at b * qk_bstride + h * (row width) (v: b * v_bstride + h * DH): H * width for separate
+// contiguous tensors, three times that where q, k, v are the three thirds of one projection's
+// output rows.  s_in/s_out ([N, KD, DH] fp32) and z_in/z_out ([N, KD] fp32) may alias.
 template <int KD, int DH, bool FUSED>
 __global__ __launch_bounds__(kThreads) void k_decode_step(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
-    const half_t* __restrict__ w, float scale, int H, const float* s_in, const float* z_in,
-    float* s_out, float* z_out, half_t* __restrict__ out) {
+    const half_t* __restrict__ w, float scale, int H, int64_t qk_bstride, int64_t v_bstride, const float* s_in,
+    const float* z_in, float* s_out, float* z_out, half_t* __restrict__ out) {
     using Cfg = DecodeCfg<KD, DH>;
     constexpr int CQ = Cfg::CQ, RPP = Cfg::RPP, NR = Cfg::NR;
     __shared__ float phi_q[KD];
@@ -80,6 +82,10 @@ __global__ __launch_bounds__(kThreads) void k_decode_step(
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int n = blockIdx.x;
     const int cq = tid % CQ, kr = tid / CQ;
+    const int b_ = n / H, h_ = n % H;
+    constexpr int QKW = FUSED ? DH : KD;          // width of a q / k row
+    const int64_t qk_off = (int64_t)b_ * qk_bstride + (int64_t)h_ * QKW;
+    const int64_t v_off = (int64_t)b_ * v_bstride + (int64_t)h_ * DH;
 
     // issue the state loads first: they are the long pole
     const float* sp = s_in + (int64_t)n * KD * DH;
@@ -88,15 +94,14 @@ __global__ __launch_bounds__(kThreads) void k_decode_step(
     for (int r = 0; r < NR; ++r) st[r] = *reinterpret_cast<const f4*>(sp + (int64_t)(kr + r * RPP) * DH + 4 * cq);
     float zv = 0.f;
     if (tid < KD) zv = z_in[(int64_t)n * KD + tid];
-    h4 vh = *reinterpret_cast<const h4*>(v + (int64_t)n * DH + 4 * cq);
+    h4 vh = *reinterpret_cast<const h4*>(v + v_off + 4 * cq);
 
     if (FUSED) {
-        decode_feature_map<KD, DH>(phi_q, phi_k, q + (int64_t)n * DH, k + (int64_t)n * DH,
-                                   w + (int64_t)(n % H) * (KD / 2) * DH, scale, tid);
+        decode_feature_map<KD, DH>(phi_q, phi_k, q + qk_off, k + qk_off, w + (int64_t)h_ * (KD / 2) * DH, scale, tid);
     } else {
         if (tid < KD) {
-            phi_q[tid] = (float)q[(int64_t)n * KD + tid];
-            phi_k[tid] = (float)k[(int64_t)n * KD + tid];
+            phi_q[tid] = (float)q[qk_off + tid];
+            phi_k[tid] = (float)k[qk_off + tid];
         }
     }
     __syncthreads();

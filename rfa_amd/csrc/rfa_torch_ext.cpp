@@ -460,6 +460,29 @@ Tensor incremental_fused(const Tensor& q, const Tensor& k, const Tensor& v, cons
     return out;
 }
 
+Tensor incremental_qkv(const Tensor& qkv, const Tensor& w, double scale, const Tensor& s, const Tensor& z,
+                       const c10::optional<Tensor>& s_out, const c10::optional<Tensor>& z_out) {
+    check_half("qkv", qkv, 5);
+    check_half("random_matrices", w, 3);
+    const int64_t steps = qkv.size(0), B = qkv.size(1), H = qkv.size(3), d = qkv.size(4), D = w.size(1);
+    TORCH_CHECK_VALUE(qkv.size(2) == 3, "qkv must be [steps, bsz, 3, heads, head_dim]");
+    TORCH_CHECK_VALUE(w.size(0) == H && w.size(2) == d, "random_matrices must be [heads, proj_dim, head_dim]");
+    check_f32("s", s, {B, H, 2 * D, d});
+    check_f32("z", z, {B, H, 2 * D});
+    TORCH_CHECK_VALUE(s_out.has_value() == z_out.has_value(), "s_out and z_out go together");
+    if (s_out.has_value()) {
+        check_f32("s_out", *s_out, {B, H, 2 * D, d});
+        check_f32("z_out", *z_out, {B, H, 2 * D});
+    }
+    Tensor out = torch::empty({steps, B, H, d}, qkv.options());
+    Launch l(qkv);
+    check_rc(rfa_incremental_qkv(ptr(qkv), ptr(w), (float)scale, s.data_ptr<float>(), z.data_ptr<float>(),
+                                 s_out.has_value() ? s_out->data_ptr<float>() : s.data_ptr<float>(),
+                                 z_out.has_value() ? z_out->data_ptr<float>() : z.data_ptr<float>(), ptr(out), steps, B,
+                                 (int)H, (int)D, (int)d, l.stream));
+    return out;
+}
+
 // ---- quadratic form with explicit masks -------------------------------------------------------
 std::tuple<Tensor, Tensor> masked_forward(const Tensor& phi_q, const Tensor& phi_k, const Tensor& v, int64_t H,
                                           const c10::optional<Tensor>& pad, const c10::optional<Tensor>& attn_mask_bytes) {
@@ -547,6 +570,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("s_out") = py::none(), py::arg("z_out") = py::none());
     m.def("incremental_fused", &incremental_fused, py::arg("q"), py::arg("k"), py::arg("v"), py::arg("w"), py::arg("scale"),
           py::arg("s"), py::arg("z"), py::arg("s_out") = py::none(), py::arg("z_out") = py::none());
+    m.def("incremental_qkv", &incremental_qkv, py::arg("qkv"), py::arg("w"), py::arg("scale"), py::arg("s"), py::arg("z"),
+          py::arg("s_out") = py::none(), py::arg("z_out") = py::none());
     m.def("masked_forward", &masked_forward, py::arg("phi_q"), py::arg("phi_k"), py::arg("v"), py::arg("H"),
           py::arg("key_padding_mask") = py::none(), py::arg("attn_mask_bytes") = py::none());
     m.def("masked_backward", &masked_backward, py::arg("phi_q"), py::arg("phi_k"), py::arg("v"), py::arg("grad_attn"),

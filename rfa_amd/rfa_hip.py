@@ -554,6 +554,33 @@ def incremental_fused(q: Tensor, k: Tensor, v: Tensor, w: Tensor, scale: float, 
     return out
 
 
+def incremental_qkv(qkv: Tensor, w: Tensor, scale: float, s: Tensor, z: Tensor,
+                    s_out: Optional[Tensor] = None, z_out: Optional[Tensor] = None) -> Tensor:
+    """incremental_fused for q, k, v that are the three thirds of one projection's output rows:
+    qkv fp16 [steps, B, 3, H, d] (one Linear layer with the q, k, v weights stacked).  Returns
+    attn fp16 [steps, B, H, d]."""
+    _check_half_cuda("qkv", qkv, 5)
+    _check_half_cuda("random_matrices", w, 3)
+    steps, B, three, H, d = qkv.shape
+    D = w.shape[1]
+    _require(three == 3, ValueError, lambda: f"qkv must be [steps, bsz, 3, heads, head_dim] (got {tuple(qkv.shape)})")
+    _require(w.shape[0] == H and w.shape[2] == d, ValueError, lambda: "random_matrices must be [heads, proj_dim, head_dim]")
+    _check_f32_cuda("s", s, (B, H, 2 * D, d))
+    _check_f32_cuda("z", z, (B, H, 2 * D))
+    _require((s_out is None) == (z_out is None), ValueError, lambda: "s_out and z_out go together")
+    if s_out is None:
+        s_out, z_out = s, z
+    else:
+        _check_f32_cuda("s_out", s_out, (B, H, 2 * D, d))
+        _check_f32_cuda("z_out", z_out, (B, H, 2 * D))
+    out = torch.empty((steps, B, H, d), dtype=torch.float16, device=qkv.device)
+    with _on_device(qkv.device):
+        _lib.check(_lib.load().rfa_incremental_qkv(
+            qkv.data_ptr(), w.data_ptr(), float(scale), s.data_ptr(), z.data_ptr(), s_out.data_ptr(), z_out.data_ptr(),
+            out.data_ptr(), steps, B, H, D, d, _stream_ptr(qkv.device)))
+    return out
+
+
 # ---------------------------------------------------------------------------
 # quadratic form with explicit masks (masked_rfa)
 # ---------------------------------------------------------------------------
@@ -629,6 +656,7 @@ _BOUND = ("supported", "feature_map_supported", "selftest_layout", "forward", "b
           "feature_map_forward_pair",
           "feature_map_backward", "feature_map_backward_pair", "project_feature_map", "linear_weight_grad", "cross_state",
           "cross_state_backward", "cross_readout", "cross_readout_backward", "incremental", "incremental_fused",
+          "incremental_qkv",
           "masked_forward", "masked_backward")
 _CTYPES_IMPL = {name: globals()[name] for name in _BOUND}
 _active = "ctypes"

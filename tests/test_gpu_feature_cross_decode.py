@@ -317,3 +317,33 @@ def test_incremental_matches_oracle(B, H, d, D, prefill, steps):
                                      v[prefill:].cuda().contiguous(), W.half().cuda(), O.SCALE, s, z).float().cpu()
     assert (out2.reshape(steps, N, d) - want[prefill:]).abs().max().item() <= OUT_ATOL
     assert _rel(s.cpu().reshape(N, K, d), ws) <= 2e-3
+
+
+@pytest.mark.usefixtures("binding")
+@pytest.mark.parametrize("B,H,d,D,steps", [(2, 4, 64, 64, 5), (3, 2, 128, 64, 3), (1, 3, 64, 128, 70), (64, 16, 64, 64, 2)])
+def test_incremental_qkv_equals_the_step_on_separate_tensors(B, H, d, D, steps):
+    """q, k, v as the three thirds of one projection's output rows ([steps, B, 3, H, d]): the bits of
+    incremental_fused on contiguous copies of the thirds, in place and into a second state, over
+    single-step calls and one multi-step call (which streams the packed rows ahead of the steps)."""
+    from rfa_amd import rfa_hip
+    K = 2 * D
+    qkv = (_randn(steps, B, 3, H, d, seed=900 + steps) * 0.7).half().cuda()
+    W = O.make_w(d, D, H).half().cuda()
+    s0 = (_randn(B, H, K, d, seed=901) * 0.3).cuda()
+    z0 = (_randn(B, H, K, seed=902).abs() * 2.0).cuda()
+    q, k, v = (qkv[:, :, i].contiguous() for i in range(3))
+    print(f"decode packed B={B} H={H} d={d} D={D} steps={steps}", flush=True)
+    s1, z1 = s0.clone(), z0.clone()
+    want = rfa_hip.incremental_fused(q, k, v, W, O.SCALE, s1, z1)
+    s2, z2 = s0.clone(), z0.clone()
+    got = rfa_hip.incremental_qkv(qkv, W, O.SCALE, s2, z2)
+    assert torch.equal(got, want) and torch.equal(s2, s1) and torch.equal(z2, z1)
+    s3, z3 = s0.clone(), z0.clone()
+    so, zo = torch.empty_like(s0), torch.empty_like(z0)
+    rows = []
+    for t in range(min(steps, 4)):           # one call per token, state into a second pair of tensors
+        rows.append(rfa_hip.incremental_qkv(qkv[t:t + 1].contiguous(), W, O.SCALE, s3, z3, so, zo))
+        s3, z3, so, zo = so, zo, s3, z3
+    assert torch.equal(torch.cat(rows), want[:len(rows)])
+    with pytest.raises(Exception, match="3, heads"):
+        rfa_hip.incremental_qkv(qkv[:, :, :2].contiguous(), W, O.SCALE, s2, z2)

@@ -123,6 +123,59 @@ def test_causal_module_decode_leaves_earlier_states_alone():
         assert half_state["prev_s"].dtype == torch.float32 and torch.equal(keep, held[2][0].half())
 
 
+def test_causal_module_decode_from_one_stacked_projection():
+    """Without autograd a decoding step takes q, k, v from one Linear layer whose weight stacks the
+    three projections, and keeps that weight and the scaled random matrices between calls.  Same
+    numbers as the step with three projections (one fp16 rounding of a projection apart); a
+    parameter changed in place, or another random_matrices tensor, is seen by the next call."""
+    from rfa_amd import CausalAttention, rfa_hip
+    torch.manual_seed(5)
+    T, B, E, H, d, D = 12, 3, 128, 2, 64, 64
+    m = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half().eval()
+    x = torch.randn(T, B, E).cuda().half()
+    W = O.make_w(d, D, H).cuda().half()
+    calls = []
+    real = rfa_hip.incremental_qkv
+
+    def spy(*a, **kw):
+        calls.append(1)
+        return real(*a, **kw)
+    rfa_hip.incremental_qkv = spy
+    try:
+        with torch.no_grad():
+            state, rows = {}, []
+            for t in range(T):
+                rows.append(m(x[t:t + 1], W, saved_state=state))
+        assert len(calls) == T - 1                      # the first token finds no state and takes the general path
+        m.requires_grad_(True)
+        state2, rows2 = {}, []
+        for t in range(T):                              # autograd on: three projections, nothing cached
+            rows2.append(m(x[t:t + 1], W, saved_state=state2).detach())
+        assert len(calls) == T - 1
+        a, b = torch.cat(rows).float(), torch.cat(rows2).float()
+        assert (a - b).abs().max().item() <= 4e-3
+        assert _rel(state["prev_s"], state2["prev_s"]) <= 2e-3
+        with torch.no_grad():
+            before = m(x[3:4], W, saved_state=dict(state))
+            again = m(x[3:4], W, saved_state=dict(state))
+            assert torch.equal(before, again)
+            m.q_proj.weight.mul_(1.5)                   # in place: the version counter moves, the stacked weight is rebuilt
+            changed = m(x[3:4], W, saved_state=dict(state))
+            assert not torch.equal(before, changed)
+            ref_state = dict(state)
+            m.requires_grad_(True)
+        with torch.enable_grad():
+            want = m(x[3:4], W, saved_state=ref_state).detach()
+        assert (changed.float() - want.float()).abs().max().item() <= 4e-3
+        with torch.no_grad():
+            other = m(x[3:4], (W * 0.5).contiguous(), saved_state=dict(state))      # another matrix tensor: W' rebuilt
+            m.sigma.mul_(0.8)
+            other2 = m(x[3:4], (W * 0.5).contiguous(), saved_state=dict(state))
+        assert not torch.equal(other, changed) and not torch.equal(other2, other)
+    finally:
+        rfa_hip.incremental_qkv = real
+
+
 def test_causal_module_training_step_runs_and_matches_oracle():
     from rfa_amd import CausalAttention
     torch.manual_seed(1)
