@@ -417,7 +417,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_fwd(
                 float dr = dparts[i];
 #pragma unroll
                 for (int h = 1; h < NH; ++h) dr += dparts[h * C + i];
-                const float inv = 1.0f / fmaxf(CAUSAL ? dr : fabsf(dr), 1.0f);
+                const float inv = rcp_nr(fmaxf(CAUSAL ? dr : fabsf(dr), 1.0f));
                 if (t0 + i < t_end) {
                     if (CAUSAL && den_out && w == 0 && G == 0) den_out[(int64_t)(t0 + i) * N + n] = dr;
 #pragma unroll
@@ -1071,7 +1071,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
         // ---- phase C: P rows of this wave; G <- G/den in place
         {
             const int i = 16 * rb + row;
-            const float inv = 1.0f / dens[i];
+            const float inv = rcp_nr(dens[i]);
             const float gzi = gzs[i];
 #pragma unroll
             for (int a = 0; a < (CAUSAL ? JPW : 0); ++a) {
@@ -1089,7 +1089,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
             for (int it = 0; it < ChunkRegs<DH, NT>::kPieces; ++it) {
                 const int p = tid + NT * it;
                 const int r_ = p / PPR, c8 = p % PPR;
-                const float sc = 1.0f / dens[r_];
+                const float sc = rcp_nr(dens[r_]);
                 h8 x = *reinterpret_cast<const h8*>(Gs + r_ * LDV + c8 * 8);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) x[e] = (half_t)((float)x[e] * sc);
@@ -1110,7 +1110,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq(
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const int i = 16 * it + row;
-                const float inv = 1.0f / dens[i];
+                const float inv = rcp_nr(dens[i]);
                 const float gzi = gzs[i];
                 h8 bp0, bp1;
                 if (CAUSAL) {
@@ -1306,21 +1306,11 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dq_saved(
         for (int it = 0; it < VP; ++it) {
             const int pc = tid + NT * it;
             const int r_ = pc / PPR, c8 = pc % PPR;
-            union { uint4 u; h8 h; } xg, xo;
-            xg.u = rg.v[it];
-            xo.u = ro.v[it];
-            float dot = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) dot += (float)xg.h[e] * (float)xo.h[e];
-#pragma unroll
-            for (int m = 1; m < PPR; m <<= 1) dot += __shfl_xor(dot, m, 64);
+            const float dot = sum_adjacent<PPR>(dot_h8(rg.v[it], ro.v[it]));
             const bool valid = r_ < rg.rows;
-            const float inv = valid ? 1.0f / fmaxf(dn[it], 1.0f) : 0.f;
+            const float inv = valid ? rcp_nr(fmaxf(dn[it], 1.0f)) : 0.f;
             const float gzv = (valid && dn[it] > 1.0f) ? -dot * inv : 0.f;
-            h8 y;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)xg.h[e] * inv);
-            *reinterpret_cast<h8*>(Gs + r_ * LDV + c8 * 8) = y;
+            *reinterpret_cast<uint4*>(Gs + r_ * LDV + c8 * 8) = scale_h8(rg.v[it], inv);
             if (c8 == 0) {
                 gzs[r_] = gzv;
                 if (valid && koff == 0) gz_ws[(int64_t)(t0 + r_) * N + n] = gzv;
@@ -1669,7 +1659,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
             chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
 #pragma unroll
             for (int it = 0; it < ChunkRegs<DH, NT>::kPieces; ++it)
-                inv_den[it] = 1.0f / fmaxf(inv_den[it], 1.0f);   // den_ws may hold raw or clamped denominators
+                inv_den[it] = rcp_nr(fmaxf(inv_den[it], 1.0f));   // den_ws may hold raw or clamped denominators
             chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
             if (tid < C) gzs[tid] = tid < rg.rows ? gz_next : 0.f;
         }
@@ -1949,7 +1939,7 @@ __device__ __forceinline__ void dkdv_role_dk(
         chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
         chunk_r2s<DH, NT>(rv, Vs, LDV, tid);
 #pragma unroll
-        for (int it = 0; it < VP; ++it) inv_den[it] = 1.0f / fmaxf(inv_den[it], 1.0f);
+        for (int it = 0; it < VP; ++it) inv_den[it] = rcp_nr(fmaxf(inv_den[it], 1.0f));
         chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
         if (tid < C) gzs[tid] = tid < rg.rows ? gz_next : 0.f;
         if (row == 0) {
@@ -2122,7 +2112,7 @@ __device__ __forceinline__ void dkdv_role_dv(
         chunk_r2s<KD, NT>(rk, Ks, LDQ, tid);
         chunk_r2s<KD, NT>(rq, Qs, LDQ, tid);
 #pragma unroll
-        for (int it = 0; it < VP; ++it) inv_den[it] = 1.0f / fmaxf(inv_den[it], 1.0f);
+        for (int it = 0; it < VP; ++it) inv_den[it] = rcp_nr(fmaxf(inv_den[it], 1.0f));
         chunk_r2s_scaled<DH, NT>(rg, inv_den, Gs, LDV, tid);
         __syncthreads();
         if (ci > 0) prefetch_a(t0 - C);

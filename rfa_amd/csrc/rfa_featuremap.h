@@ -375,10 +375,23 @@ __global__ __launch_bounds__(kThreads) void k_build_random_matrices_dsigma(const
         const int c = c0 + lane;
         float acc = 0.f;
         if (c < d) {
-#pragma unroll 8
-            for (int j = slice; j < D; j += 4) {     // unrolled: the loads of eight rows are in flight together
-                const half_t t = (half_t)((float)gh[j * d + c] / tau);
-                acc += (float)(half_t)((float)t * (float)wh[j * d + c]);
+            // the kernel is one memory round trip after another: request the rows of a whole group (16 rows
+            // of g and of w per thread) before the first is used, so that D = 64 takes one trip
+            for (int j0 = slice; j0 < D; j0 += 64) {
+                half_t gv[16], wv[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    const int j = min(j0 + 4 * u, D - 1);
+                    gv[u] = gh[j * d + c];
+                    wv[u] = wh[j * d + c];
+                }
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    if (j0 + 4 * u < D) {
+                        const half_t t = (half_t)((float)gv[u] / tau);
+                        acc += (float)(half_t)((float)t * (float)wv[u]);
+                    }
+                }
             }
         }
         red[slice][lane] = acc;
