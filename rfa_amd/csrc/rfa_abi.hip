@@ -386,12 +386,12 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
         // one launch that needs none
         rfa::SegBounds bounds{};
         if (allow_recompute && !savedS && recompute_bounds(T, p.nseg, &bounds) &&
-            (int64_t)rfa::kChunk * N * KD * 2 < ((int64_t)1 << 32)) {
+            (int64_t)rfa::kChunk * N * (KD > DH ? KD : DH) * 2 < ((int64_t)1 << 32)) {
             auto kern = rfa::k_causal_fwd_pipe<KD, DH, true>;
             if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
             RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(512), rfa::FwdPipeCfg<KD, DH>::kLds, st, q, k, v, out,
                        (const float*)nullptr, (const float*)nullptr, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, 0,
-                       savedHdr, pw, bounds);
+                       savedHdr, pw, bounds, 0);
             RFA_HIP_TRY(hipGetLastError());
             return RFA_OK;
         }
@@ -412,7 +412,7 @@ int launch_forward(const rfa::half_t* q, const rfa::half_t* k, const rfa::half_t
         if (int rc = set_lds(kern, rfa::FwdPipeCfg<KD, DH>::kLds)) return rc;
         RFA_LAUNCH(CAUSAL_FWD, kern, dim3(N * p.nseg), dim3(512), rfa::FwdPipeCfg<KD, DH>::kLds, st, q, k, v, out,
                            wsS, wsZ, savedDen, final_s, final_z, T, N, p.nseg, p.seg_len, p.prefixed, savedHdr, pw,
-                           rfa::SegBounds{});
+                           rfa::SegBounds{}, (int64_t)rfa::kChunk * N * (KD > DH ? KD : DH) * 2 >= ((int64_t)1 << 32) ? 1 : 0);
     } else {
         auto kern = rfa::k_causal_fwd<KD, DH, NW, true>;
         if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;

@@ -509,7 +509,9 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
     const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
     half_t* __restrict__ out, const float* __restrict__ wsS, const float* __restrict__ wsZ,
     float* __restrict__ den_out, float* __restrict__ final_s, float* __restrict__ final_z, int T, int N,
-    int nseg, int seg_len, int prefixed, int* __restrict__ hdr_out, PlanWords plan, SegBounds bounds) {
+    int nseg, int seg_len, int prefixed, int* __restrict__ hdr_out, PlanWords plan, SegBounds bounds, int wide_rows) {
+    // wide_rows: 64 rows of a tensor span 4 GiB or more, beyond the 32-bit lane offsets of the
+    // full-chunk loads; every chunk then takes the clamped 64-bit row addresses (never with RECOMPUTE)
     plan_write(hdr_out, plan);
     using Cfg = FwdPipeCfg<KD, DH>;
     constexpr int NT = 256;      // threads per group
@@ -634,7 +636,8 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
             if (live) {
                 const int t0 = t_begin + it * C;
                 const int rows_next = t_end - t0 - C;
-                if (rows_next >= C) pq_.load_full(rq, (int64_t)(t0 + C) * k_stride);
+                const bool fast_rows = rows_next >= C && !wide_rows;
+                if (fast_rows) pq_.load_full(rq, (int64_t)(t0 + C) * k_stride);
                 else if (rows_next > 0) chunk_g2r<KD, NT>(rq, qb + (int64_t)(t0 + C) * k_stride, k_stride, rows_next, tid);
                 RFA_TICK_AT(3, 0);
                 // rows i in [16w, 16w+16) of A as A^T tiles (m=j, n=i), all four j tiles
@@ -647,7 +650,7 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
 #pragma unroll
                     for (int a = 0; a < 4; ++a) at[a] = mfma32(row8(Ks, LDQ, 16 * a + row, ks * 32, G), bq, at[a]);
                 }
-                if (rows_next >= C) {         // second part of the next chunk's rows
+                if (fast_rows) {              // second part of the next chunk's rows
                     pk_.load_full(rk, (int64_t)(t0 + C) * k_stride);
                     pv_.load_full(rv, (int64_t)(t0 + C) * v_stride);
                 } else if (rows_next > 0) {
@@ -705,7 +708,6 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
         }
     } else {
         half_t* ob = out + (int64_t)n * DH;
-        const unsigned out_lane_off = (unsigned)row * (unsigned)(N * DH * 2) + 8u * G;   // bytes: row of a 16-step tile, 4 halves from 4G
         f4 S[NKT][NCT];
 #pragma unroll
         for (int a = 0; a < NKT; ++a)
@@ -809,7 +811,7 @@ __global__ __launch_bounds__(512) void k_causal_fwd_pipe(
                         for (int ct = 0; ct < NCT; ++ct) {
                             f4 o = acc[i4][ct];
                             o[0] *= inv; o[1] *= inv; o[2] *= inv; o[3] *= inv;
-                            store_lane(ob + (int64_t)(t0 + 16 * i4) * v_stride + w * DS + 16 * ct, out_lane_off, to_h4(o));
+                            *reinterpret_cast<h4*>(ob + (int64_t)(t0 + i) * v_stride + w * DS + 16 * ct + 4 * G) = to_h4(o);
                         }
                     }
                 }

@@ -40,6 +40,24 @@ def test_rfa_apply_autograd_matches_oracle_grad_check_recipe():
     assert torch.equal(RFA.forward_cuda(cq.detach(), ck.detach(), cv.detach()), out.detach())
 
 
+def test_rfa_forward_matches_oracle_grad_check_forward_recipe():
+    """The forward recipe of the reference's grad_check.py (:17-28): T=50, one sequence, K=128, d=64,
+    U(-.5,.5) inputs that are NOT normalised, seed 3, compared with forward_torch under the
+    reference's own pass rule."""
+    from rfa_amd import RFA
+    torch.manual_seed(3)
+    T, N, K, d = 50, 1, 128, 64
+    q, k, v = ((torch.rand(T, N, n) - .5).half() for n in (K, K, d))
+    ref = O.causal_forward_cumsum(q.float(), k.float(), v.float())
+    cq, ck, cv = (t.cuda() for t in (q, k, v))
+    out = RFA.forward_cuda(cq, ck, cv)
+    assert ((out.float().cpu() - ref) ** 2 < 1e-4).all()
+    # outputs reach |out| ~ 10 with these inputs, where one fp16 step is 7.8e-3: within one rounding of the fp32 value
+    assert ((out.float().cpu() - ref).abs() <= 1e-3 * ref.abs().clamp_min(1.0)).all()
+    # forward_torch, the formula the reference compares its kernel with, on the same device tensors
+    assert ((RFA.forward_torch(cq.float(), ck.float(), cv.float()).cpu() - ref) ** 2 < 1e-4).all()
+
+
 def test_functional_chain_with_padding_mask_and_grads():
     """random_project -> cuda_causal_rfa with a key padding mask, gradients down to the
     raw q, k, v and the random matrix."""
