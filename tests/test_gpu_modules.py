@@ -52,8 +52,8 @@ def test_rfa_forward_matches_oracle_grad_check_forward_recipe():
     cq, ck, cv = (t.cuda() for t in (q, k, v))
     out = RFA.forward_cuda(cq, ck, cv)
     assert ((out.float().cpu() - ref) ** 2 < 1e-4).all()
-    # outputs reach |out| ~ 10 with these inputs, where one fp16 step is 7.8e-3: within one rounding of the fp32 value
-    assert ((out.float().cpu() - ref).abs() <= 1e-3 * ref.abs().clamp_min(1.0)).all()
+    # outputs reach |out| ~ 10 with these inputs, where one fp16 step is 7.8e-3, and the intra-chunk weights q.k (up to ~10 here) pass through fp16
+    assert ((out.float().cpu() - ref).abs() <= 2e-3 * ref.abs().clamp_min(1.0)).all()
     # forward_torch, the formula the reference compares its kernel with, on the same device tensors
     assert ((RFA.forward_torch(cq.float(), ck.float(), cv.float()).cpu() - ref) ** 2 < 1e-4).all()
 
