@@ -154,9 +154,9 @@ def main():
     achieved = dom_bytes / (kern_us[dominant] * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": _profile_traffic_bytes({"k_causal_fwd": "k_causal_fwd_pipe<128, 64>",
+                "traffic": _profile_traffic_bytes({"k_causal_fwd": "k_causal_fwd_pipe<128, 64, true>",
                                                    "k_segment_state": "k_segment_state<128, 64, 4, true, false>",
-                                                   "k_sliced_bwd": "k_sliced_bwd<128, 64>"}.get(dominant, dominant + "<")),
+                                                   "k_sliced_bwd": "k_sliced_bwd<128, 64, 64>"}.get(dominant, dominant + "<")),
                 "traffic_source": TRAFFIC_PROFILE + " (FETCH_SIZE + WRITE_SIZE of this kernel at this shape, a profile run "
                                   "of this file, not measured in this run)",
                 "bytes_per_launch": dom_bytes, "avg_us": round(kern_us[dominant], 2),

@@ -108,7 +108,7 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int grp = w < 4 ? 0 : 1 + (w - 4) / NPW;      // loader | NPW dQ waves | NPW dK waves
     const int wf = w & 3;                       // loader: row block of the P tiles
-    const int tid = threadIdx.x & (NT - 1);     // thread inside the loader group
+    const int tid = (w & 3) * 64 + lane;        // thread inside the loader group
     const int row = lane & 15, G = lane >> 4;
     const int kl0 = 32 * ((w - 4) % NPW);       // product waves: first of this wave's 32 features, local to the slice arrays
     const unsigned out_lane_off = (unsigned)row * (unsigned)(N * KD * 2) + 8u * G;   // bytes: row `row` of a 16-step tile, 4 halves from 4G
@@ -446,10 +446,10 @@ __device__ __forceinline__ void sliced_bwd_dv(
     constexpr size_t kStage = Cfg::kLds / 2;
 
     const int lane = threadIdx.x & 63;
+    if ((threadIdx.x >> 6) >= 8) return;        // the role has 8 waves; the launch may carry more for the other role
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (w >= 8) return;                         // the role has 8 waves; the launch may carry more for the other role
     const int grp = w >> 2, wc = w & 3;         // loader: column block of the A^T tiles
-    const int tid = threadIdx.x & (NT - 1);
+    const int tid = (w & 3) * 64 + lane;
     const int row = lane & 15, G = lane >> 4;
     const int jh = (w >> 1) & 1;                // product waves 4..7: half of the chunk's rows ...
     const int cl0 = 32 * (w & 1);               // ... and first of this wave's 32 columns, local to the slice array
