@@ -795,14 +795,30 @@ int feature_bwd_blocks(int64_t R, int H, int ntens = 1) {
     return (int)nblk;
 }
 
+// Workgroups along x for the streaming feature-map kernels: eight waves each, a wave per group of
+// 16 rows, one workgroup per CU in all (their registers leave room for one; a second round of
+// workgroups would pay the staging of W' and, in the backward, the sum over the waves again);
+// more rows make the waves walk further.  Never more than feature_bwd_blocks, which sizes the
+// workspace of the backward's partial sums.
+int feature_stream_blocks(int64_t R, int H, int ntens, int waves = rfa::kFeatureWaves) {
+    const int64_t ngrp = (R + 15) / 16, full = (ngrp + waves - 1) / waves;
+    int64_t target = std::min(device_cus(), 512);
+    if (tune::get(tune::FEATURE_WG) >= 1) target = tune::get(tune::FEATURE_WG);
+    int64_t nblk = (target + (int64_t)H * ntens - 1) / ((int64_t)H * ntens);
+    if (nblk > full) nblk = full;
+    if (nblk < 1) nblk = 1;
+    return (int)nblk;
+}
+
 template <int D, int DH>
 int launch_feature_fwd(const rfa::half_t* x, const rfa::half_t* w, rfa::half_t* phi, const rfa::half_t* x1,
                        rfa::half_t* phi1, int R, int H, float scale, hipStream_t st) {
     using Cfg = rfa::FeatureCfg<D, DH>;
     auto kern = rfa::k_feature_map_fwd<D, DH>;
+    const int ntens = x1 ? 2 : 1;
     if (int rc = set_lds(kern, Cfg::kFwdLds)) return rc;
-    RFA_LAUNCH(FEATURE_FWD, kern, dim3((R + 63) / 64, H, x1 ? 2 : 1), dim3(rfa::kThreads), Cfg::kFwdLds, st, x, w, phi, x1,
-               phi1, R, H, scale);
+    RFA_LAUNCH(FEATURE_FWD, kern, dim3(feature_stream_blocks(R, H, ntens), H, ntens), dim3(rfa::kFeatureThreads), Cfg::kFwdLds,
+               st, x, w, phi, x1, phi1, R, H, scale);
     RFA_HIP_TRY(hipGetLastError());
     return RFA_OK;
 }
@@ -811,13 +827,23 @@ template <int D, int DH>
 int launch_feature_bwd(const rfa::half_t* x, const rfa::half_t* w, const rfa::half_t* gphi, rfa::half_t* dx,
                        const rfa::half_t* x1, const rfa::half_t* gphi1, rfa::half_t* dx1,
                        float* dw, float* part, int R, int H, float scale, hipStream_t st) {
-    using Cfg = rfa::FeatureCfg<D, DH>;
     const int ntens = x1 ? 2 : 1;       // two tensors through the same w: one launch, one reduction
-    const int nblk = feature_bwd_blocks(R, H, ntens);
-    auto kern = rfa::k_feature_map_bwd<D, DH>;
-    if (int rc = set_lds(kern, Cfg::kBwdLds)) return rc;
-    RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H, ntens), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, x1, gphi1,
-               dx1, part, R, H, scale);
+    int nblk;
+    if constexpr (rfa::FeatureStreamCfg<D, DH>::kFits) {
+        using Cfg = rfa::FeatureStreamCfg<D, DH>;
+        nblk = feature_stream_blocks(R, H, ntens, rfa::kFeatureBwdWaves);      // never more than feature_bwd_blocks, which sized the workspace
+        auto kern = rfa::k_feature_map_bwd_stream<D, DH>;
+        if (int rc = set_lds(kern, Cfg::kLds)) return rc;
+        RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H, ntens), dim3(rfa::kFeatureBwdThreads), Cfg::kLds, st, x, w, gphi, dx, x1,
+                   gphi1, dx1, part, R, H, scale);
+    } else {
+        using Cfg = rfa::FeatureCfg<D, DH>;
+        nblk = feature_bwd_blocks(R, H, ntens);
+        auto kern = rfa::k_feature_map_bwd<D, DH>;
+        if (int rc = set_lds(kern, Cfg::kBwdLds)) return rc;
+        RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H, ntens), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, x1, gphi1,
+                   dx1, part, R, H, scale);
+    }
     const int64_t elems = (int64_t)H * D * DH;
     static_assert((D * DH) % 256 == 0, "dw reduce works on blocks of 256 elements");
     RFA_LAUNCH(FEATURE_DW_REDUCE, rfa::k_feature_map_dw_reduce, dim3((unsigned)(elems / 256)), dim3(rfa::kThreads), 0, st,

@@ -205,12 +205,16 @@ __device__ __forceinline__ h8 h8_ones() {
 // |u| rarely above 10; the error of x * (1/2pi) in fp32 (2^-24 relative) and of the unit
 // itself stay below 1e-6 absolute there, far inside the fp16 resolution of the outputs
 // (3e-4 relative at |phi| ~ 0.1).  About ten times fewer instructions than sincosf.
-__device__ __forceinline__ void fast_sincos(float x, float& s, float& c) {
-    float t = x * 0.15915494309189535f;
-    t = t - floorf(t);                  // v_fract: keeps the unit inside its valid range
+//
+// sin and cos of 2 pi t.  The hardware functions take their argument in turns and are valid on
+// [-256, 256]: the fractional part (one instruction) keeps any t inside.
+__device__ __forceinline__ void sincos_turns(float t, float& s, float& c) {
+    t = __builtin_amdgcn_fractf(t);
     s = __builtin_amdgcn_sinf(t);
     c = __builtin_amdgcn_cosf(t);
 }
+
+__device__ __forceinline__ void fast_sincos(float x, float& s, float& c) { sincos_turns(x * 0.15915494309189535f, s, c); }
 
 // sum over the four 16-lane groups (lanes i, i+16, i+32, i+48)
 // Sum of the per-segment slots [s_first, s_last) of a carried state.  A loop that loads and adds one

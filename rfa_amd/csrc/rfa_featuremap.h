@@ -23,7 +23,7 @@ struct FeatureCfg {
     // 8-byte fragment writes of 16 rows over all banks
     static constexpr int LDP = 2 * D + 16;
     static constexpr int LDG = (2 * D > DH ? 2 * D : DH) + 16;   // backward: grad_phi rows in, dx rows out
-    static constexpr size_t kFwdLds = (size_t)(D * LDW + 64 * LDP) * 2;
+    static constexpr size_t kFwdLds = (size_t)(D * LDW) * 2;                                     // W' only
     static constexpr size_t kBwdLds = (size_t)(D * LDW + 64 * LDW + 64 * LDU + 64 * LDG) * 2;
 };
 
@@ -97,66 +97,107 @@ __device__ __forceinline__ void load_w_to_lds(half_t* Ws, const half_t* __restri
     }
 }
 
-// grid = (ceil(R / 64), H, 1 or 2); wave w handles rows [64*bx + 16w, +16).  gridDim.z = 2 maps two
-// tensors through the same W' in one launch (q and k of a module): workgroups with
-// blockIdx.z = 1 take x1 / phi1.
+// ---- streaming kernels: waves that never wait for each other ---------------------------------
+// A wave owns groups of 16 rows of one head and walks them with a stride; W' sits in LDS, read
+// only.  Nothing a wave writes is read by another wave, so the row loop has no workgroup barrier.
+//
+// "Pair order": MFMA tile t of 16 features (or of 16 input columns) is made of the indices
+//     32 (t / 2) + 8 G + 4 (t % 2) + e        at accumulator position m = 4 G + e,
+// so that the accumulators of tiles 2p and 2p+1 together give lane (i, G) the 8 consecutive
+// indices 32 p + 8 G .. + 7 of row i: 16 bytes that go to (and come from) global memory
+// directly, without a pass through LDS to re-form rows.  pair_pos(f) is the row of the operand
+// matrix that holds index f.
+constexpr int kFeatureWaves = 8;
+constexpr int kFeatureThreads = 64 * kFeatureWaves;
+
+__host__ __device__ constexpr int pair_pos(int f) { return (f & ~31) | ((f & 4) << 2) | ((f & 24) >> 1) | (f & 3); }
+
+// W' of one head -> LDS with its rows (features) in pair order
+template <int D, int DH, int NT = kFeatureThreads>
+__device__ __forceinline__ void load_w_pair_order(half_t* Ws, const half_t* __restrict__ wh, int tid) {
+    constexpr int LDW = FeatureCfg<D, DH>::LDW;
+    constexpr int PPR = DH / 8;
+    for (int p = tid; p < D * PPR; p += NT) {
+        const int r = p / PPR, c8 = p % PPR;
+        *reinterpret_cast<uint4*>(Ws + pair_pos(r) * LDW + c8 * 8) = *reinterpret_cast<const uint4*>(wh + r * DH + c8 * 8);
+    }
+}
+
+// grid = (nblk, H, 1 or 2); wave w of workgroup b takes the row groups 8 b + w, + 8 nblk, ...
+// gridDim.z = 2 maps two tensors through the same W' in one launch (q and k of a module):
+// workgroups with blockIdx.z = 1 take x1 / phi1.
 template <int D, int DH>
-__global__ __launch_bounds__(kThreads) void k_feature_map_fwd(
+__global__ __launch_bounds__(kFeatureThreads) void k_feature_map_fwd(
     const half_t* __restrict__ x0, const half_t* __restrict__ w, half_t* __restrict__ phi0,
     const half_t* __restrict__ x1, half_t* __restrict__ phi1, int R, int H, float scale) {
     const bool second = blockIdx.z != 0;
     const half_t* __restrict__ x = second ? x1 : x0;
     half_t* __restrict__ phi = second ? phi1 : phi0;
-    using Cfg = FeatureCfg<D, DH>;
-    constexpr int LDW = Cfg::LDW, LDP = Cfg::LDP;
+    constexpr int LDW = FeatureCfg<D, DH>::LDW;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     half_t* Ws = reinterpret_cast<half_t*>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    half_t* Ps = Ws + D * LDW + wv * 16 * LDP;     // this wave's 16 output rows
     const int i = lane & 15, G = lane >> 4;
     const int h = blockIdx.y;
-    const int r = blockIdx.x * 64 + 16 * wv + i;
 
-    load_w_to_lds<D, DH>(Ws, w + (int64_t)h * D * DH, tid);
+    load_w_pair_order<D, DH>(Ws, w + (int64_t)h * D * DH, tid);
 
-    h8 xb[DH / 32];
-    float ss = 0.f;
+    const int ngrp = (R + 15) / 16, gstride = gridDim.x * kFeatureWaves;
+    int grp = blockIdx.x * kFeatureWaves + wv;
+    // Two sets of row registers: the loads of the next group are issued into the set the
+    // current group does not use, so no set is ever copied (a third set, two groups in flight,
+    // measured no faster).  Rows past R read the last row (no branch around the loads) and are
+    // not stored.
+    struct Rows { h8 x[DH / 32]; };
+    auto issue_loads = [&](Rows& t, int g) {
+        const half_t* px = x + ((int64_t)min(g * 16 + i, R - 1) * H + h) * DH + 8 * G;
 #pragma unroll
-    for (int cs = 0; cs < DH / 32; ++cs) {
-        if (r < R) {
-            xb[cs] = *reinterpret_cast<const h8*>(x + ((int64_t)r * H + h) * DH + cs * 32 + 8 * G);
-        } else {
+        for (int cs = 0; cs < DH / 32; ++cs) t.x[cs] = *reinterpret_cast<const h8*>(px + cs * 32);
+    };
+    auto process = [&](const Rows& t, int g) {
+        const int r = g * 16 + i;
+        float ss = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) xb[cs][e] = (half_t)0.f;
+        for (int cs = 0; cs < DH / 32; ++cs) ss += dot_h8(__builtin_bit_cast(uint4, t.x[cs]), __builtin_bit_cast(uint4, t.x[cs]));
+        ss = sum_over_groups(ss);
+        const float inv_turns = rcp_nr(__builtin_amdgcn_sqrtf(ss) + 1e-3f) * 0.15915494309189535f;
+        half_t* po = phi + ((int64_t)r * H + h) * (2 * D) + 8 * G;
+#pragma unroll
+        for (int p = 0; p < D / 32; ++p) {
+            f4 acc[2] = {f4_zero(), f4_zero()};   // u^T tiles 2p, 2p+1 (m = feature, n = row)
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+#pragma unroll
+                for (int cs = 0; cs < DH / 32; ++cs)
+                    acc[q] = mfma32(row8(Ws, LDW, 32 * p + 16 * q + i, cs * 32, G), t.x[cs], acc[q]);
+            h8 sv, cv;
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float s_, c_;
+                    sincos_turns(acc[q][e] * inv_turns, s_, c_);
+                    sv[4 * q + e] = (half_t)(scale * s_);
+                    cv[4 * q + e] = (half_t)(scale * c_);
+                }
+            if (r < R) {
+                *reinterpret_cast<h8*>(po + 32 * p) = sv;
+                *reinterpret_cast<h8*>(po + D + 32 * p) = cv;
+            }
         }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ss += (float)xb[cs][e] * (float)xb[cs][e];
+    };
+    Rows ra, rb;
+    if (grp < ngrp) issue_loads(ra, grp);
+    __syncthreads();   // W' in place
+    while (grp < ngrp) {
+        if (grp + gstride < ngrp) issue_loads(rb, grp + gstride);
+        process(ra, grp);
+        if ((grp += gstride) >= ngrp) break;
+        if (grp + gstride < ngrp) issue_loads(ra, grp + gstride);
+        process(rb, grp);
+        grp += gstride;
     }
-    ss = sum_over_groups(ss);
-    const float inv = rcp_nr(sqrtf(ss) + 1e-3f);
-    __syncthreads();
-
-#pragma unroll
-    for (int jt = 0; jt < D / 16; ++jt) {
-        f4 acc = f4_zero();   // u^T tile (m = feature j, n = row)
-#pragma unroll
-        for (int cs = 0; cs < DH / 32; ++cs) acc = mfma32(row8(Ws, LDW, 16 * jt + i, cs * 32, G), xb[cs], acc);
-        h4 sv, cv;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            float s_, c_;
-            fast_sincos(acc[e] * inv, s_, c_);
-            sv[e] = (half_t)(scale * s_);
-            cv[e] = (half_t)(scale * c_);
-        }
-        *reinterpret_cast<h4*>(Ps + i * LDP + 16 * jt + 4 * G) = sv;
-        *reinterpret_cast<h4*>(Ps + i * LDP + D + 16 * jt + 4 * G) = cv;
-    }
-    // the fragment layout holds 8 bytes per lane and row: stage through LDS so that the
-    // stores to HBM cover whole 4D-byte rows
-    wave_lds_order();
-    wave_rows_s2g<2 * D>(Ps, LDP, phi, blockIdx.x * 64 + 16 * wv, R, H, h, lane);
 }
 
 // Backward.  grid = (nblk, H); workgroup (b, h) walks row blocks b, b+nblk, ...
@@ -304,6 +345,214 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
 #pragma unroll
         for (int jt = 0; jt < D / 16; ++jt)
             *reinterpret_cast<f4*>(po + (16 * jt + i) * DH + 16 * (wv * NCTW + a) + 4 * G) = dwacc[a][jt];
+}
+
+// LDS of the streaming backward: W' twice (rows in pair order for u = W' x; transposed, with the
+// input columns in pair order, for y = du W'), per wave 16 rows of x and of du for the
+// transposing reads of the dW product, and after the row loop the same bytes again as the
+// area in which the eight waves add up their dW.
+#ifndef RFA_FEATURE_BWD_WAVES
+#define RFA_FEATURE_BWD_WAVES 8
+#endif
+constexpr int kFeatureBwdWaves = RFA_FEATURE_BWD_WAVES;
+constexpr int kFeatureBwdThreads = 64 * kFeatureBwdWaves;
+
+template <int D, int DH>
+struct FeatureStreamCfg {
+    static constexpr int LDW = DH + lds_pad(DH), LDT = D + lds_pad(D);
+    // a row stride of 32 bytes mod 256 spreads the 8-byte pieces of a transposing read over all banks
+    static constexpr int LDX = DH + 16, LDU = D + 16;
+    static constexpr int kTiles = (DH / 16) * (D / 16);
+    // the whole dW'[D][DH] of a head sits in the accumulators of every wave: 4 registers per tile
+    static constexpr bool kFits = D * DH <= 4096;
+    static constexpr size_t kLoop = (size_t)(D * LDW + DH * LDT + kFeatureBwdWaves * 16 * (LDX + LDU)) * 2;
+    static constexpr size_t kReduce = (size_t)(kFeatureBwdWaves / 2) * D * DH * 4;
+    static constexpr size_t kLds = kLoop > kReduce ? kLoop : kReduce;
+};
+
+__device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) { return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0); }
+
+// Backward of the feature map, streaming form (shapes with D * DH <= 4096).  grid = (nblk, H,
+// 1 or 2) like the forward; wave w of workgroup b takes the row groups 8 b + w, + 8 nblk, ...
+// Per group of 16 rows, with n = ||x||, inv = 1 / (n + 1e-3), u = W' x inv:
+//     du  = scale (cos u * g_sin - sin u * g_cos) inv          accumulators of u, in registers
+//     y   = du W'                                               du is the MFMA operand as it stands
+//     dx  = y - x (x . y) / (n (n + 1e-3))   (0 where n = 0)    16 bytes per lane, stored directly
+//     dW' += du^T x                                             over the wave's own 16 rows (k = 16 MFMA),
+//                                                               operands by transposing LDS reads
+// x and grad_phi arrive in the lane's own operand / accumulator positions (pair order), so no
+// row is re-formed in LDS and no wave reads what another wrote: no workgroup barrier in the row
+// loop.  At the end the eight waves add their dW' through LDS and the workgroup writes one
+// partial sum, dw_part[(z nblk + b)][h]; k_feature_map_dw_reduce sums the shares.
+template <int D, int DH>
+__global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
+    const half_t* __restrict__ x0, const half_t* __restrict__ w, const half_t* __restrict__ gphi0,
+    half_t* __restrict__ dx0, const half_t* __restrict__ x1, const half_t* __restrict__ gphi1,
+    half_t* __restrict__ dx1, float* __restrict__ dw_part, int R, int H, float scale) {
+    const bool second = blockIdx.z != 0;
+    const half_t* __restrict__ x = second ? x1 : x0;
+    const half_t* __restrict__ gphi = second ? gphi1 : gphi0;
+    half_t* __restrict__ dx = second ? dx1 : dx0;
+    using Cfg = FeatureStreamCfg<D, DH>;
+    static_assert(Cfg::kFits, "dW' of one head must fit the accumulators of a wave");
+    constexpr int LDW = Cfg::LDW, LDT = Cfg::LDT, LDX = Cfg::LDX, LDU = Cfg::LDU;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    half_t* Ws = reinterpret_cast<half_t*>(smem_raw);
+    half_t* WT = Ws + D * LDW;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    half_t* Xs = WT + DH * LDT + wv * 16 * (LDX + LDU);
+    half_t* Us = Xs + 16 * LDX;
+    const int i = lane & 15, G = lane >> 4;
+    const int h = blockIdx.y;
+    const half_t* wh = w + (int64_t)h * D * DH;
+
+    load_w_pair_order<D, DH, kFeatureBwdThreads>(Ws, wh, tid);
+    for (int p = tid; p < D * DH / 8; p += kFeatureBwdThreads) {
+        const int j = p / (DH / 8), c8 = p % (DH / 8);
+        const h8 v = *reinterpret_cast<const h8*>(wh + j * DH + c8 * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) WT[pair_pos(c8 * 8 + e) * LDT + j] = v[e];
+    }
+
+    f4 dwacc[DH / 16][D / 16];   // (m = c, n = j)
+#pragma unroll
+    for (int a = 0; a < DH / 16; ++a)
+#pragma unroll
+        for (int b = 0; b < D / 16; ++b) dwacc[a][b] = f4_zero();
+
+    const int ngrp = (R + 15) / 16, gstride = gridDim.x * kFeatureBwdWaves;
+    int grp = blockIdx.x * kFeatureBwdWaves + wv;
+    // Two sets of row registers: the loads of the next group are issued into the set the
+    // current group does not use, so no set is ever copied.  Rows past R read the last row (no
+    // branch around the loads); their du is forced to 0, which keeps them out of dW', and their
+    // dx is not stored.
+    struct Rows { h8 x[DH / 32], gs[D / 32], gc[D / 32]; };
+    auto issue_loads = [&](Rows& t, int g) {
+        const int64_t row = (int64_t)min(g * 16 + i, R - 1) * H + h;
+        const half_t* px = x + row * DH + 8 * G;
+        const half_t* pg = gphi + row * (2 * D) + 8 * G;
+#pragma unroll
+        for (int cs = 0; cs < DH / 32; ++cs) t.x[cs] = *reinterpret_cast<const h8*>(px + cs * 32);
+#pragma unroll
+        for (int p = 0; p < D / 32; ++p) {
+            t.gs[p] = *reinterpret_cast<const h8*>(pg + 32 * p);
+            t.gc[p] = *reinterpret_cast<const h8*>(pg + D + 32 * p);
+        }
+    };
+    const int trow = 4 * G + (i >> 2), tcol = 4 * (i & 3);    // this lane's address in a transposing read
+    auto process = [&](const Rows& t, int g) {
+        const int r = g * 16 + i;
+        float ss = 0.f;
+#pragma unroll
+        for (int cs = 0; cs < DH / 32; ++cs) {
+            *reinterpret_cast<h8*>(Xs + i * LDX + cs * 32 + 8 * G) = t.x[cs];
+            ss += dot_h8(__builtin_bit_cast(uint4, t.x[cs]), __builtin_bit_cast(uint4, t.x[cs]));
+        }
+        ss = sum_over_groups(ss);
+        const float nrm = __builtin_amdgcn_sqrtf(ss);
+        const float inv = rcp_nr(nrm + 1e-3f);
+        const float coef = nrm > 0.f ? inv * rcp_nr(nrm) : 0.f;
+        const float inv_turns = inv * 0.15915494309189535f;
+        const float sinv = r < R ? scale * inv : 0.f;
+
+        h8 du[D / 32];
+#pragma unroll
+        for (int p = 0; p < D / 32; ++p) {
+            f4 acc[2] = {f4_zero(), f4_zero()};   // u^T tiles 2p, 2p+1 (m = feature, n = row)
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+#pragma unroll
+                for (int cs = 0; cs < DH / 32; ++cs)
+                    acc[q] = mfma32(row8(Ws, LDW, 32 * p + 16 * q + i, cs * 32, G), t.x[cs], acc[q]);
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float s_, c_;
+                    sincos_turns(acc[q][e] * inv_turns, s_, c_);
+                    du[p][4 * q + e] = (half_t)(sinv * (c_ * (float)t.gs[p][4 * q + e] - s_ * (float)t.gc[p][4 * q + e]));
+                }
+            *reinterpret_cast<h8*>(Us + i * LDU + 32 * p + 8 * G) = du[p];
+        }
+
+        // y^T tiles (m = input column in pair order, n = row)
+        f4 y[DH / 16];
+        float xdot = 0.f;
+#pragma unroll
+        for (int ct = 0; ct < DH / 16; ++ct) {
+            f4 acc = f4_zero();
+#pragma unroll
+            for (int p = 0; p < D / 32; ++p) acc = mfma32(row8(WT, LDT, 16 * ct + i, 32 * p, G), du[p], acc);
+            y[ct] = acc;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) xdot += acc[e] * (float)t.x[ct / 2][4 * (ct % 2) + e];
+        }
+        xdot = sum_over_groups(xdot) * coef;
+        half_t* po = dx + ((int64_t)r * H + h) * DH + 8 * G;
+#pragma unroll
+        for (int u = 0; u < DH / 32; ++u) {
+            h8 o;
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[4 * q + e] = (half_t)(y[2 * u + q][e] - (float)t.x[u][4 * q + e] * xdot);
+            if (r < R) *reinterpret_cast<h8*>(po + 32 * u) = o;
+        }
+
+        // dW' (m = c, n = j) += x^T du over the 16 rows of the group
+        wave_lds_order();
+        h4 xa[DH / 16];
+#pragma unroll
+        for (int a = 0; a < DH / 16; ++a) xa[a] = tr_read4(Xs + trow * LDX + 16 * a + tcol);
+#pragma unroll
+        for (int b = 0; b < D / 16; ++b) {
+            const h4 ub = tr_read4(Us + trow * LDU + 16 * b + tcol);
+#pragma unroll
+            for (int a = 0; a < DH / 16; ++a) dwacc[a][b] = mfma16(xa[a], ub, dwacc[a][b]);
+        }
+        wave_lds_order();   // before the next group's rows overwrite Xs / Us
+    };
+    Rows ra, rb;
+    if (grp < ngrp) issue_loads(ra, grp);
+    __syncthreads();   // both copies of W' in place
+    while (grp < ngrp) {
+        if (grp + gstride < ngrp) issue_loads(rb, grp + gstride);
+        process(ra, grp);
+        if ((grp += gstride) >= ngrp) break;
+        if (grp + gstride < ngrp) issue_loads(ra, grp + gstride);
+        process(rb, grp);
+        grp += gstride;
+    }
+
+    // the waves' sums -> wave 0: per round the upper half of the remaining waves hands its sums to the lower
+    f4* red = reinterpret_cast<f4*>(smem_raw);
+#pragma unroll
+    for (int n = kFeatureBwdWaves; n > 1; n = (n + 1) / 2) {
+        const int half = (n + 1) / 2;
+        __syncthreads();   // row loop (first round) / previous round's reads done
+        if (wv >= half && wv < n) {
+#pragma unroll
+            for (int a = 0; a < DH / 16; ++a)
+#pragma unroll
+                for (int b = 0; b < D / 16; ++b) red[((wv - half) * Cfg::kTiles + a * (D / 16) + b) * 64 + lane] = dwacc[a][b];
+        }
+        __syncthreads();
+        if (wv < n - half) {
+#pragma unroll
+            for (int a = 0; a < DH / 16; ++a)
+#pragma unroll
+                for (int b = 0; b < D / 16; ++b) dwacc[a][b] += red[(wv * Cfg::kTiles + a * (D / 16) + b) * 64 + lane];
+        }
+    }
+    if (wv == 0) {
+        float* out = dw_part + ((int64_t)(blockIdx.z * gridDim.x + blockIdx.x) * H + h) * D * DH;
+#pragma unroll
+        for (int a = 0; a < DH / 16; ++a)
+#pragma unroll
+            for (int b = 0; b < D / 16; ++b)
+                *reinterpret_cast<f4*>(out + (16 * b + i) * DH + 16 * a + 4 * G) = dwacc[a][b];
+    }
 }
 
 // dw[e] = sum_b dw_part[b][e].  One workgroup of 4 waves per 256 consecutive elements

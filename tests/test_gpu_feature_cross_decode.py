@@ -26,7 +26,8 @@ def _randn(*shape, seed):
 
 
 # ------------------------------------------------------------------ feature map
-FEATURE_SHAPES = [(128, 2, 4, 64, 64), (3, 1, 2, 64, 32), (70, 3, 2, 128, 128), (1, 1, 1, 64, 128), (33, 2, 3, 128, 64)]
+FEATURE_SHAPES = [(128, 2, 4, 64, 64), (3, 1, 2, 64, 32), (70, 3, 2, 128, 128), (1, 1, 1, 64, 128), (33, 2, 3, 128, 64),
+                  (45, 2, 2, 128, 32)]
 
 
 @pytest.mark.parametrize("L,B,H,d,D", FEATURE_SHAPES)
@@ -102,6 +103,35 @@ def test_feature_map_backward_pair(L, B, H, d, D):
     _, rw0 = O.random_project_backward(x0.float().cpu(), w.float().cpu(), g0.float().cpu())
     _, rw1 = O.random_project_backward(x1.float().cpu(), w.float().cpu(), g1.float().cpu())
     assert _rel(dw.cpu(), rw0 + rw1) <= GRAD_RTOL
+
+
+@pytest.mark.parametrize("L,B,H,d,D,wgs", [(333, 2, 2, 64, 64, 4), (333, 2, 2, 64, 64, 2), (100, 3, 1, 128, 32, 1),
+                                           (257, 1, 2, 64, 32, 6)])
+def test_feature_map_waves_that_walk_many_row_groups(L, B, H, d, D, wgs, knobs):
+    """With few workgroups every wave of the streaming kernels walks several groups of 16 rows
+    (ragged: some waves one group more than others, odd and even counts, a last group that is not
+    full): phi and dx carry the bits of the default launch, dW' is the same sum in another order."""
+    from rfa_amd import rfa_hip
+    x0 = (_randn(L, B, H, d, seed=40 + L) * 1.3).half().cuda()
+    x1 = (_randn(L, B, H, d, seed=41 + L) * 0.7).half().cuda()
+    w = (_randn(H, D, d, seed=42) * 0.9).half().cuda()
+    g0 = _randn(L, B, H, 2 * D, seed=43).half().cuda()
+    g1 = _randn(L, B, H, 2 * D, seed=44).half().cuda()
+    want_phi = rfa_hip.feature_map_forward_pair(x0, x1, w, O.SCALE)
+    want_dx0, want_dx1, want_dw = rfa_hip.feature_map_backward_pair(x0, x1, w, g0, g1, O.SCALE)
+    want_sx, want_sw = rfa_hip.feature_map_backward(x0, w, g0, O.SCALE)
+    knobs(feature_wg=wgs)
+    print(f"phi with {wgs} workgroups L={L} B={B} H={H} d={d} D={D}", flush=True)
+    p0, p1 = rfa_hip.feature_map_forward_pair(x0, x1, w, O.SCALE)
+    assert torch.equal(p0, want_phi[0]) and torch.equal(p1, want_phi[1])
+    assert torch.equal(rfa_hip.feature_map_forward(x1, w, O.SCALE), want_phi[1])
+    dx0, dx1, dw = rfa_hip.feature_map_backward_pair(x0, x1, w, g0, g1, O.SCALE)
+    assert torch.equal(dx0, want_dx0) and torch.equal(dx1, want_dx1)
+    assert _rel(dw.cpu(), want_dw.cpu()) <= 1e-5
+    sx, sw = rfa_hip.feature_map_backward(x0, w, g0, O.SCALE)
+    assert torch.equal(sx, want_sx) and _rel(sw.cpu(), want_sw.cpu()) <= 1e-5
+    _, rw0 = O.random_project_backward(x0.float().cpu(), w.float().cpu(), g0.float().cpu())
+    assert _rel(sw.cpu(), rw0) <= GRAD_RTOL
 
 
 @pytest.mark.parametrize("H,D,d,tau,with_sigma", [(8, 64, 64, 1.0, True), (3, 32, 128, 0.7, True),
