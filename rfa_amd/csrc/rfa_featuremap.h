@@ -6,6 +6,12 @@
 // cat, mul) by one kernel per direction.  The projection W' of one head stays
 // resident in LDS while a workgroup streams rows of x through the MFMA.
 //
+// Two forms.  Streaming (k_feature_map_fwd, k_feature_map_bwd_stream): every wave walks its own
+// groups of 16 rows, rows move between registers and global memory in the lanes' own operand
+// positions, no workgroup barrier in the row loop; the backward needs dW'[D][DH] of a head in one
+// wave's accumulators (D * DH <= 4096).  Row blocks (k_feature_map_bwd, the other shapes): four
+// waves share blocks of 64 rows through LDS and split dW' between them.
+//
 // Layouts:  x   [R, H, DH] fp16   (R = seq_len * bsz rows, row-major)
 //           w   [H, D, DH] fp16   (already sigma * W / tau, utils.py:90-97)
 //           phi [R, H, 2D] fp16   (sin block in columns [0, D), cos block in [D, 2D))
