@@ -162,8 +162,9 @@ int rfa_causal_num_segments(int64_t T, int64_t N, int K, int d);
  *             Unset: for up to 4 segments.  Its output has the bits of the one-segment scan.
  *   "prefix_cost"  cost of a rebuilt 64-step block in percent of a scanned one (default 12): moves
  *             the cut of that forward into segments
- *   "feature_wg"  workgroups the feature-map backward aims for (default 512, two per compute unit;
- *             each walks several 64-row blocks and leaves one partial dW' for the reduction)
+ *   "feature_wg"  workgroups the feature-map kernels aim for (default: one per compute unit for the
+ *             eight-wave streaming kernels, 512 for the row-block backward of the wide shapes; in
+ *             the backward each leaves one partial dW' for the reduction)
  * Initial values come from the environment variables RFA_HIP_<NAME>, read once per process and
  * never on the launch path.  No counterpart in the reference. */
 int rfa_tuning_set(const char* name, int value);
