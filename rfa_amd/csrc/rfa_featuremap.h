@@ -356,7 +356,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
 // LDS of the streaming backward: W' twice (rows in pair order for u = W' x; transposed, with the
 // input columns in pair order, for y = du W'), per wave 16 rows of x and of du for the
 // transposing reads of the dW product, and after the row loop the same bytes again as the
-// area in which the eight waves add up their dW.
+// area through which the eight waves exchange their dW (one copy of dW'[D][DH] per wave).
 #ifndef RFA_FEATURE_BWD_WAVES
 #define RFA_FEATURE_BWD_WAVES 8
 #endif
@@ -372,7 +372,7 @@ struct FeatureStreamCfg {
     // the whole dW'[D][DH] of a head sits in the accumulators of every wave: 4 registers per tile
     static constexpr bool kFits = D * DH <= 4096;
     static constexpr size_t kLoop = (size_t)(D * LDW + DH * LDT + kFeatureBwdWaves * 16 * (LDX + LDU)) * 2;
-    static constexpr size_t kReduce = (size_t)(kFeatureBwdWaves / 2) * D * DH * 4;
+    static constexpr size_t kReduce = (size_t)kFeatureBwdWaves * D * DH * 4;
     static constexpr size_t kLds = kLoop > kReduce ? kLoop : kReduce;
 };
 
@@ -388,8 +388,9 @@ __device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) { return __builtin_amdgcn
 //                                                               operands by transposing LDS reads
 // x and grad_phi arrive in the lane's own operand / accumulator positions (pair order), so no
 // row is re-formed in LDS and no wave reads what another wrote: no workgroup barrier in the row
-// loop.  At the end the eight waves add their dW' through LDS and the workgroup writes one
-// partial sum, dw_part[(z nblk + b)][h]; k_feature_map_dw_reduce sums the shares.
+// loop.  At the end the eight waves add their dW' through LDS (one exchange, every wave sums and
+// stores an eighth of the tiles) and the workgroup leaves one partial sum,
+// dw_part[(z nblk + b)][h]; k_feature_map_dw_reduce sums the shares.
 template <int D, int DH>
 __global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
     const half_t* __restrict__ x0, const half_t* __restrict__ w, const half_t* __restrict__ gphi0,
@@ -531,33 +532,22 @@ __global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
         grp += gstride;
     }
 
-    // the waves' sums -> wave 0: per round the upper half of the remaining waves hands its sums to the lower
+    // The waves' sums, one round: every wave leaves its dW' in LDS, then wave w adds up tiles
+    // w, w + 8, ... of all the waves, in wave order, and stores them.
     f4* red = reinterpret_cast<f4*>(smem_raw);
+    __syncthreads();   // every wave is out of the row loop: its LDS becomes the exchange area
 #pragma unroll
-    for (int n = kFeatureBwdWaves; n > 1; n = (n + 1) / 2) {
-        const int half = (n + 1) / 2;
-        __syncthreads();   // row loop (first round) / previous round's reads done
-        if (wv >= half && wv < n) {
+    for (int a = 0; a < DH / 16; ++a)
 #pragma unroll
-            for (int a = 0; a < DH / 16; ++a)
+        for (int b = 0; b < D / 16; ++b) red[(wv * Cfg::kTiles + a * (D / 16) + b) * 64 + lane] = dwacc[a][b];
+    __syncthreads();
+    float* out = dw_part + ((int64_t)(blockIdx.z * gridDim.x + blockIdx.x) * H + h) * D * DH;
+    for (int t = wv; t < Cfg::kTiles; t += kFeatureBwdWaves) {
+        f4 sum = red[t * 64 + lane];
 #pragma unroll
-                for (int b = 0; b < D / 16; ++b) red[((wv - half) * Cfg::kTiles + a * (D / 16) + b) * 64 + lane] = dwacc[a][b];
-        }
-        __syncthreads();
-        if (wv < n - half) {
-#pragma unroll
-            for (int a = 0; a < DH / 16; ++a)
-#pragma unroll
-                for (int b = 0; b < D / 16; ++b) dwacc[a][b] += red[(wv * Cfg::kTiles + a * (D / 16) + b) * 64 + lane];
-        }
-    }
-    if (wv == 0) {
-        float* out = dw_part + ((int64_t)(blockIdx.z * gridDim.x + blockIdx.x) * H + h) * D * DH;
-#pragma unroll
-        for (int a = 0; a < DH / 16; ++a)
-#pragma unroll
-            for (int b = 0; b < D / 16; ++b)
-                *reinterpret_cast<f4*>(out + (16 * b + i) * DH + 16 * a + 4 * G) = dwacc[a][b];
+        for (int o = 1; o < kFeatureBwdWaves; ++o) sum += red[(o * Cfg::kTiles + t) * 64 + lane];
+        const int a = t / (D / 16), b = t % (D / 16);
+        *reinterpret_cast<f4*>(out + (16 * b + i) * DH + 16 * a + 4 * G) = sum;
     }
 }
 
