@@ -217,6 +217,19 @@ int rfa_feature_map_backward_pair(const void* x0, const void* x1, const void* w,
                                   int D, int d, float scale, void* workspace, size_t workspace_bytes,
                                   void* stream);
 
+/* The same launch for the backward of a module's three input projections
+ * (causal_attention.py:228-247 under autograd, where the gradients of q_proj's, k_proj's and
+ * v_proj's outputs each meet their weight in a GEMM of their own): with E = H * d, `packed` is
+ * fp16 [R, 3E] and receives  [ dx0 | dx1 | third ]  side by side -- dx0, dx1 as above, `third` (fp16
+ * [R, E], e.g. the gradient of v; may be NULL: that block is left untouched) copied by further
+ * workgroups of the launch -- so that one product  packed x [Wq; Wk; Wv]  gives the gradient of the
+ * projections' input and one  packed^T x  all three weight gradients.  dw and the workspace as for
+ * rfa_feature_map_backward_pair. */
+int rfa_feature_map_backward_pair_packed(const void* x0, const void* x1, const void* w, const void* grad_phi0,
+                                         const void* grad_phi1, const void* third, void* packed, float* dw,
+                                         int64_t R, int H, int D, int d, float scale, void* workspace,
+                                         size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Linear projections to heads with the feature map in the epilogue.
  *

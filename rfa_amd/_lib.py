@@ -59,6 +59,7 @@ SIGNATURES = {
     "rfa_feature_map_backward": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p]),
     "rfa_feature_map_backward_pair_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int]),
     "rfa_feature_map_backward_pair": (c_int, [c_void_p] * 8 + [c_int64, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p]),
+    "rfa_feature_map_backward_pair_packed": (c_int, [c_void_p] * 8 + [c_int64, c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p]),
     "rfa_project_feature_map": (c_int, [c_void_p] * 5 + [c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "rfa_linear_weight_grad_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int]),
     "rfa_linear_weight_grad": (c_int, [c_void_p] * 4 + [c_int, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p]),

@@ -19,6 +19,7 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import rfa_hip
+from ._derived import derived
 from .projection import fused_projection_supported, linear_out, project_heads
 from .rfa import RFA
 from .utils import (EPS, SCALE, build_random_matrices, random_project, random_project_pair,
@@ -193,20 +194,12 @@ class CausalAttention(nn.Module):
 
     # ---- inference-time caches ------------------------------------------------------------------
     # Decoding calls forward once per token with the same parameters: what depends on the parameters
-    # alone is then kept between calls (only while autograd is off), keyed by the storage address
-    # and version counter of every tensor it was made from, so an optimizer step, load_state_dict
-    # or another random_matrices tensor makes it anew.
-    @staticmethod
-    def _tensor_key(t: Optional[Tensor]):
-        return None if t is None else (t.data_ptr(), t._version, t.dtype, tuple(t.shape), str(t.device))
-
-    def _cached(self, name: str, key, make):
-        cache = self.__dict__.setdefault("_inference_cache", {})
-        hit = cache.get(name)
-        if hit is None or hit[0] != key:
-            hit = (key, make())
-            cache[name] = hit
-        return hit[1]
+    # alone is then kept between calls (only while autograd is off) for as long as every tensor it
+    # was made from is the same object in the same state (version counter, address, dtype, shape),
+    # so an optimizer step, load_state_dict, a replaced parameter or another random_matrices tensor
+    # makes it anew.
+    def _cached(self, name: str, sources, extra, make):
+        return derived(self.__dict__.setdefault("_inference_cache", {}), name, sources, extra, make)
 
     def _scaled_matrices(self, random_matrices: Tensor) -> Tensor:
         sigma = self.sigma if self.reparam_proj else None
@@ -214,20 +207,18 @@ class CausalAttention(nn.Module):
                                              reparam_proj=self.reparam_proj)
         if torch.is_grad_enabled():
             return make()
-        key = (self._tensor_key(random_matrices), self._tensor_key(sigma), self.tau, self.reparam_proj)
-        return self._cached("w", key, make)
+        return self._cached("w", (random_matrices, sigma), (self.tau, self.reparam_proj), make)
 
     def _stacked_qkv(self):
         """(weight [3E, E], bias [3E] or None) of one Linear layer that computes q_proj, k_proj and v_proj at once."""
         layers = (self.q_proj, self.k_proj, self.v_proj)
-        key = tuple(self._tensor_key(t) for layer in layers for t in (layer.weight, layer.bias))
 
         def make():
             weight = torch.cat([layer.weight.detach() for layer in layers], 0).contiguous()
             biases = [layer.bias for layer in layers]
             bias = None if any(b is None for b in biases) else torch.cat([b.detach() for b in biases], 0).contiguous()
             return weight, bias
-        return self._cached("qkv", key, make)
+        return self._cached("qkv", tuple(t for layer in layers for t in (layer.weight, layer.bias)), None, make)
 
     def _packed_decode_ok(self, x: Tensor) -> bool:
         layers = (self.q_proj, self.k_proj, self.v_proj)

@@ -46,14 +46,14 @@ int fail(int code, const char* fmt, ...) {
 namespace prof {
 enum Id { SEG_STATE, CAUSAL_FWD, CAUSAL_BWD_DQ, CAUSAL_BWD_DKDV, CROSS_READOUT, CROSS_READOUT_BWD,
           CROSS_STATE_BWD, DECODE_STEP, FEATURE_FWD, FEATURE_BWD, FEATURE_DW_REDUCE, MASKED_FWD, MASKED_PREP, MASKED_DQ, MASKED_DKDV, PROJECT_PHI, WGRAD_PARTIAL, WGRAD_REDUCE, TOTALS_SCAN, ZERO_FILL,
-          SELFTEST, BUILD_W, DECODE_TOUCH, CAUSAL_BWD_SLICED, COUNT };
+          SELFTEST, BUILD_W, DECODE_TOUCH, CAUSAL_BWD_SLICED, COPY_ROWS, COUNT };
 const char* const kNames[COUNT] = {"k_segment_state", "k_causal_fwd", "k_causal_bwd_dq", "k_causal_bwd_dkdv",
                                    "k_cross_readout", "k_cross_readout_bwd", "k_cross_state_bwd", "k_decode_step",
                                    "k_feature_map_fwd", "k_feature_map_bwd", "k_feature_map_dw_reduce",
                                    "k_masked_fwd", "k_masked_bwd_prep", "k_masked_dq", "k_masked_dkdv", "k_project_phi",
                                    "k_weight_grad_partial", "k_weight_grad_reduce", "k_totals_scan",
                                    "k_zero_f32", "k_selftest", "k_build_random_matrices", "k_touch_rows",
-                                   "k_sliced_bwd"};
+                                   "k_sliced_bwd", "k_copy_rows_strided"};
 struct Rec { int id; hipEvent_t a, b; };
 std::mutex mu;
 bool enabled = false;
@@ -823,26 +823,39 @@ int launch_feature_fwd(const rfa::half_t* x, const rfa::half_t* w, rfa::half_t* 
     return RFA_OK;
 }
 
+// dx_rs: halves between consecutive rows of dx / dx1 (H * DH for tensors of their own).  copy_src
+// [R, H * DH] (or NULL) is copied to rows of copy_dst of the same pitch: the third block of a
+// packed gradient, by a third set of workgroups of the same launch where the kernel has that job.
 template <int D, int DH>
 int launch_feature_bwd(const rfa::half_t* x, const rfa::half_t* w, const rfa::half_t* gphi, rfa::half_t* dx,
                        const rfa::half_t* x1, const rfa::half_t* gphi1, rfa::half_t* dx1,
-                       float* dw, float* part, int R, int H, float scale, hipStream_t st) {
+                       float* dw, float* part, int R, int H, float scale, hipStream_t st,
+                       int64_t dx_rs = 0, const rfa::half_t* copy_src = nullptr, rfa::half_t* copy_dst = nullptr) {
     const int ntens = x1 ? 2 : 1;       // two tensors through the same w: one launch, one reduction
+    if (dx_rs == 0) dx_rs = (int64_t)H * DH;
     int nblk;
     if constexpr (rfa::FeatureStreamCfg<D, DH>::kFits) {
         using Cfg = rfa::FeatureStreamCfg<D, DH>;
         nblk = feature_stream_blocks(R, H, ntens, rfa::kFeatureBwdWaves);      // never more than feature_bwd_blocks, which sized the workspace
         auto kern = rfa::k_feature_map_bwd_stream<D, DH>;
         if (int rc = set_lds(kern, Cfg::kLds)) return rc;
-        RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H, ntens), dim3(rfa::kFeatureBwdThreads), Cfg::kLds, st, x, w, gphi, dx, x1,
-                   gphi1, dx1, part, R, H, scale);
+        const bool copy_job = copy_src && ntens == 2;
+        RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H, ntens + (copy_job ? 1 : 0)), dim3(rfa::kFeatureBwdThreads), Cfg::kLds, st,
+                   x, w, gphi, dx, x1, gphi1, dx1, part, R, H, scale, dx_rs, copy_src, copy_dst);
+        if (copy_job) copy_src = nullptr;
     } else {
         using Cfg = rfa::FeatureCfg<D, DH>;
         nblk = feature_bwd_blocks(R, H, ntens);
         auto kern = rfa::k_feature_map_bwd<D, DH>;
         if (int rc = set_lds(kern, Cfg::kBwdLds)) return rc;
         RFA_LAUNCH(FEATURE_BWD, kern, dim3(nblk, H, ntens), dim3(rfa::kThreads), Cfg::kBwdLds, st, x, w, gphi, dx, x1, gphi1,
-                   dx1, part, R, H, scale);
+                   dx1, part, R, H, scale, dx_rs);
+    }
+    if (copy_src) {
+        const int64_t pieces = (int64_t)R * H * DH / 8;
+        const unsigned blocks = (unsigned)std::min<int64_t>((pieces + rfa::kThreads - 1) / rfa::kThreads, 4 * (int64_t)device_cus());
+        RFA_LAUNCH(COPY_ROWS, rfa::k_copy_rows_strided, dim3(blocks), dim3(rfa::kThreads), 0, st, copy_src, copy_dst, (int64_t)R,
+                   H * DH, dx_rs);
     }
     const int64_t elems = (int64_t)H * D * DH;
     static_assert((D * DH) % 256 == 0, "dw reduce works on blocks of 256 elements");
@@ -1715,6 +1728,42 @@ int rfa_feature_map_backward_pair(const void* x0, const void* x1, const void* w,
                                static_cast<const rfa::half_t*>(grad_phi0), static_cast<rfa::half_t*>(dx0),        \
                                static_cast<const rfa::half_t*>(x1), static_cast<const rfa::half_t*>(grad_phi1),   \
                                static_cast<rfa::half_t*>(dx1), dw, part, (int)R, H, scale, st)
+    RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
+#undef RFA_CALL
+    return fail(RFA_ERR_UNSUPPORTED, "unreachable");
+}
+
+int rfa_feature_map_backward_pair_packed(const void* x0, const void* x1, const void* w, const void* grad_phi0,
+                                         const void* grad_phi1, const void* third, void* packed, float* dw, int64_t R,
+                                         int H, int D, int d, float scale, void* workspace, size_t workspace_bytes,
+                                         void* stream) {
+    if (int rc = check_feature_dims("rfa_feature_map_backward_pair_packed", R, H, D, d)) return rc;
+    if (!dw) return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward_pair_packed: NULL dw");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (R == 0) {
+        zero_f32(dw, (int64_t)H * D * d, st);
+        return RFA_OK;
+    }
+    if (!x0 || !x1 || !w || !grad_phi0 || !grad_phi1 || !packed)
+        return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward_pair_packed: NULL tensor pointer");
+    if (!aligned16(x0) || !aligned16(x1) || !aligned16(w) || !aligned16(grad_phi0) || !aligned16(grad_phi1) ||
+        !aligned16(third) || !aligned16(packed) || !aligned16(dw))
+        return fail(RFA_ERR_ALIGNMENT, "rfa_feature_map_backward_pair_packed: tensors must be 16-byte aligned");
+    if ((int64_t)R * 3 * H * d >= ((int64_t)1 << 40))
+        return fail(RFA_ERR_BAD_SHAPE, "rfa_feature_map_backward_pair_packed: sizes exceed the supported range");
+    const size_t need = rfa_feature_map_backward_pair_workspace_bytes(R, H, D, d);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+        return fail(RFA_ERR_WORKSPACE, "rfa_feature_map_backward_pair_packed: workspace of %zu bytes required, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    float* part = static_cast<float*>(workspace);
+    const int64_t E = (int64_t)H * d;
+    auto* pk = static_cast<rfa::half_t*>(packed);
+#define RFA_CALL(DD, DH)                                                                                         \
+    launch_feature_bwd<DD, DH>(static_cast<const rfa::half_t*>(x0), static_cast<const rfa::half_t*>(w),           \
+                               static_cast<const rfa::half_t*>(grad_phi0), pk,                                    \
+                               static_cast<const rfa::half_t*>(x1), static_cast<const rfa::half_t*>(grad_phi1),   \
+                               pk + E, dw, part, (int)R, H, scale, st, 3 * E,                                     \
+                               static_cast<const rfa::half_t*>(third), pk + 2 * E)
     RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
 #undef RFA_CALL
     return fail(RFA_ERR_UNSUPPORTED, "unreachable");

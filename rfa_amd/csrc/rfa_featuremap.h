@@ -59,6 +59,20 @@ __device__ __forceinline__ void wave_rows_s2g(const half_t* Ss, int ld, half_t* 
     }
 }
 
+// Same, for a destination whose rows lie `rs` halves apart: dst points at this head's first column.
+template <int F>
+__device__ __forceinline__ void wave_rows_s2g_strided(const half_t* Ss, int ld, half_t* __restrict__ dst, int64_t rs,
+                                                      int r0, int R, int lane) {
+    constexpr int PPR = F / 8, RPI = 64 / PPR;
+    static_assert(PPR <= 64 && 64 % PPR == 0, "row too long for one wave");
+#pragma unroll
+    for (int k = 0; k < 16 / RPI; ++k) {
+        const int lr = k * RPI + lane / PPR, pc = lane % PPR;
+        const uint4 val = *reinterpret_cast<const uint4*>(Ss + lr * ld + pc * 8);
+        if (r0 + lr < R) *reinterpret_cast<uint4*>(dst + (int64_t)(r0 + lr) * rs + pc * 8) = val;
+    }
+}
+
 // The reverse, split so that the loads can be issued one row block ahead: global rows
 // -> registers (zero beyond R) -> this wave's staging rows.
 template <int F>
@@ -215,11 +229,12 @@ __global__ __launch_bounds__(kFeatureThreads) void k_feature_map_fwd(
 // gridDim.z = 2 differentiates two tensors that went through the same W' in one launch (phi(q) and
 // phi(k) of a module): workgroups with blockIdx.z = 1 take x1 / gphi1 / dx1 and the partial
 // sums nblk .. 2 nblk - 1, so that the reduction over 2 nblk shares yields the sum of both dW'.
+// The rows of dx lie dx_rs halves apart (H * DH for a tensor of its own).
 template <int D, int DH>
 __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
     const half_t* __restrict__ x0, const half_t* __restrict__ w, const half_t* __restrict__ gphi0,
     half_t* __restrict__ dx0, const half_t* __restrict__ x1, const half_t* __restrict__ gphi1,
-    half_t* __restrict__ dx1, float* __restrict__ dw_part, int R, int H, float scale) {
+    half_t* __restrict__ dx1, float* __restrict__ dw_part, int R, int H, float scale, int64_t dx_rs) {
     const bool second = blockIdx.z != 0;
     const half_t* __restrict__ x = second ? x1 : x0;
     const half_t* __restrict__ gphi = second ? gphi1 : gphi0;
@@ -327,7 +342,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
             *reinterpret_cast<h4*>(Gs + i * LDG + 16 * ct + 4 * G) = o;
         }
         wave_lds_order();
-        wave_rows_s2g<DH>(Gs, LDG, dx, r0, R, H, h, lane);
+        wave_rows_s2g_strided<DH>(Gs, LDG, dx + h * DH, dx_rs, r0, R, lane);
 
         // dW (m = c, n = j) += X^T Us over the 64 rows of the block
 #pragma unroll
@@ -395,7 +410,25 @@ template <int D, int DH>
 __global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
     const half_t* __restrict__ x0, const half_t* __restrict__ w, const half_t* __restrict__ gphi0,
     half_t* __restrict__ dx0, const half_t* __restrict__ x1, const half_t* __restrict__ gphi1,
-    half_t* __restrict__ dx1, float* __restrict__ dw_part, int R, int H, float scale) {
+    half_t* __restrict__ dx1, float* __restrict__ dw_part, int R, int H, float scale, int64_t dx_rs,
+    const half_t* __restrict__ copy_src, half_t* __restrict__ copy_dst) {
+    if (blockIdx.z == 2) {
+        // third job of a launch that fills a packed gradient: rows of copy_src [R, H, DH] -> rows of
+        // copy_dst, dx_rs halves apart (this workgroup: head blockIdx.y, its waves' row groups)
+        constexpr int PPR = DH / 8, RPI = 64 / PPR;
+        const int lane = threadIdx.x & 63, h = blockIdx.y;
+        const int ngrp = (R + 15) / 16;
+        for (int g = blockIdx.x * kFeatureBwdWaves + (threadIdx.x >> 6); g < ngrp; g += gridDim.x * kFeatureBwdWaves) {
+#pragma unroll
+            for (int k = 0; k < 16 / RPI; ++k) {
+                const int r = g * 16 + k * RPI + lane / PPR, pc = lane % PPR;
+                if (r < R)
+                    *reinterpret_cast<uint4*>(copy_dst + (int64_t)r * dx_rs + h * DH + pc * 8) =
+                        *reinterpret_cast<const uint4*>(copy_src + ((int64_t)r * H + h) * DH + pc * 8);
+            }
+        }
+        return;
+    }
     const bool second = blockIdx.z != 0;
     const half_t* __restrict__ x = second ? x1 : x0;
     const half_t* __restrict__ gphi = second ? gphi1 : gphi0;
@@ -496,7 +529,7 @@ __global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
             for (int e = 0; e < 4; ++e) xdot += acc[e] * (float)t.x[ct / 2][4 * (ct % 2) + e];
         }
         xdot = sum_over_groups(xdot) * coef;
-        half_t* po = dx + ((int64_t)r * H + h) * DH + 8 * G;
+        half_t* po = dx + (int64_t)r * dx_rs + h * DH + 8 * G;
 #pragma unroll
         for (int u = 0; u < DH / 32; ++u) {
             h8 o;
@@ -548,6 +581,19 @@ __global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
         for (int o = 1; o < kFeatureBwdWaves; ++o) sum += red[(o * Cfg::kTiles + t) * 64 + lane];
         const int a = t / (D / 16), b = t % (D / 16);
         *reinterpret_cast<f4*>(out + (16 * b + i) * DH + 16 * a + 4 * G) = sum;
+    }
+}
+
+// Rows of src [R, W] (W halves, multiple of 8) -> rows of dst that lie rs halves apart; 16 bytes per
+// thread.  The copy job of a packed gradient for the shapes whose backward has none of its own.
+__global__ __launch_bounds__(kThreads) void k_copy_rows_strided(const half_t* __restrict__ src, half_t* __restrict__ dst,
+                                                                int64_t R, int W, int64_t rs) {
+    const int ppr = W / 8;
+    const int64_t total = R * ppr;
+    for (int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x; p < total; p += (int64_t)gridDim.x * kThreads) {
+        const int64_t r = p / ppr;
+        const int pc = (int)(p % ppr);
+        *reinterpret_cast<uint4*>(dst + r * rs + pc * 8) = *reinterpret_cast<const uint4*>(src + r * W + pc * 8);
     }
 }
 

@@ -250,6 +250,34 @@ std::tuple<Tensor, Tensor, Tensor> feature_map_backward_pair(const Tensor& x0, c
     return {dx0, dx1, dw};
 }
 
+std::tuple<Tensor, Tensor> feature_map_backward_pair_packed(const Tensor& x0, const Tensor& x1, const Tensor& w,
+                                                            const Tensor& g0, const Tensor& g1,
+                                                            const c10::optional<Tensor>& third, double scale) {
+    check_feature_args(x0, w);
+    check_feature_args(x1, w);
+    TORCH_CHECK_VALUE(x0.sizes() == x1.sizes(), "the two tensors must have one shape");
+    const int64_t L = x0.size(0), B = x0.size(1);
+    const int H = (int)x0.size(2), d = (int)x0.size(3), D = (int)w.size(1);
+    for (const Tensor* g : {&g0, &g1}) {
+        check_half("grad_phi", *g, 4);
+        TORCH_CHECK_VALUE(g->size(0) == L && g->size(1) == B && g->size(2) == H && g->size(3) == 2 * D, "grad_phi ",
+                          g->sizes(), " must be [", L, ", ", B, ", ", H, ", ", 2 * D, "]");
+    }
+    if (third) {
+        check_half("third", *third, third->dim());
+        TORCH_CHECK_VALUE(third->numel() == x0.numel(), "third ", third->sizes(), " must hold ", L * B, " rows of ", H * d);
+    }
+    Tensor packed = torch::empty({L * B, 3 * (int64_t)H * d}, x0.options());
+    Tensor dw = torch::empty({H, D, d}, x0.options().dtype(torch::kFloat32));
+    Launch l(x0);
+    const size_t nbytes = rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d);
+    Tensor ws = workspace(nbytes, x0);
+    check_rc(rfa_feature_map_backward_pair_packed(ptr(x0), ptr(x1), ptr(w), ptr(g0), ptr(g1), third ? ptr(*third) : nullptr,
+                                                  ptr(packed), dw.data_ptr<float>(), L * B, H, D, d, (float)scale, ptr(ws),
+                                                  nbytes, l.stream));
+    return {packed, dw};
+}
+
 // ---- projections ----------------------------------------------------------------------
 // keep_y = false: a projection whose phi is asked for returns None in place of y (nothing will
 // differentiate through it)
@@ -557,6 +585,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("feature_map_backward", &feature_map_backward, py::arg("x"), py::arg("w"), py::arg("grad_phi"), py::arg("scale"));
     m.def("feature_map_backward_pair", &feature_map_backward_pair, py::arg("x0"), py::arg("x1"), py::arg("w"),
           py::arg("grad_phi0"), py::arg("grad_phi1"), py::arg("scale"));
+    m.def("feature_map_backward_pair_packed", &feature_map_backward_pair_packed, py::arg("x0"), py::arg("x1"), py::arg("w"),
+          py::arg("grad_phi0"), py::arg("grad_phi1"), py::arg("third"), py::arg("scale"));
     m.def("project_feature_map", &project_feature_map, py::arg("x"), py::arg("weights"), py::arg("biases"),
           py::arg("want_phi"), py::arg("w"), py::arg("heads"), py::arg("scale"), py::arg("keep_y") = true);
     m.def("linear_weight_grad", &linear_weight_grad, py::arg("x"), py::arg("dys"), py::arg("want_bias"));

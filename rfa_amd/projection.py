@@ -14,6 +14,7 @@ import torch
 from torch import Tensor, nn
 
 from . import rfa_hip
+from ._derived import derived
 
 
 def linear_param_grads(x2: Tensor, dys: Sequence[Tensor], has_bias: Sequence[bool]):
@@ -24,6 +25,28 @@ def linear_param_grads(x2: Tensor, dys: Sequence[Tensor], has_bias: Sequence[boo
             and rfa_hip.linear_weight_grad_supported(e_out, e_in) and 1 <= len(dys) <= 3):
         return rfa_hip.linear_weight_grad(x2.contiguous(), [d.contiguous() for d in dys], list(has_bias))
     return ([torch.mm(d.t(), x2) for d in dys], [d.sum(0) if b else None for d, b in zip(dys, has_bias)])
+
+
+_STACKED: dict = {}      # ids of the three weights -> their [3 * E_out, E_in] stack
+
+
+def _stacked_weights(weights: Sequence[Tensor]) -> Tensor:
+    """[Wq; Wk; Wv] as one matrix.  Outside stream capture the stack is kept for as long as the
+    three weights are the same tensor objects in the same state (an optimizer step moves their
+    version counters); under capture it is always formed, so that a replayed graph reads the
+    weights of the day."""
+    make = lambda: torch.cat(list(weights), 0)
+    if torch.cuda.is_current_stream_capturing():
+        return make()
+    return derived(_STACKED, tuple(id(w) for w in weights), tuple(weights), None, make, limit=8)
+
+
+def _packed_backward_ok(ctx, grads, weights) -> bool:
+    """q and k through the feature map, v plain, an input gradient wanted, equal fp16 weights: the
+    three dx products can be one over the packed gradient."""
+    return (len(ctx.want_phi) == 3 and tuple(ctx.want_phi) == (True, True, False) and ctx.needs_input_grad[0]
+            and all(g is not None and g.is_cuda and g.dtype == torch.float16 for g in grads)
+            and all(w.dtype == torch.float16 and w.shape == weights[0].shape for w in weights))
 
 
 class _ProjectHeads(torch.autograd.Function):
@@ -59,6 +82,19 @@ class _ProjectHeads(torch.autograd.Function):
         dwf = None
         dys = []
         yi = 0
+        if _packed_backward_ok(ctx, grads, weights):
+            # [dy_q | dy_k | dv] side by side, written by the feature-map backward launch itself: one
+            # GEMM for dx and one contraction for the three weight gradients
+            e_out = weights[0].shape[0]
+            packed, dwf = rfa_hip.feature_map_backward_pair_packed(ys[0], ys[1], wf, grads[0].contiguous(),
+                                                                   grads[1].contiguous(), grads[2].contiguous(), ctx.scale)
+            dx = torch.mm(packed, _stacked_weights(weights)).view(L, B, E)
+            dws, dbs = linear_param_grads(x2, [packed], [any(ctx.has_bias)])
+            dparams = []
+            for p in range(n):
+                dparams += [dws[0][p * e_out:(p + 1) * e_out],
+                            dbs[0][p * e_out:(p + 1) * e_out] if ctx.has_bias[p] else None]
+            return (dx, dwf.to(wf.dtype), None, None, None, None, *dparams)
         phi_idx = [p for p in range(n) if ctx.want_phi[p]]
         pair = {}
         if len(phi_idx) == 2:       # phi(q) and phi(k): both through the same w, one launch for the two

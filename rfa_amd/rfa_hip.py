@@ -408,6 +408,35 @@ def feature_map_backward_pair(x0: Tensor, x1: Tensor, w: Tensor, grad_phi0: Tens
     return dx0, dx1, dw
 
 
+def feature_map_backward_pair_packed(x0: Tensor, x1: Tensor, w: Tensor, grad_phi0: Tensor, grad_phi1: Tensor,
+                                     third: Optional[Tensor], scale: float):
+    """feature_map_backward_pair that leaves [dx0 | dx1 | third] side by side in one fp16 [L*B, 3*H*d]
+    matrix (third: [L, B, H, d] or [L*B, H*d], copied by the same launch; None leaves that block
+    unset) and returns (packed, dw): the operand of one GEMM for the three input projections."""
+    _check_feature_args(x0, w)
+    _check_feature_args(x1, w)
+    _require(x0.shape == x1.shape, ValueError, lambda: "the two tensors must have one shape")
+    L, B, H, d = x0.shape
+    D = w.shape[1]
+    for name, g in (("grad_phi0", grad_phi0), ("grad_phi1", grad_phi1)):
+        _check_half_cuda(name, g, 4)
+        _require(tuple(g.shape) == (L, B, H, 2 * D), ValueError, lambda: f"{name} {tuple(g.shape)} must be {(L, B, H, 2 * D)}")
+    if third is not None:
+        _check_half_cuda("third", third, third.dim())
+        _require(third.numel() == x0.numel(), ValueError, lambda: f"third {tuple(third.shape)} must hold {L * B} rows of {H * d}")
+    lib = _lib.load()
+    packed = torch.empty((L * B, 3 * H * d), dtype=torch.float16, device=x0.device)
+    dw = torch.empty((H, D, d), dtype=torch.float32, device=x0.device)
+    with _on_device(x0.device):
+        nbytes = lib.rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d)
+        ws = _workspace(nbytes, x0.device)
+        _lib.check(lib.rfa_feature_map_backward_pair_packed(
+            x0.data_ptr(), x1.data_ptr(), w.data_ptr(), grad_phi0.data_ptr(), grad_phi1.data_ptr(),
+            None if third is None else third.data_ptr(), packed.data_ptr(), dw.data_ptr(), L * B, H, D, d, float(scale),
+            ws.data_ptr(), nbytes, _stream_ptr(x0.device)))
+    return packed, dw
+
+
 # ---------------------------------------------------------------------------
 # cross attention
 # ---------------------------------------------------------------------------
@@ -654,7 +683,7 @@ def masked_backward(phi_q: Tensor, phi_k: Tensor, v: Tensor, grad_attn: Tensor, 
 _BOUND = ("supported", "feature_map_supported", "selftest_layout", "forward", "backward", "prefill", "forward_save",
           "backward_saved", "build_random_matrices", "build_random_matrices_backward", "feature_map_forward",
           "feature_map_forward_pair",
-          "feature_map_backward", "feature_map_backward_pair", "project_feature_map", "linear_weight_grad", "cross_state",
+          "feature_map_backward", "feature_map_backward_pair", "feature_map_backward_pair_packed", "project_feature_map", "linear_weight_grad", "cross_state",
           "cross_state_backward", "cross_readout", "cross_readout_backward", "incremental", "incremental_fused",
           "incremental_qkv",
           "masked_forward", "masked_backward")

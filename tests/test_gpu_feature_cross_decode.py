@@ -105,6 +105,41 @@ def test_feature_map_backward_pair(L, B, H, d, D):
     assert _rel(dw.cpu(), rw0 + rw1) <= GRAD_RTOL
 
 
+@pytest.mark.parametrize("L,B,H,d,D", FEATURE_SHAPES + [(300, 3, 4, 64, 64)])
+@pytest.mark.parametrize("with_third", [True, False])
+def test_feature_map_backward_pair_packed(L, B, H, d, D, with_third):
+    """[dx0 | dx1 | third] side by side in one [R, 3 H d] matrix: every block carries the bits of
+    the separate tensors, dW' those of the pair call, and without a third tensor its block is left
+    as it was."""
+    from rfa_amd import _lib, rfa_hip
+    x0 = (_randn(L, B, H, d, seed=50 + L) * 1.3).half().cuda()
+    x1 = (_randn(L, B, H, d, seed=51 + L) * 0.7).half().cuda()
+    w = (_randn(H, D, d, seed=52) * 0.9).half().cuda()
+    g0 = _randn(L, B, H, 2 * D, seed=53).half().cuda()
+    g1 = _randn(L, B, H, 2 * D, seed=54).half().cuda()
+    third = _randn(L, B, H, d, seed=55).half().cuda() if with_third else None
+    want0, want1, want_dw = rfa_hip.feature_map_backward_pair(x0, x1, w, g0, g1, O.SCALE)
+    print(f"phi bwd packed L={L} B={B} H={H} d={d} D={D} third={with_third}", flush=True)
+    E = H * d
+    if with_third:
+        packed, dw = rfa_hip.feature_map_backward_pair_packed(x0, x1, w, g0, g1, third, O.SCALE)
+        assert torch.equal(packed[:, 2 * E:], third.view(L * B, E))
+    else:       # through the C ABI into a buffer of known contents
+        lib = _lib.load()
+        packed = torch.full((L * B, 3 * E), 7.0, dtype=torch.float16, device="cuda")
+        dw = torch.empty(H, D, d, dtype=torch.float32, device="cuda")
+        nbytes = lib.rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d)
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+        _lib.check(lib.rfa_feature_map_backward_pair_packed(
+            x0.data_ptr(), x1.data_ptr(), w.data_ptr(), g0.data_ptr(), g1.data_ptr(), None, packed.data_ptr(),
+            dw.data_ptr(), L * B, H, D, d, O.SCALE, ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert bool((packed[:, 2 * E:] == 7.0).all())
+    assert packed.shape == (L * B, 3 * E)
+    assert torch.equal(packed[:, :E], want0.view(L * B, E)) and torch.equal(packed[:, E:2 * E], want1.view(L * B, E))
+    assert torch.equal(dw, want_dw)
+
+
 @pytest.mark.parametrize("L,B,H,d,D,wgs", [(333, 2, 2, 64, 64, 4), (333, 2, 2, 64, 64, 2), (100, 3, 1, 128, 32, 1),
                                            (257, 1, 2, 64, 32, 6)])
 def test_feature_map_waves_that_walk_many_row_groups(L, B, H, d, D, wgs, knobs):

@@ -325,6 +325,102 @@ def test_module_step_replays_from_a_hip_graph():
         captured = grads_before
 
 
+def test_projection_backward_on_the_packed_gradient(monkeypatch):
+    """q, k through the feature map and v plain: the backward that forms [dy_q | dy_k | dv] in one
+    matrix (one GEMM for dx, one contraction for the three dW) against the one with a GEMM per
+    projection.  dW, db and dW' carry the same bits (the same row-split sums); dx is one sum of 3E
+    products in place of three rounded partial sums."""
+    from rfa_amd import projection
+    torch.manual_seed(11)
+    L, B, E, H, d, D = 130, 3, 256, 4, 64, 64
+    layers = [torch.nn.Linear(E, H * d).cuda().half() for _ in range(3)]
+    layers[1].bias = None
+    wf = (torch.randn(H, D, d) * 0.9).half().cuda().requires_grad_(True)
+    x = (torch.randn(L, B, E) * 0.7).half().cuda().requires_grad_(True)
+    gs = [torch.randn(L, B, H, 2 * D).half().cuda(), torch.randn(L, B, H, 2 * D).half().cuda(),
+          torch.randn(L, B, H, d).half().cuda()]
+
+    def run():
+        for t in [x, wf] + [p for l in layers for p in l.parameters()]:
+            t.grad = None
+        outs = projection.project_heads(x, layers, [True, True, False], H, wf, O.SCALE)
+        torch.autograd.backward(outs, gs)
+        return [x.grad.clone(), wf.grad.clone()] + [p.grad.clone() for l in layers for p in l.parameters()]
+
+    used = []
+    real = projection.rfa_hip.feature_map_backward_pair_packed
+    monkeypatch.setattr(projection.rfa_hip, "feature_map_backward_pair_packed", lambda *a: (used.append(1), real(*a))[1])
+    print("projection backward, packed gradient", flush=True)
+    packed = run()
+    assert used, "the packed path was not taken"
+    key = tuple(id(l.weight) for l in layers)           # the stack of the weights is kept between eager steps ...
+    stack = projection._STACKED[key].value
+    again = run()
+    assert projection._STACKED[key].value is stack and all(torch.equal(a, b) for a, b in zip(packed, again))
+    with torch.no_grad():
+        layers[2].weight.mul_(1.5)                      # ... until a weight changes
+    changed = run()
+    assert projection._STACKED[key].value is not stack and not torch.equal(changed[0], packed[0])
+    with torch.no_grad():
+        layers[2].weight.div_(1.5)                      # exact in fp16
+    used.clear()
+    packed = run()
+    monkeypatch.setattr(projection, "_packed_backward_ok", lambda *a: False)
+    plain = run()
+    assert len(used) == 1 and len(packed) == len(plain) == 2 + 5
+    scale = plain[0].float().abs().max().item()
+    assert (packed[0].float() - plain[0].float()).abs().max().item() <= 4e-3 * scale
+    for a, b in zip(packed[1:], plain[1:]):
+        assert torch.equal(a, b)
+
+
+def test_packed_backward_in_a_graph_follows_weight_updates():
+    """The stacked weights [Wq; Wk; Wv] of the packed backward are kept between eager steps but
+    formed inside a captured graph: a replay after an in-place weight update gives the eager
+    gradients of the updated weights."""
+    from rfa_amd import CausalAttention
+    torch.manual_seed(13)
+    T, B, E, H, d, D = 192, 2, 256, 4, 64, 64
+    m = CausalAttention(embed_dim=E, num_heads=H, head_dim=d, proj_dim=D).cuda().half()
+    W = O.make_w(d, D, H).cuda().half()
+    x = (torch.randn(T, B, E) * 0.6).half().cuda().requires_grad_(True)
+    go = torch.randn(T, B, E).half().cuda()
+
+    def step():
+        m.zero_grad(set_to_none=True)
+        x.grad = None
+        m(x, W).backward(go)
+        return x.grad.detach().clone()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()                      # also fills the eager cache of the stacked weights
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    m.zero_grad(set_to_none=True)
+    x.grad = None
+    print("packed backward: capture", flush=True)
+    with torch.cuda.graph(graph):
+        m(x, W).backward(go)
+    gx = x.grad
+    for rep in range(3):
+        with torch.no_grad():
+            for p in (m.q_proj.weight, m.k_proj.weight, m.v_proj.weight):
+                p.mul_(1.0 + 0.25 * (rep + 1))
+        gx.zero_()
+        torch.cuda.synchronize()
+        print(f"packed backward: replay {rep}", flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = gx.clone()
+        want = step()                   # eager, on the updated weights (rebinds x.grad; the graph keeps gx)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), rep
+
+
 def test_empty_input():
     """No rows: the projections come back empty, the weight and bias gradients as zeros."""
     from rfa_amd import rfa_hip

@@ -250,3 +250,51 @@ def test_binding_built_after_the_package_was_imported_is_found(tmp_path):
         "print('found')\n")
     proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=str(tmp_path))
     assert proc.returncode == 0 and "found" in proc.stdout, proc.stdout + proc.stderr
+
+
+def test_derived_values_answer_only_for_the_same_live_tensors_in_the_same_state():
+    """The keep-until-changed store behind the stacked projection weights and the scaled random
+    matrices: a hit needs the same tensor objects with unchanged version, address, dtype and shape;
+    a tensor that died cannot be stood in for by another one, whatever address or id it got."""
+    import gc
+    from rfa_amd._derived import derived
+    slot, made = {}, []
+
+    def make_from(*ts):
+        def make():
+            made.append(1)
+            return sum(float(t.sum()) for t in ts if t is not None)
+        return make
+
+    a, b = torch.ones(4), torch.full((4,), 2.0)
+    assert derived(slot, "k", (a, b, None), 1, make_from(a, b)) == 12.0 and len(made) == 1
+    assert derived(slot, "k", (a, b, None), 1, make_from(a, b)) == 12.0 and len(made) == 1      # hit
+    assert derived(slot, "k", (a, b, None), 2, make_from(a, b)) == 12.0 and len(made) == 2      # other extra
+    a.add_(1.0)                                                                                   # version moves
+    assert derived(slot, "k", (a, b, None), 2, make_from(a, b)) == 16.0 and len(made) == 3
+    a.data = torch.zeros(4)                                                                       # address moves, version does not
+    assert derived(slot, "k", (a, b, None), 2, make_from(a, b)) == 8.0 and len(made) == 4
+    c = b.clone()                                                                                 # equal state, another object
+    assert derived(slot, "k", (a, c, None), 2, make_from(a, c)) == 8.0 and len(made) == 5
+    assert derived(slot, "k", (a, None, None), 2, make_from(a)) == 0.0 and len(made) == 6       # None where a tensor was
+    # a dead source: the entry must not answer for a newcomer in the same state, even at the same address
+    t = torch.full((1024,), 3.0)
+    derived(slot, "dead", (t,), None, make_from(t))
+    n_made, ptr = len(made), t.data_ptr()
+    del t
+    gc.collect()
+    for _ in range(8):
+        u = torch.full((1024,), 5.0)
+        if u.data_ptr() == ptr:
+            break
+    assert derived(slot, "dead", (u,), None, make_from(u)) == 5.0 * 1024 and len(made) == n_made + 1
+    # bounded slots drop entries of dead sources first
+    small = {}
+    keep = [torch.ones(2) for _ in range(3)]
+    for i, t in enumerate(keep):
+        derived(small, i, (t,), None, make_from(t), limit=3)
+    del keep[0]
+    gc.collect()
+    extra = torch.ones(2)
+    derived(small, "new", (extra,), None, make_from(extra), limit=3)
+    assert set(small) == {1, 2, "new"}
