@@ -201,6 +201,12 @@ class CausalAttention(nn.Module):
     def _cached(self, name: str, sources, extra, make):
         return derived(self.__dict__.setdefault("_inference_cache", {}), name, sources, extra, make)
 
+    def __getstate__(self):
+        # copies and pickles of the module start without the cache (it holds weak references)
+        state = self.__dict__.copy()
+        state.pop("_inference_cache", None)
+        return state
+
     def _scaled_matrices(self, random_matrices: Tensor) -> Tensor:
         sigma = self.sigma if self.reparam_proj else None
         make = lambda: build_random_matrices(random_matrices=random_matrices, tau=self.tau, sigma=sigma,

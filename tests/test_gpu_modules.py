@@ -190,6 +190,16 @@ def test_causal_module_decode_from_one_stacked_projection():
             m.sigma.mul_(0.8)
             other2 = m(x[3:4], (W * 0.5).contiguous(), saved_state=dict(state))
         assert not torch.equal(other, changed) and not torch.equal(other2, other)
+        # a module with a filled cache copies and pickles (the cache stays behind), and the copy decodes alike
+        import copy
+        import io
+        assert m.__dict__.get("_inference_cache")
+        twin = copy.deepcopy(m)
+        buf = io.BytesIO()
+        torch.save(m, buf)
+        assert "_inference_cache" not in twin.__dict__
+        with torch.no_grad():
+            assert torch.equal(twin(x[3:4], (W * 0.5).contiguous(), saved_state=dict(state)), other2)
     finally:
         rfa_hip.incremental_qkv = real
 
