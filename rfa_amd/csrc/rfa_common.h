@@ -130,6 +130,12 @@ __device__ __forceinline__ h8 col8(const half_t* X, int ld, int r0, int c0, int 
     return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// "Pair order" of the rows of an MFMA operand matrix: row pair_pos(f) holds index f, so that tile t
+// of 16 rows is made of the indices 32 (t / 2) + 8 G + 4 (t % 2) + e at accumulator position
+// m = 4 G + e, and the accumulators of tiles 2p and 2p + 1 together give lane (i, G) the 8
+// consecutive indices 32 p + 8 G .. + 7: 16 bytes per lane and row, ready for one store.
+__host__ __device__ constexpr int pair_pos(int f) { return (f & ~31) | ((f & 4) << 2) | ((f & 24) >> 1) | (f & 3); }
+
 // Two fp32 values -> packed fp16 hi and lo with hi + lo carrying ~22 bits of each.  The
 // residual x - float(hi) is exact in fp32 and is formed as fma(hi, -1, x): with the -1 and the
 // packed hi opaque to the optimiser the compiler selects the mixed-precision fma that reads the

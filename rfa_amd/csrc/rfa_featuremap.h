@@ -125,12 +125,11 @@ __device__ __forceinline__ void load_w_to_lds(half_t* Ws, const half_t* __restri
 //     32 (t / 2) + 8 G + 4 (t % 2) + e        at accumulator position m = 4 G + e,
 // so that the accumulators of tiles 2p and 2p+1 together give lane (i, G) the 8 consecutive
 // indices 32 p + 8 G .. + 7 of row i: 16 bytes that go to (and come from) global memory
-// directly, without a pass through LDS to re-form rows.  pair_pos(f) is the row of the operand
-// matrix that holds index f.
+// directly, without a pass through LDS to re-form rows.  pair_pos(f) (rfa_common.h) is the row of
+// the operand matrix that holds index f.
 constexpr int kFeatureWaves = 8;
 constexpr int kFeatureThreads = 64 * kFeatureWaves;
 
-__host__ __device__ constexpr int pair_pos(int f) { return (f & ~31) | ((f & 4) << 2) | ((f & 24) >> 1) | (f & 3); }
 
 // W' of one head -> LDS with its rows (features) in pair order
 template <int D, int DH, int NT = kFeatureThreads>
