@@ -204,6 +204,9 @@ int rfa_feature_map_forward(const void* x, const void* w, void* phi, int64_t R, 
  * rfa_feature_map_forward calls. */
 int rfa_feature_map_forward_pair(const void* x0, const void* x1, const void* w, void* phi0, void* phi1,
                                  int64_t R, int H, int D, int d, float scale, void* stream);
+/* In the three backward entry points dw may be NULL: w then counts as a constant (random matrices
+ * that are not reparametrised, utils.py:90-97 with reparam_proj off), only dx is formed, no
+ * workspace is needed and the reduction launch is not made. */
 size_t rfa_feature_map_backward_workspace_bytes(int64_t R, int H, int D, int d);
 int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi, void* dx, float* dw,
                              int64_t R, int H, int D, int d, float scale, void* workspace,

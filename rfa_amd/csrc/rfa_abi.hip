@@ -857,6 +857,10 @@ int launch_feature_bwd(const rfa::half_t* x, const rfa::half_t* w, const rfa::ha
         RFA_LAUNCH(COPY_ROWS, rfa::k_copy_rows_strided, dim3(blocks), dim3(rfa::kThreads), 0, st, copy_src, copy_dst, (int64_t)R,
                    H * DH, dx_rs);
     }
+    if (!dw) {                  // dx only: the kernels got no place for partial sums and formed none
+        RFA_HIP_TRY(hipGetLastError());
+        return RFA_OK;
+    }
     const int64_t elems = (int64_t)H * D * DH;
     static_assert((D * DH) % 256 == 0, "dw reduce works on blocks of 256 elements");
     RFA_LAUNCH(FEATURE_DW_REDUCE, rfa::k_feature_map_dw_reduce, dim3((unsigned)(elems / 256)), dim3(rfa::kThreads), 0, st,
@@ -1675,24 +1679,23 @@ int rfa_feature_map_backward(const void* x, const void* w, const void* grad_phi,
                              int H, int D, int d, float scale, void* workspace, size_t workspace_bytes,
                              void* stream) {
     if (int rc = check_feature_dims("rfa_feature_map_backward", R, H, D, d)) return rc;
-    if (!dw) return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward: NULL dw");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (R == 0) {
-        zero_f32(dw, (int64_t)H * D * d, st);
+        if (dw) zero_f32(dw, (int64_t)H * D * d, st);
         return RFA_OK;
     }
     if (!x || !w || !grad_phi || !dx) return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward: NULL tensor pointer");
     if (!aligned16(x) || !aligned16(w) || !aligned16(grad_phi) || !aligned16(dx) || !aligned16(dw))
         return fail(RFA_ERR_ALIGNMENT, "rfa_feature_map_backward: tensors must be 16-byte aligned");
-    const size_t need = rfa_feature_map_backward_workspace_bytes(R, H, D, d);
-    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+    const size_t need = dw ? rfa_feature_map_backward_workspace_bytes(R, H, D, d) : 0;
+    if (dw && (!workspace || workspace_bytes < need || !aligned16(workspace)))
         return fail(RFA_ERR_WORKSPACE, "rfa_feature_map_backward: workspace of %zu bytes required, got %zu", need,
                     workspace ? workspace_bytes : (size_t)0);
     auto* xh = static_cast<const rfa::half_t*>(x);
     auto* wh = static_cast<const rfa::half_t*>(w);
     auto* gh = static_cast<const rfa::half_t*>(grad_phi);
     auto* dxh = static_cast<rfa::half_t*>(dx);
-    float* part = static_cast<float*>(workspace);
+    float* part = dw ? static_cast<float*>(workspace) : nullptr;
 #define RFA_CALL(DD, DH) launch_feature_bwd<DD, DH>(xh, wh, gh, dxh, nullptr, nullptr, nullptr, dw, part, (int)R, H, scale, st)
     RFA_DISPATCH_FEATURE(D, d, RFA_CALL)
 #undef RFA_CALL
@@ -1707,10 +1710,9 @@ int rfa_feature_map_backward_pair(const void* x0, const void* x1, const void* w,
                                   const void* grad_phi1, void* dx0, void* dx1, float* dw, int64_t R, int H, int D,
                                   int d, float scale, void* workspace, size_t workspace_bytes, void* stream) {
     if (int rc = check_feature_dims("rfa_feature_map_backward_pair", R, H, D, d)) return rc;
-    if (!dw) return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward_pair: NULL dw");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (R == 0) {
-        zero_f32(dw, (int64_t)H * D * d, st);
+        if (dw) zero_f32(dw, (int64_t)H * D * d, st);
         return RFA_OK;
     }
     if (!x0 || !x1 || !w || !grad_phi0 || !grad_phi1 || !dx0 || !dx1)
@@ -1718,11 +1720,11 @@ int rfa_feature_map_backward_pair(const void* x0, const void* x1, const void* w,
     if (!aligned16(x0) || !aligned16(x1) || !aligned16(w) || !aligned16(grad_phi0) || !aligned16(grad_phi1) ||
         !aligned16(dx0) || !aligned16(dx1) || !aligned16(dw))
         return fail(RFA_ERR_ALIGNMENT, "rfa_feature_map_backward_pair: tensors must be 16-byte aligned");
-    const size_t need = rfa_feature_map_backward_pair_workspace_bytes(R, H, D, d);
-    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+    const size_t need = dw ? rfa_feature_map_backward_pair_workspace_bytes(R, H, D, d) : 0;
+    if (dw && (!workspace || workspace_bytes < need || !aligned16(workspace)))
         return fail(RFA_ERR_WORKSPACE, "rfa_feature_map_backward_pair: workspace of %zu bytes required, got %zu", need,
                     workspace ? workspace_bytes : (size_t)0);
-    float* part = static_cast<float*>(workspace);
+    float* part = dw ? static_cast<float*>(workspace) : nullptr;
 #define RFA_CALL(DD, DH)                                                                                         \
     launch_feature_bwd<DD, DH>(static_cast<const rfa::half_t*>(x0), static_cast<const rfa::half_t*>(w),           \
                                static_cast<const rfa::half_t*>(grad_phi0), static_cast<rfa::half_t*>(dx0),        \
@@ -1738,10 +1740,9 @@ int rfa_feature_map_backward_pair_packed(const void* x0, const void* x1, const v
                                          int H, int D, int d, float scale, void* workspace, size_t workspace_bytes,
                                          void* stream) {
     if (int rc = check_feature_dims("rfa_feature_map_backward_pair_packed", R, H, D, d)) return rc;
-    if (!dw) return fail(RFA_ERR_NULL_POINTER, "rfa_feature_map_backward_pair_packed: NULL dw");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (R == 0) {
-        zero_f32(dw, (int64_t)H * D * d, st);
+        if (dw) zero_f32(dw, (int64_t)H * D * d, st);
         return RFA_OK;
     }
     if (!x0 || !x1 || !w || !grad_phi0 || !grad_phi1 || !packed)
@@ -1751,11 +1752,11 @@ int rfa_feature_map_backward_pair_packed(const void* x0, const void* x1, const v
         return fail(RFA_ERR_ALIGNMENT, "rfa_feature_map_backward_pair_packed: tensors must be 16-byte aligned");
     if ((int64_t)R * 3 * H * d >= ((int64_t)1 << 40))
         return fail(RFA_ERR_BAD_SHAPE, "rfa_feature_map_backward_pair_packed: sizes exceed the supported range");
-    const size_t need = rfa_feature_map_backward_pair_workspace_bytes(R, H, D, d);
-    if (!workspace || workspace_bytes < need || !aligned16(workspace))
+    const size_t need = dw ? rfa_feature_map_backward_pair_workspace_bytes(R, H, D, d) : 0;
+    if (dw && (!workspace || workspace_bytes < need || !aligned16(workspace)))
         return fail(RFA_ERR_WORKSPACE, "rfa_feature_map_backward_pair_packed: workspace of %zu bytes required, got %zu", need,
                     workspace ? workspace_bytes : (size_t)0);
-    float* part = static_cast<float*>(workspace);
+    float* part = dw ? static_cast<float*>(workspace) : nullptr;
     const int64_t E = (int64_t)H * d;
     auto* pk = static_cast<rfa::half_t*>(packed);
 #define RFA_CALL(DD, DH)                                                                                         \

@@ -345,7 +345,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
 
         // dW (m = c, n = j) += X^T Us over the 64 rows of the block
 #pragma unroll
-        for (int rs = 0; rs < 2; ++rs) {
+        for (int rs = 0; rs < (dw_part ? 2 : 0); ++rs) {
             h8 xa[NCTW];
 #pragma unroll
             for (int a = 0; a < NCTW; ++a) xa[a] = col8(Xs, LDW, rs * 32, 16 * (wv * NCTW + a), lane);
@@ -359,6 +359,7 @@ __global__ __launch_bounds__(kThreads) void k_feature_map_bwd(
         __syncthreads();   // all reads of Xs / Us / Gs done before the next block overwrites them
     }
 
+    if (!dw_part) return;      // dx only
     float* po = dw_part + ((int64_t)(blockIdx.z * gridDim.x + blockIdx.x) * H + h) * D * DH;
 #pragma unroll
     for (int a = 0; a < NCTW; ++a)
@@ -480,12 +481,13 @@ __global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
         }
     };
     const int trow = 4 * G + (i >> 2), tcol = 4 * (i & 3);    // this lane's address in a transposing read
+    const bool want_dw = dw_part != nullptr;                  // no partial sums asked for: dx only
     auto process = [&](const Rows& t, int g) {
         const int r = g * 16 + i;
         float ss = 0.f;
 #pragma unroll
         for (int cs = 0; cs < DH / 32; ++cs) {
-            *reinterpret_cast<h8*>(Xs + i * LDX + cs * 32 + 8 * G) = t.x[cs];
+            if (want_dw) *reinterpret_cast<h8*>(Xs + i * LDX + cs * 32 + 8 * G) = t.x[cs];
             ss += dot_h8(__builtin_bit_cast(uint4, t.x[cs]), __builtin_bit_cast(uint4, t.x[cs]));
         }
         ss = sum_over_groups(ss);
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
                     sincos_turns(acc[q][e] * inv_turns, s_, c_);
                     du[p][4 * q + e] = (half_t)(sinv * (c_ * (float)t.gs[p][4 * q + e] - s_ * (float)t.gc[p][4 * q + e]));
                 }
-            *reinterpret_cast<h8*>(Us + i * LDU + 32 * p + 8 * G) = du[p];
+            if (want_dw) *reinterpret_cast<h8*>(Us + i * LDU + 32 * p + 8 * G) = du[p];
         }
 
         // y^T tiles (m = input column in pair order, n = row)
@@ -540,6 +542,7 @@ __global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
         }
 
         // dW' (m = c, n = j) += x^T du over the 16 rows of the group
+        if (!want_dw) return;
         wave_lds_order();
         h4 xa[DH / 16];
 #pragma unroll
@@ -566,6 +569,7 @@ __global__ __launch_bounds__(kFeatureBwdThreads) void k_feature_map_bwd_stream(
 
     // The waves' sums, one round: every wave leaves its dW' in LDS, then wave w adds up tiles
     // w, w + 8, ... of all the waves, in wave order, and stores them.
+    if (!want_dw) return;
     f4* red = reinterpret_cast<f4*>(smem_raw);
     __syncthreads();   // every wave is out of the row loop: its LDS becomes the exchange area
 #pragma unroll

@@ -211,7 +211,8 @@ std::tuple<Tensor, Tensor> feature_map_forward_pair(const Tensor& x0, const Tens
     return {phi0, phi1};
 }
 
-std::tuple<Tensor, Tensor> feature_map_backward(const Tensor& x, const Tensor& w, const Tensor& grad_phi, double scale) {
+std::tuple<Tensor, c10::optional<Tensor>> feature_map_backward(const Tensor& x, const Tensor& w, const Tensor& grad_phi,
+                                                               double scale, bool need_dw) {
     check_feature_args(x, w);
     const int64_t L = x.size(0), B = x.size(1);
     const int H = (int)x.size(2), d = (int)x.size(3), D = (int)w.size(1);
@@ -219,17 +220,19 @@ std::tuple<Tensor, Tensor> feature_map_backward(const Tensor& x, const Tensor& w
     TORCH_CHECK_VALUE(grad_phi.size(0) == L && grad_phi.size(1) == B && grad_phi.size(2) == H && grad_phi.size(3) == 2 * D,
                       "grad_phi ", grad_phi.sizes(), " must be [", L, ", ", B, ", ", H, ", ", 2 * D, "]");
     Tensor dx = torch::empty_like(x);
-    Tensor dw = torch::empty({H, D, d}, x.options().dtype(torch::kFloat32));
+    c10::optional<Tensor> dw;       // need_dw = false: w counts as a constant, no gradient formed
+    if (need_dw) dw = torch::empty({H, D, d}, x.options().dtype(torch::kFloat32));
     Launch l(x);
-    const size_t nbytes = rfa_feature_map_backward_workspace_bytes(L * B, H, D, d);
+    const size_t nbytes = need_dw ? rfa_feature_map_backward_workspace_bytes(L * B, H, D, d) : 0;
     Tensor ws = workspace(nbytes, x);
-    check_rc(rfa_feature_map_backward(ptr(x), ptr(w), ptr(grad_phi), ptr(dx), dw.data_ptr<float>(), L * B, H, D, d,
-                                      (float)scale, ptr(ws), nbytes, l.stream));
+    check_rc(rfa_feature_map_backward(ptr(x), ptr(w), ptr(grad_phi), ptr(dx), need_dw ? dw->data_ptr<float>() : nullptr,
+                                      L * B, H, D, d, (float)scale, need_dw ? ptr(ws) : nullptr, nbytes, l.stream));
     return {dx, dw};
 }
 
-std::tuple<Tensor, Tensor, Tensor> feature_map_backward_pair(const Tensor& x0, const Tensor& x1, const Tensor& w,
-                                                             const Tensor& g0, const Tensor& g1, double scale) {
+std::tuple<Tensor, Tensor, c10::optional<Tensor>> feature_map_backward_pair(const Tensor& x0, const Tensor& x1,
+                                                                            const Tensor& w, const Tensor& g0,
+                                                                            const Tensor& g1, double scale, bool need_dw) {
     check_feature_args(x0, w);
     check_feature_args(x1, w);
     TORCH_CHECK_VALUE(x0.sizes() == x1.sizes(), "the two tensors must have one shape");
@@ -241,18 +244,22 @@ std::tuple<Tensor, Tensor, Tensor> feature_map_backward_pair(const Tensor& x0, c
                           g->sizes(), " must be [", L, ", ", B, ", ", H, ", ", 2 * D, "]");
     }
     Tensor dx0 = torch::empty_like(x0), dx1 = torch::empty_like(x1);
-    Tensor dw = torch::empty({H, D, d}, x0.options().dtype(torch::kFloat32));
+    c10::optional<Tensor> dw;
+    if (need_dw) dw = torch::empty({H, D, d}, x0.options().dtype(torch::kFloat32));
     Launch l(x0);
-    const size_t nbytes = rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d);
+    const size_t nbytes = need_dw ? rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d) : 0;
     Tensor ws = workspace(nbytes, x0);
     check_rc(rfa_feature_map_backward_pair(ptr(x0), ptr(x1), ptr(w), ptr(g0), ptr(g1), ptr(dx0), ptr(dx1),
-                                           dw.data_ptr<float>(), L * B, H, D, d, (float)scale, ptr(ws), nbytes, l.stream));
+                                           need_dw ? dw->data_ptr<float>() : nullptr, L * B, H, D, d, (float)scale,
+                                           need_dw ? ptr(ws) : nullptr, nbytes, l.stream));
     return {dx0, dx1, dw};
 }
 
-std::tuple<Tensor, Tensor> feature_map_backward_pair_packed(const Tensor& x0, const Tensor& x1, const Tensor& w,
-                                                            const Tensor& g0, const Tensor& g1,
-                                                            const c10::optional<Tensor>& third, double scale) {
+std::tuple<Tensor, c10::optional<Tensor>> feature_map_backward_pair_packed(const Tensor& x0, const Tensor& x1,
+                                                                           const Tensor& w, const Tensor& g0,
+                                                                           const Tensor& g1,
+                                                                           const c10::optional<Tensor>& third,
+                                                                           double scale, bool need_dw) {
     check_feature_args(x0, w);
     check_feature_args(x1, w);
     TORCH_CHECK_VALUE(x0.sizes() == x1.sizes(), "the two tensors must have one shape");
@@ -268,13 +275,14 @@ std::tuple<Tensor, Tensor> feature_map_backward_pair_packed(const Tensor& x0, co
         TORCH_CHECK_VALUE(third->numel() == x0.numel(), "third ", third->sizes(), " must hold ", L * B, " rows of ", H * d);
     }
     Tensor packed = torch::empty({L * B, 3 * (int64_t)H * d}, x0.options());
-    Tensor dw = torch::empty({H, D, d}, x0.options().dtype(torch::kFloat32));
+    c10::optional<Tensor> dw;
+    if (need_dw) dw = torch::empty({H, D, d}, x0.options().dtype(torch::kFloat32));
     Launch l(x0);
-    const size_t nbytes = rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d);
+    const size_t nbytes = need_dw ? rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d) : 0;
     Tensor ws = workspace(nbytes, x0);
     check_rc(rfa_feature_map_backward_pair_packed(ptr(x0), ptr(x1), ptr(w), ptr(g0), ptr(g1), third ? ptr(*third) : nullptr,
-                                                  ptr(packed), dw.data_ptr<float>(), L * B, H, D, d, (float)scale, ptr(ws),
-                                                  nbytes, l.stream));
+                                                  ptr(packed), need_dw ? dw->data_ptr<float>() : nullptr, L * B, H, D, d,
+                                                  (float)scale, need_dw ? ptr(ws) : nullptr, nbytes, l.stream));
     return {packed, dw};
 }
 
@@ -582,11 +590,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("grad_out"), py::arg("tau"), py::arg("want_dsigma"), py::arg("want_dw"));
     m.def("feature_map_forward", &feature_map_forward, py::arg("x"), py::arg("w"), py::arg("scale"));
     m.def("feature_map_forward_pair", &feature_map_forward_pair, py::arg("x0"), py::arg("x1"), py::arg("w"), py::arg("scale"));
-    m.def("feature_map_backward", &feature_map_backward, py::arg("x"), py::arg("w"), py::arg("grad_phi"), py::arg("scale"));
+    m.def("feature_map_backward", &feature_map_backward, py::arg("x"), py::arg("w"), py::arg("grad_phi"), py::arg("scale"),
+          py::arg("need_dw") = true);
     m.def("feature_map_backward_pair", &feature_map_backward_pair, py::arg("x0"), py::arg("x1"), py::arg("w"),
-          py::arg("grad_phi0"), py::arg("grad_phi1"), py::arg("scale"));
+          py::arg("grad_phi0"), py::arg("grad_phi1"), py::arg("scale"), py::arg("need_dw") = true);
     m.def("feature_map_backward_pair_packed", &feature_map_backward_pair_packed, py::arg("x0"), py::arg("x1"), py::arg("w"),
-          py::arg("grad_phi0"), py::arg("grad_phi1"), py::arg("third"), py::arg("scale"));
+          py::arg("grad_phi0"), py::arg("grad_phi1"), py::arg("third"), py::arg("scale"), py::arg("need_dw") = true);
     m.def("project_feature_map", &project_feature_map, py::arg("x"), py::arg("weights"), py::arg("biases"),
           py::arg("want_phi"), py::arg("w"), py::arg("heads"), py::arg("scale"), py::arg("keep_y") = true);
     m.def("linear_weight_grad", &linear_weight_grad, py::arg("x"), py::arg("dys"), py::arg("want_bias"));

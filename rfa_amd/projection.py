@@ -87,29 +87,32 @@ class _ProjectHeads(torch.autograd.Function):
             # GEMM for dx and one contraction for the three weight gradients
             e_out = weights[0].shape[0]
             packed, dwf = rfa_hip.feature_map_backward_pair_packed(ys[0], ys[1], wf, grads[0].contiguous(),
-                                                                   grads[1].contiguous(), grads[2].contiguous(), ctx.scale)
+                                                                   grads[1].contiguous(), grads[2].contiguous(), ctx.scale,
+                                                                   need_dw=ctx.needs_input_grad[1])
             dx = torch.mm(packed, _stacked_weights(weights)).view(L, B, E)
             dws, dbs = linear_param_grads(x2, [packed], [any(ctx.has_bias)])
             dparams = []
             for p in range(n):
                 dparams += [dws[0][p * e_out:(p + 1) * e_out],
                             dbs[0][p * e_out:(p + 1) * e_out] if ctx.has_bias[p] else None]
-            return (dx, dwf.to(wf.dtype), None, None, None, None, *dparams)
+            return (dx, None if dwf is None else dwf.to(wf.dtype), None, None, None, None, *dparams)
         phi_idx = [p for p in range(n) if ctx.want_phi[p]]
         pair = {}
         if len(phi_idx) == 2:       # phi(q) and phi(k): both through the same w, one launch for the two
             p0, p1 = phi_idx
             dy0, dy1, dwf = rfa_hip.feature_map_backward_pair(ys[0], ys[1], wf, grads[p0].contiguous(),
-                                                              grads[p1].contiguous(), ctx.scale)
+                                                              grads[p1].contiguous(), ctx.scale,
+                                                              need_dw=ctx.needs_input_grad[1])
             pair = {p0: dy0, p1: dy1}
         for p in range(n):
             g = grads[p].contiguous()
             if p in pair:
                 dy = pair[p]
             elif ctx.want_phi[p]:
-                dy, dw = rfa_hip.feature_map_backward(ys[yi], wf, g, ctx.scale)
+                dy, dw = rfa_hip.feature_map_backward(ys[yi], wf, g, ctx.scale, need_dw=ctx.needs_input_grad[1])
                 yi += 1
-                dwf = dw if dwf is None else dwf + dw
+                if dw is not None:
+                    dwf = dw if dwf is None else dwf + dw
             else:
                 dy = g
             dy2 = dy.reshape(L * B, -1)

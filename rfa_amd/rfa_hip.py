@@ -365,8 +365,9 @@ def linear_weight_grad(x: Tensor, dys, want_bias):
     return dws, dbs
 
 
-def feature_map_backward(x: Tensor, w: Tensor, grad_phi: Tensor, scale: float):
-    """(dx fp16 [L,B,H,d], dw fp32 [H,D,d])."""
+def feature_map_backward(x: Tensor, w: Tensor, grad_phi: Tensor, scale: float, need_dw: bool = True):
+    """(dx fp16 [L,B,H,d], dw fp32 [H,D,d]); with ``need_dw=False`` w counts as a constant: dw is None
+    and neither formed nor reduced."""
     _check_feature_args(x, w)
     L, B, H, d = x.shape
     D = w.shape[1]
@@ -375,19 +376,20 @@ def feature_map_backward(x: Tensor, w: Tensor, grad_phi: Tensor, scale: float):
              lambda: f"grad_phi {tuple(grad_phi.shape)} must be {(L, B, H, 2 * D)}")
     lib = _lib.load()
     dx = torch.empty_like(x)
-    dw = torch.empty((H, D, d), dtype=torch.float32, device=x.device)
+    dw = torch.empty((H, D, d), dtype=torch.float32, device=x.device) if need_dw else None
     with _on_device(x.device):
-        nbytes = lib.rfa_feature_map_backward_workspace_bytes(L * B, H, D, d)
-        ws = _workspace(nbytes, x.device)
+        nbytes = lib.rfa_feature_map_backward_workspace_bytes(L * B, H, D, d) if need_dw else 0
+        ws = _workspace(nbytes, x.device) if need_dw else None
         _lib.check(lib.rfa_feature_map_backward(
-            x.data_ptr(), w.data_ptr(), grad_phi.data_ptr(), dx.data_ptr(), dw.data_ptr(),
-            L * B, H, D, d, float(scale), ws.data_ptr(), nbytes, _stream_ptr(x.device)))
+            x.data_ptr(), w.data_ptr(), grad_phi.data_ptr(), dx.data_ptr(), dw.data_ptr() if need_dw else None,
+            L * B, H, D, d, float(scale), ws.data_ptr() if need_dw else None, nbytes, _stream_ptr(x.device)))
     return dx, dw
 
 
-def feature_map_backward_pair(x0: Tensor, x1: Tensor, w: Tensor, grad_phi0: Tensor, grad_phi1: Tensor, scale: float):
+def feature_map_backward_pair(x0: Tensor, x1: Tensor, w: Tensor, grad_phi0: Tensor, grad_phi1: Tensor, scale: float,
+                              need_dw: bool = True):
     """Two tensors that went through the same w in one launch: (dx0, dx1 fp16 [L,B,H,d], dw fp32 [H,D,d]
-    = the sum of both contributions)."""
+    = the sum of both contributions, or None with ``need_dw=False``)."""
     _check_feature_args(x0, w)
     _check_feature_args(x1, w)
     _require(x0.shape == x1.shape, ValueError, lambda: "the two tensors must have one shape")
@@ -398,21 +400,23 @@ def feature_map_backward_pair(x0: Tensor, x1: Tensor, w: Tensor, grad_phi0: Tens
         _require(tuple(g.shape) == (L, B, H, 2 * D), ValueError, lambda: f"{name} {tuple(g.shape)} must be {(L, B, H, 2 * D)}")
     lib = _lib.load()
     dx0, dx1 = torch.empty_like(x0), torch.empty_like(x1)
-    dw = torch.empty((H, D, d), dtype=torch.float32, device=x0.device)
+    dw = torch.empty((H, D, d), dtype=torch.float32, device=x0.device) if need_dw else None
     with _on_device(x0.device):
-        nbytes = lib.rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d)
-        ws = _workspace(nbytes, x0.device)
+        nbytes = lib.rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d) if need_dw else 0
+        ws = _workspace(nbytes, x0.device) if need_dw else None
         _lib.check(lib.rfa_feature_map_backward_pair(
             x0.data_ptr(), x1.data_ptr(), w.data_ptr(), grad_phi0.data_ptr(), grad_phi1.data_ptr(), dx0.data_ptr(),
-            dx1.data_ptr(), dw.data_ptr(), L * B, H, D, d, float(scale), ws.data_ptr(), nbytes, _stream_ptr(x0.device)))
+            dx1.data_ptr(), dw.data_ptr() if need_dw else None, L * B, H, D, d, float(scale),
+            ws.data_ptr() if need_dw else None, nbytes, _stream_ptr(x0.device)))
     return dx0, dx1, dw
 
 
 def feature_map_backward_pair_packed(x0: Tensor, x1: Tensor, w: Tensor, grad_phi0: Tensor, grad_phi1: Tensor,
-                                     third: Optional[Tensor], scale: float):
+                                     third: Optional[Tensor], scale: float, need_dw: bool = True):
     """feature_map_backward_pair that leaves [dx0 | dx1 | third] side by side in one fp16 [L*B, 3*H*d]
     matrix (third: [L, B, H, d] or [L*B, H*d], copied by the same launch; None leaves that block
-    unset) and returns (packed, dw): the operand of one GEMM for the three input projections."""
+    unset) and returns (packed, dw): the operand of one GEMM for the three input projections.
+    ``need_dw=False``: dw is None, w counts as a constant."""
     _check_feature_args(x0, w)
     _check_feature_args(x1, w)
     _require(x0.shape == x1.shape, ValueError, lambda: "the two tensors must have one shape")
@@ -426,14 +430,14 @@ def feature_map_backward_pair_packed(x0: Tensor, x1: Tensor, w: Tensor, grad_phi
         _require(third.numel() == x0.numel(), ValueError, lambda: f"third {tuple(third.shape)} must hold {L * B} rows of {H * d}")
     lib = _lib.load()
     packed = torch.empty((L * B, 3 * H * d), dtype=torch.float16, device=x0.device)
-    dw = torch.empty((H, D, d), dtype=torch.float32, device=x0.device)
+    dw = torch.empty((H, D, d), dtype=torch.float32, device=x0.device) if need_dw else None
     with _on_device(x0.device):
-        nbytes = lib.rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d)
-        ws = _workspace(nbytes, x0.device)
+        nbytes = lib.rfa_feature_map_backward_pair_workspace_bytes(L * B, H, D, d) if need_dw else 0
+        ws = _workspace(nbytes, x0.device) if need_dw else None
         _lib.check(lib.rfa_feature_map_backward_pair_packed(
             x0.data_ptr(), x1.data_ptr(), w.data_ptr(), grad_phi0.data_ptr(), grad_phi1.data_ptr(),
-            None if third is None else third.data_ptr(), packed.data_ptr(), dw.data_ptr(), L * B, H, D, d, float(scale),
-            ws.data_ptr(), nbytes, _stream_ptr(x0.device)))
+            None if third is None else third.data_ptr(), packed.data_ptr(), dw.data_ptr() if need_dw else None, L * B, H,
+            D, d, float(scale), ws.data_ptr() if need_dw else None, nbytes, _stream_ptr(x0.device)))
     return packed, dw
 
 

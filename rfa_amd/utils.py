@@ -124,8 +124,10 @@ class _FeatureMap(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_phi: Tensor):
         xh, wh = ctx.saved_tensors
-        dx, dw = rfa_hip.feature_map_backward(xh, wh, grad_phi.to(torch.float16).contiguous(), ctx.scale)
-        return dx.to(ctx.in_dtypes[0]), dw.to(ctx.in_dtypes[1]), None
+        # matrices that take no gradient (not reparametrised, or frozen): dW' is neither formed nor reduced
+        dx, dw = rfa_hip.feature_map_backward(xh, wh, grad_phi.to(torch.float16).contiguous(), ctx.scale,
+                                              need_dw=ctx.needs_input_grad[1])
+        return dx.to(ctx.in_dtypes[0]), None if dw is None else dw.to(ctx.in_dtypes[1]), None
 
 
 class _FeatureMapPair(torch.autograd.Function):
@@ -146,8 +148,9 @@ class _FeatureMapPair(torch.autograd.Function):
     def backward(ctx, g0: Tensor, g1: Tensor):
         x0h, x1h, wh = ctx.saved_tensors
         dx0, dx1, dw = rfa_hip.feature_map_backward_pair(x0h, x1h, wh, g0.to(torch.float16).contiguous(),
-                                                         g1.to(torch.float16).contiguous(), ctx.scale)
-        return dx0.to(ctx.in_dtypes[0]), dx1.to(ctx.in_dtypes[1]), dw.to(ctx.in_dtypes[2]), None
+                                                         g1.to(torch.float16).contiguous(), ctx.scale,
+                                                         need_dw=ctx.needs_input_grad[2])
+        return dx0.to(ctx.in_dtypes[0]), dx1.to(ctx.in_dtypes[1]), None if dw is None else dw.to(ctx.in_dtypes[2]), None
 
 
 def random_project_pair(*, x0: Tensor, x1: Tensor, random_matrices: Tensor, scale: float = SCALE):

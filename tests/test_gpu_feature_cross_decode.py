@@ -140,6 +140,47 @@ def test_feature_map_backward_pair_packed(L, B, H, d, D, with_third):
     assert torch.equal(dw, want_dw)
 
 
+@pytest.mark.parametrize("L,B,H,d,D", FEATURE_SHAPES)
+def test_feature_map_backward_without_dw(L, B, H, d, D):
+    """Matrices that take no gradient: dx carries the bits of the full backward, dW' is neither
+    formed nor reduced (None), no workspace is asked for; through the autograd Functions a frozen
+    random_matrices tensor gets no gradient and x the same one."""
+    from rfa_amd import _lib, rfa_hip
+    from rfa_amd.utils import random_project, random_project_pair
+    x0 = (_randn(L, B, H, d, seed=60 + L) * 1.3).half().cuda()
+    x1 = (_randn(L, B, H, d, seed=61 + L) * 0.7).half().cuda()
+    w = (_randn(H, D, d, seed=62) * 0.9).half().cuda()
+    g0 = _randn(L, B, H, 2 * D, seed=63).half().cuda()
+    g1 = _randn(L, B, H, 2 * D, seed=64).half().cuda()
+    third = _randn(L, B, H, d, seed=65).half().cuda()
+    print(f"phi bwd, dx only L={L} B={B} H={H} d={d} D={D}", flush=True)
+    want, _ = rfa_hip.feature_map_backward(x0, w, g0, O.SCALE)
+    got, dw = rfa_hip.feature_map_backward(x0, w, g0, O.SCALE, need_dw=False)
+    assert dw is None and torch.equal(got, want)
+    w0, w1, _ = rfa_hip.feature_map_backward_pair(x0, x1, w, g0, g1, O.SCALE)
+    a0, a1, dw = rfa_hip.feature_map_backward_pair(x0, x1, w, g0, g1, O.SCALE, need_dw=False)
+    assert dw is None and torch.equal(a0, w0) and torch.equal(a1, w1)
+    wp, _ = rfa_hip.feature_map_backward_pair_packed(x0, x1, w, g0, g1, third, O.SCALE)
+    gp, dw = rfa_hip.feature_map_backward_pair_packed(x0, x1, w, g0, g1, third, O.SCALE, need_dw=False)
+    assert dw is None and torch.equal(gp, wp)
+    # the C ABI with a NULL dw takes a NULL workspace
+    lib = _lib.load()
+    dx = torch.empty_like(x0)
+    _lib.check(lib.rfa_feature_map_backward(x0.data_ptr(), w.data_ptr(), g0.data_ptr(), dx.data_ptr(), None, L * B, H, D, d,
+                                            O.SCALE, None, 0, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.equal(dx, want)
+    # autograd: frozen matrices
+    xa, xb = x0.clone().requires_grad_(True), x1.clone().requires_grad_(True)
+    wf = w.clone()                                   # requires_grad False
+    p0, p1 = random_project_pair(x0=xa, x1=xb, random_matrices=wf, scale=O.SCALE)
+    torch.autograd.backward([p0, p1], [g0, g1])
+    assert wf.grad is None and torch.equal(xa.grad, w0) and torch.equal(xb.grad, w1)
+    xc = x0.clone().requires_grad_(True)
+    random_project(x=xc, random_matrices=wf, scale=O.SCALE).backward(g0)
+    assert torch.equal(xc.grad, want)
+
+
 @pytest.mark.parametrize("L,B,H,d,D,wgs", [(333, 2, 2, 64, 64, 4), (333, 2, 2, 64, 64, 2), (100, 3, 1, 128, 32, 1),
                                            (257, 1, 2, 64, 32, 6)])
 def test_feature_map_waves_that_walk_many_row_groups(L, B, H, d, D, wgs, knobs):

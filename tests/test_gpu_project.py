@@ -349,7 +349,8 @@ def test_projection_backward_on_the_packed_gradient(monkeypatch):
 
     used = []
     real = projection.rfa_hip.feature_map_backward_pair_packed
-    monkeypatch.setattr(projection.rfa_hip, "feature_map_backward_pair_packed", lambda *a: (used.append(1), real(*a))[1])
+    monkeypatch.setattr(projection.rfa_hip, "feature_map_backward_pair_packed",
+                        lambda *a, **kw: (used.append(1), real(*a, **kw))[1])
     print("projection backward, packed gradient", flush=True)
     packed = run()
     assert used, "the packed path was not taken"
