@@ -283,11 +283,6 @@ void drop(const void* saved) {
     std::lock_guard<std::mutex> lk(mu);
     table.erase(saved);
 }
-
-size_t size() {
-    std::lock_guard<std::mutex> lk(mu);
-    return table.size();
-}
 }  // namespace registry
 
 size_t align_up(size_t x) { return (x + 255) & ~size_t(255); }

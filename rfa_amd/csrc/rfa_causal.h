@@ -1509,7 +1509,7 @@ __global__ __launch_bounds__(64 * NW) void k_causal_bwd_dkdv(
     const int rb = w & 3, half = w >> 2;   // tile-phase role: 16-row block and which of its tiles
     const int ws = SPLIT ? (w & 3) : w;    // state-phase slice
     const bool do_dk = !SPLIT || w < 4, do_dv = !SPLIT || w >= 4;
-    constexpr int JPW = Cfg::JPW, NH = Cfg::NH;
+    constexpr int JPW = Cfg::JPW;
     int n, seg;
     seq_seg_of_block(blockIdx.x, N, nseg, n, seg);
     const int t_begin = seg * seg_len;

@@ -99,7 +99,7 @@ __device__ __forceinline__ void sliced_bwd_dqdk(
     using Cfg = SlicedBwdCfg<KD, DH, SW>;
     constexpr int NT = kGroupThreads, C = Cfg::C, KSL = Cfg::KSL, NPW = Cfg::NPW;
     constexpr int LDK = Cfg::LDS_, LDV = Cfg::LDV, LDA = Cfg::LDA;
-    constexpr int kDqTick = 256, kDkTick = 256 + 64 * NPW;     // first thread of the dQ / dK waves
+    [[maybe_unused]] constexpr int kDqTick = 256, kDkTick = 256 + 64 * NPW;     // first thread of the dQ / dK waves (phase timing)
     constexpr int NCT = DH / 16;
     constexpr int PPR = DH / 8, VP = ChunkRegs<DH, NT>::kPieces;
     constexpr size_t kStage = Cfg::kLds / 2;
